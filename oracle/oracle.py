@@ -1,0 +1,374 @@
+"""ctypes front end of the CPU oracle (oracle/fortis_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the benchmark's
+cpu_baseline leg.  The product package never imports this module.
+"""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+f32p = C.POINTER(C.c_float)
+f64p = C.POINTER(C.c_double)
+i32p = C.POINTER(C.c_int)
+
+
+def build():
+    subprocess.check_call(["make", "-s", "-C", _HERE, "liboracle.so"])
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(path):
+            build()
+        _LIB = C.CDLL(path)
+    return _LIB
+
+
+def _f(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a, a.ctypes.data_as(f32p)
+
+
+class Ref(C.Structure):
+    _fields_ = [("array", C.c_int), ("planar", C.c_int), ("base", C.c_long), ("si", C.c_long),
+                ("sj", C.c_long), ("plane", C.c_long)]
+
+
+class Ins(C.Structure):
+    _fields_ = [("op", C.c_int), ("a", C.c_int), ("b", C.c_int)]
+
+
+# ---------------------------------------------------------------------------------------------
+# descriptor handling (independent of the product's parser on purpose)
+# ---------------------------------------------------------------------------------------------
+def refs_from_descriptor(arrays, entries):
+    """arrays: gather.json/scatter.json "arrays"; entries: list of {"array", "idx"} (slots, scalars or
+    stores).  Column-major strides; the 'v' dims must be trailing (driver/fortis_gather_emit.py:19-26)."""
+    out = (Ref * len(entries))()
+    for n, e in enumerate(entries):
+        shape = arrays[e["array"]]["shape"]
+        strides = [1]
+        for d in shape[:-1]:
+            strides.append(strides[-1] * d)
+        base = si = sj = plane = 0
+        planar = 0
+        for d, (kind, off) in enumerate(e["idx"]):
+            if kind == "v":
+                planar = 1
+                if plane == 0:
+                    plane = strides[d]
+                continue
+            base += (off - 1) * strides[d]
+            if kind == "i":
+                si += strides[d]
+            else:
+                sj += strides[d]
+        out[n] = Ref(e["array"], planar, base, si, sj, plane)
+    return out
+
+
+_TOK = re.compile(r"\s*(tv|S\d+|[-+]?(?:\d+\.\d*|\.\d+|\d+)(?:[eE][-+]?\d+)?f?|[()+\-*/])")
+
+
+def compile_exprs(exprs):
+    """C expression strings over tv, S<n> and float literals -> (instructions, constants) in the
+    oracle's three-address form.  Several expressions are applied in order, each replacing tv
+    (driver/fortis_gather_emit.py:59-61)."""
+    ins, consts = [], []
+    cur = 0  # operand code of the current tv value
+
+    def parse(tokens, tvcode):
+        pos = [0]
+
+        def peek():
+            return tokens[pos[0]] if pos[0] < len(tokens) else None
+
+        def take():
+            t = tokens[pos[0]]
+            pos[0] += 1
+            return t
+
+        def atom():
+            t = take()
+            if t == "(":
+                v = expr()
+                assert take() == ")"
+                return v
+            if t == "tv":
+                return tvcode
+            if t.startswith("S"):
+                return 1 + int(t[1:])
+            consts.append(np.float32(float(t.rstrip("f"))))
+            return 16 + len(consts) - 1
+
+        def term():
+            v = atom()
+            while peek() in ("*", "/"):
+                op = take()
+                r = atom()
+                ins.append((2 if op == "*" else 3, v, r))
+                v = 32 + len(ins) - 1
+            return v
+
+        def expr():
+            v = term()
+            while peek() in ("+", "-"):
+                op = take()
+                r = term()
+                ins.append((0 if op == "+" else 1, v, r))
+                v = 32 + len(ins) - 1
+            return v
+
+        v = expr()
+        assert pos[0] == len(tokens)
+        return v
+
+    for e in exprs:
+        toks = _TOK.findall(e)
+        assert "".join(toks).replace(" ", "") == e.replace(" ", ""), e
+        cur = parse(toks, cur)
+    arr = (Ins * max(1, len(ins)))(*[Ins(*t) for t in ins])
+    cst = np.array(consts if consts else [0.0], dtype=np.float32)
+    return arr, len(ins), cst
+
+
+def _arrays_ptr(arrs):
+    p = (f32p * len(arrs))(*[a.ctypes.data_as(f32p) for a in arrs])
+    return p
+
+
+def stencil_gather(desc, arrays, count, nk, ilo=0, jlo=0, ni=1, cells=None):
+    """desc: parsed gather.json.  arrays: list of float32 Fortran-ordered numpy arrays (flattened 'F')."""
+    L = lib()
+    slots = refs_from_descriptor(desc["arrays"], desc["slots"])
+    scal = refs_from_descriptor(desc["arrays"], desc["scalars"])
+    ins, nins, consts = compile_exprs(desc["exprs"])
+    flat = [np.ascontiguousarray(a.reshape(-1, order="F"), dtype=np.float32) for a in arrays]
+    X = np.empty((count * nk, len(desc["slots"])), dtype=np.float32)
+    cp = None
+    if cells is not None:
+        cells = np.ascontiguousarray(cells, dtype=np.int32)
+        cp = cells.ctypes.data_as(i32p)
+    sx = desc["arrays"][0]["shape"][0]
+    L.orc_stencil_gather(len(desc["slots"]), slots, len(desc["scalars"]), scal, nins, ins,
+                         consts.ctypes.data_as(f32p), _arrays_ptr(flat), C.c_long(count), nk, cp, sx,
+                         ilo, jlo, ni, X.ctypes.data_as(f32p))
+    return X
+
+
+def stencil_scatter(desc, arrays, Y, count, kk, ilo=0, jlo=0, ni=1, cells=None):
+    """In-place on `arrays` (list of flat float32 arrays in Fortran element order)."""
+    L = lib()
+    stores = sorted(desc["stores"], key=lambda s: s["slot"])
+    st = refs_from_descriptor(desc["arrays"], stores)
+    scal = refs_from_descriptor(desc["arrays"], desc["scalars"])
+    ins, nins, consts = compile_exprs(desc["exprs"])
+    Y = np.ascontiguousarray(Y, dtype=np.float32)
+    cp = None
+    if cells is not None:
+        cells = np.ascontiguousarray(cells, dtype=np.int32)
+        cp = cells.ctypes.data_as(i32p)
+    sx = desc["arrays"][0]["shape"][0]
+    for a in arrays:
+        assert a.dtype == np.float32 and a.flags.c_contiguous and a.ndim == 1
+    L.orc_stencil_scatter(desc["n"], st, len(desc["scalars"]), scal, nins, ins,
+                          consts.ctypes.data_as(f32p), _arrays_ptr(arrays), C.c_long(count), kk, cp, sx,
+                          ilo, jlo, ni, Y.ctypes.data_as(f32p))
+
+
+# ---------------------------------------------------------------------------------------------
+# MLPs
+# ---------------------------------------------------------------------------------------------
+def _mlp_args(Ws, bs):
+    widths = [Ws[0].shape[1]] + [w.shape[0] for w in Ws]
+    keep = [np.ascontiguousarray(w, dtype=np.float32) for w in Ws]
+    keepb = [np.ascontiguousarray(b if b is not None else np.zeros(w.shape[0]), dtype=np.float32)
+             for w, b in zip(Ws, bs)]
+    wp = (f32p * len(Ws))(*[w.ctypes.data_as(f32p) for w in keep])
+    bp = (f32p * len(Ws))(*[b.ctypes.data_as(f32p) for b in keepb])
+    wid = (C.c_int * len(widths))(*widths)
+    return widths, keep, keepb, wp, bp, wid
+
+
+def mlp_native(Ws, bs, X, in_norms=None, out_norms=None):
+    """Shipped ANN_apply loop order, fp32, ReLU on hidden layers (mom6_zb/fwd_native_zb.f90:30-77)."""
+    widths, kw, kb, wp, bp, wid = _mlp_args(Ws, bs)
+    X, xp = _f(X)
+    rows = X.shape[0]
+    Y = np.empty((rows, widths[-1]), dtype=np.float32)
+    inn = _f(in_norms) if in_norms is not None else (None, None)
+    outn = _f(out_norms) if out_norms is not None else (None, None)
+    lib().orc_mlp_native(len(Ws), wid, wp, bp, inn[1], outn[1], C.c_long(rows), xp, Y.ctypes.data_as(f32p))
+    return Y
+
+
+ACT = {"none": 0, "relu": 1, "leaky": 2}
+
+
+def mlp_f64(Ws, bs, acts, X, alphas=None, in_norms=None, out_norms=None, mask_tail=0):
+    """fp64-accumulated GEMM+bias+activation chain, fp32 between layers."""
+    widths, kw, kb, wp, bp, wid = _mlp_args(Ws, bs)
+    X, xp = _f(X)
+    rows = X.shape[0]
+    Y = np.empty((rows, widths[-1]), dtype=np.float32)
+    act = (C.c_int * len(Ws))(*[ACT[a] if isinstance(a, str) else a for a in acts])
+    al = np.ascontiguousarray(alphas if alphas is not None else np.zeros(len(Ws)), dtype=np.float32)
+    inn = _f(in_norms) if in_norms is not None else (None, None)
+    outn = _f(out_norms) if out_norms is not None else (None, None)
+    lib().orc_mlp_f64(len(Ws), wid, wp, bp, act, al.ctypes.data_as(f32p), inn[1], outn[1], mask_tail,
+                      C.c_long(rows), xp, Y.ctypes.data_as(f32p))
+    return Y
+
+
+def gemm(A, W):
+    A, ap = _f(A)
+    W, wp = _f(W)
+    B, K = A.shape
+    N = W.shape[0]
+    Cc = np.empty((B, N), dtype=np.float32)
+    lib().orc_gemm(C.c_long(B), C.c_long(N), C.c_long(K), ap, wp, Cc.ctypes.data_as(f32p))
+    return Cc
+
+
+# ---------------------------------------------------------------------------------------------
+# ZB host
+# ---------------------------------------------------------------------------------------------
+def zb_fields(sx=68, sy=78, nz=15):
+    n3, n2 = sx * sy * nz, sx * sy
+    out = [np.empty(n3, np.float32) for _ in range(3)] + [np.empty(n2, np.float32) for _ in range(3)]
+    lib().orc_zb_fields(sx, sy, nz, *[a.ctypes.data_as(f32p) for a in out])
+    return dict(zip(["sh_xy", "sh_xx", "vort_xy", "mask2dT", "mask2dBu", "kappa_h"], out))
+
+
+def zb_prep(F, sx=68, sy=78, nz=15, halo=4):
+    n3 = sx * sy * nz
+    out = [np.empty(n3, np.float32) for _ in range(3)]
+    lib().orc_zb_prep(sx, sy, nz, halo, *[F[k].ctypes.data_as(f32p) for k in ("sh_xy", "sh_xx", "vort_xy", "mask2dT")],
+                      *[a.ctypes.data_as(f32p) for a in out])
+    return dict(zip(["sh_xy_h", "vort_xy_h", "norm_h"], out))
+
+
+def zb_step_native(F, P, Ws, bs, in_norms, out_norms, sx=68, sy=78, nz=15, halo=4):
+    widths, kw, kb, wp, bp, wid = _mlp_args(Ws, bs)
+    n3, n2 = sx * sy * nz, sx * sy
+    Txx, Tyy, Txy = [np.zeros(n3, np.float32) for _ in range(3)]
+    Txy_h = np.zeros(n2, np.float32)
+    inn = _f(in_norms) if in_norms is not None else (None, None)
+    outn = _f(out_norms) if out_norms is not None else (None, None)
+    lib().orc_zb_step_native(sx, sy, nz, halo, P["sh_xy_h"].ctypes.data_as(f32p), F["sh_xx"].ctypes.data_as(f32p),
+                             P["vort_xy_h"].ctypes.data_as(f32p), P["norm_h"].ctypes.data_as(f32p),
+                             F["kappa_h"].ctypes.data_as(f32p), F["mask2dBu"].ctypes.data_as(f32p),
+                             len(Ws), wid, wp, bp, inn[1], outn[1],
+                             *[a.ctypes.data_as(f32p) for a in (Txx, Tyy, Txy, Txy_h)])
+    return dict(Txx=Txx, Tyy=Tyy, Txy=Txy, Txy_h=Txy_h)
+
+
+# ---------------------------------------------------------------------------------------------
+# boundary, convs, pools
+# ---------------------------------------------------------------------------------------------
+def boundary_pre(A, mean, vmax, vmin):
+    """A: (NI, NK) Fortran-ordered host array (f32 or f64) -> X[NI][NK] float32."""
+    NI, NK = A.shape
+    X = np.empty((NI, NK), dtype=np.float32)
+    if A.dtype == np.float64:
+        a = np.asfortranarray(A)
+        args = [np.ascontiguousarray(v, dtype=np.float64) for v in (mean, vmax, vmin)]
+        lib().orc_boundary_pre_f64(C.c_long(NI), C.c_long(NK), a.ctypes.data_as(f64p),
+                                   *[v.ctypes.data_as(f64p) for v in args], X.ctypes.data_as(f32p))
+    else:
+        a = np.asfortranarray(A, dtype=np.float32)
+        args = [np.ascontiguousarray(v, dtype=np.float32) for v in (mean, vmax, vmin)]
+        lib().orc_boundary_pre_f32(C.c_long(NI), C.c_long(NK), a.ctypes.data_as(f32p),
+                                   *[v.ctypes.data_as(f32p) for v in args], X.ctypes.data_as(f32p))
+    return X
+
+
+def boundary_post(Y, scale, dtype=np.float32):
+    Y, yp = _f(Y)
+    NI, NK = Y.shape
+    if dtype == np.float64:
+        B = np.empty((NI, NK), dtype=np.float64, order="F")
+        s = np.ascontiguousarray(scale, dtype=np.float64)
+        lib().orc_boundary_post_f64(C.c_long(NI), C.c_long(NK), yp, s.ctypes.data_as(f64p), B.ctypes.data_as(f64p))
+    else:
+        B = np.empty((NI, NK), dtype=np.float32, order="F")
+        s = np.ascontiguousarray(scale, dtype=np.float32)
+        lib().orc_boundary_post_f32(C.c_long(NI), C.c_long(NK), yp, s.ctypes.data_as(f32p), B.ctypes.data_as(f32p))
+    return B
+
+
+def _l(*v):
+    return [C.c_long(int(t)) for t in v]
+
+
+def conv3d(x, w, stride=(1, 1, 1), pad=(0, 0, 0)):
+    x, xp = _f(x)
+    w, wp = _f(w)
+    N, Cc, D, H, W = x.shape
+    F, _, KD, KH, KW = w.shape
+    Do = (D + 2 * pad[0] - KD) // stride[0] + 1
+    Ho = (H + 2 * pad[1] - KH) // stride[1] + 1
+    Wo = (W + 2 * pad[2] - KW) // stride[2] + 1
+    y = np.empty((N, F, Do, Ho, Wo), dtype=np.float32)
+    lib().orc_conv3d(*_l(N, Cc, D, H, W, F, KD, KH, KW, Do, Ho, Wo, *stride, *pad), xp, wp, y.ctypes.data_as(f32p))
+    return y
+
+
+def conv2d(x, w, stride=(1, 1), pad=(0, 0)):
+    x = np.asarray(x, dtype=np.float32)
+    w = np.asarray(w, dtype=np.float32)
+    y = conv3d(x[:, :, None], w[:, :, None], (1,) + tuple(stride), (0,) + tuple(pad))
+    return y[:, :, 0]
+
+
+def convt2d(x, w, stride, pad, output_padding=0):
+    """x [C][H][W], w [C][F][KH][KW] (PyTorch ConvTranspose2d layout)."""
+    x, xp = _f(x)
+    w, wp = _f(w)
+    Cc, H, W = x.shape
+    _, F, KH, KW = w.shape
+    Ho = (H - 1) * stride - 2 * pad + KH + output_padding
+    Wo = (W - 1) * stride - 2 * pad + KW + output_padding
+    y = np.empty((F, Ho, Wo), dtype=np.float32)
+    lib().orc_convt2d(*_l(Cc, H, W, F, KH, KW, Ho, Wo, stride, pad), xp, wp, y.ctypes.data_as(f32p))
+    return y
+
+
+def maxpool2d(x, k=2):
+    x, xp = _f(x)
+    Cc, H, W = x.shape
+    y = np.empty((Cc, H // k, W // k), dtype=np.float32)
+    lib().orc_maxpool2d(*_l(Cc, H, W, k), xp, y.ctypes.data_as(f32p))
+    return y
+
+
+def upsample_nearest(x, s=2):
+    """x [C][H][W] or [C][D][H][W]."""
+    x, xp = _f(x)
+    if x.ndim == 3:
+        Cc, H, W = x.shape
+        y = np.empty((Cc, H * s, W * s), dtype=np.float32)
+        lib().orc_upsample_nearest(*_l(Cc, 1, H, W, s), 2, xp, y.ctypes.data_as(f32p))
+    else:
+        Cc, D, H, W = x.shape
+        y = np.empty((Cc, D * s, H * s, W * s), dtype=np.float32)
+        lib().orc_upsample_nearest(*_l(Cc, D, H, W, s), 3, xp, y.ctypes.data_as(f32p))
+    return y
+
+
+def bn_eval(x, mean, var, gamma, beta, eps=1e-5):
+    x, xp = _f(x)
+    Cc = x.shape[0]
+    S = x.size // Cc
+    y = np.empty_like(x)
+    args = [_f(v) for v in (mean, var, gamma, beta)]
+    lib().orc_bn_eval(C.c_long(Cc), C.c_long(S), *[a[1] for a in args], C.c_float(eps), xp, y.ctypes.data_as(f32p))
+    return y
