@@ -1,0 +1,100 @@
+// Internal declarations shared by the HIP sources of libfortis_rt.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include "../../include/fortis_rt.h"
+#include "../../include/fortis_step.h"
+
+#define HIP_OK(call)                                                                              \
+    do {                                                                                          \
+        hipError_t e_ = (call);                                                                   \
+        if (e_ != hipSuccess)                                                                     \
+            fprintf(stderr, "fortis: %s failed: %s (%s:%d)\n", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+    } while (0)
+
+static inline hipStream_t fortis_stream_get() { return (hipStream_t)mgpuStreamCreate(); }
+static inline long cdiv(long a, long b) { return (a + b - 1) / b; }
+
+// ---- fused GEMM + bias + activation (gemm.hip) -------------------------------------------
+// C[B][N] = epi(A[B][K] . W[N][K]^T): + bias[n], activation, * out_scale[n], ReLU on the last
+// mask_tail columns.  bias/out_scale may be null.  Returns 0, or -1 on an unsupported shape.
+int fortis_launch_gemm(const float* A, const float* W, const float* bias, float* C, long B, long N,
+                       long K, int act, float alpha, const float* out_scale, long mask_tail,
+                       hipStream_t s);
+
+// ---- fused MLP chain (chain.hip) ----------------------------------------------------------
+#define FORTIS_CHAIN_MAX_LAYERS 8
+#define FORTIS_CHAIN_MAX_WIDTH 256
+struct ChainLayer {
+    const float* Wp;    // packed weights: [Np/32][Kp/8][64 lanes][4]
+    const float* bias;  // [Np], zero padded
+    int K, N, Kp, Np;
+    int act;
+    float alpha;
+};
+struct ChainDesc {
+    int nlayers;
+    ChainLayer L[FORTIS_CHAIN_MAX_LAYERS];
+    const float* in_div;   // x / in_div[c] before layer 0, or null
+    const float* out_mul;  // y * out_mul[c] after the last layer, or null
+    int mask_tail;         // ReLU on the last mask_tail outputs
+    int ld;                // LDS row pitch in floats
+};
+// Packs W[N][K] for the chain kernel into a freshly allocated device buffer (stream-ordered).
+float* fortis_chain_pack_weights(const float* W_host, long N, long K, int* Kp, int* Np);
+float* fortis_chain_pack_bias(const float* b_host, long N, int Np);
+int  fortis_chain_ld(const ChainDesc& d);
+void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows, hipStream_t s);
+// ---- stencil tables as the kernels see them (stencil.hip) --------------------------------
+struct CellStep { int op, code, tv_left; };
+struct StencilDev {
+    int narrays;
+    long plane[FORTIS_MAX_ARRAYS];
+    int nrefs;
+    fortis_ref_t refs[FORTIS_MAX_REFS];
+    int nscal;
+    fortis_ref_t scal[FORTIS_MAX_SCAL];
+    int ncell;                         // per-cell instructions (no tv operand)
+    fortis_ins_t cell[FORTIS_MAX_INS];
+    int nchain;                        // tv chain: tv = tv op x  or  x op tv
+    CellStep chain[FORTIS_MAX_INS];
+    float consts[FORTIS_MAX_CONST];
+    long count;
+    int nk;
+    int ilo, jlo, ni, sx;
+    const int* cells;                  // device copy of the cell list, or null
+};
+// Splits the straight-line program into per-cell code and a tv chain.  Returns -1 if tv is used
+// in a way that is not a single chain.
+int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out);
+
+// ---- elementwise / layout kernels (elementwise.hip) --------------------------------------
+void fortis_launch_scale(const float* src, float* dst, const float* vec, long rows, long n, int divide, hipStream_t s);
+void fortis_launch_mask_relu(const float* src, float* dst, long rows, long n, long tail, hipStream_t s);
+void fortis_launch_boundary_pre(const void* A, float* X, long NI, long NK, const void* mean, const void* vmax,
+                                const void* vmin, int host_esz, hipStream_t s);
+void fortis_launch_boundary_post(const float* Y, void* B, long NI, long NK, const void* scale, int host_esz, hipStream_t s);
+void fortis_launch_permute(const float* src, float* dst, long C, long S, int to_channels_first, hipStream_t s);
+
+// ---- convolution family (conv.hip) ---------------------------------------------------------
+struct ConvEpi {
+    const float* scale;  // per output channel multiplier (folded BatchNorm), or null
+    const float* shift;  // per output channel additive term (bias, folded BatchNorm), or null
+    int act;
+    float alpha;
+    const float* res;    // residual tensor added after the activation (same shape as output), or null
+};
+int fortis_launch_conv2d(const float* x, const float* w, float* y, long C, long H, long Wd, long F, long KH,
+                         long KW, long Ho, long Wo, long sh, long sw, long ph, long pw, const ConvEpi& e,
+                         long coff, long ctot, hipStream_t s);
+int fortis_launch_convt2d(const float* x, const float* w, float* y, long C, long H, long Wd, long F, long KH,
+                          long KW, long Ho, long Wo, long stride, long pad, const ConvEpi& e, long coff,
+                          long ctot, hipStream_t s);
+int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long D, long H, long Wd, long F,
+                         long KD, long KH, long KW, long Do, long Ho, long Wo, long pd, long ph, long pw,
+                         const ConvEpi& e, hipStream_t s);
+void fortis_launch_maxpool2d(const float* x, float* y, long C, long H, long Wd, long k, hipStream_t s);
+void fortis_launch_upsample(const float* x, float* y, long C, long D, long H, long Wd, long sfac, int nd, hipStream_t s);
+void fortis_launch_concat_copy(const float* x, float* y, long C, long S, long coff, hipStream_t s);

@@ -1,0 +1,111 @@
+// Memory-bound helpers of the step: per-feature scaling, the masked-ReLU head, the boundary
+// pre/post kernels (column-major host array <-> batch-major fp32 activations with the lifted
+// normalisation) and layout permutes.  All of them are HBM-bound; the transposing ones go through
+// a 32 x 33 LDS tile so that both the read and the write side are coalesced (the reference's
+// fortis_pre_k / fortis_post_k, trt_backend/e3sm_boundary.cu:9-20, are one-thread-per-element and
+// strided on one side).
+#include "common.h"
+
+#define EW_THREADS 256
+
+__global__ void scale_kernel(const float* __restrict__ src, float* __restrict__ dst, const float* __restrict__ vec,
+                             long total, long n, int divide)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const float v = src[idx], s = vec[idx % n];
+    dst[idx] = divide ? __fdiv_rn(v, s) : __fmul_rn(v, s);
+}
+void fortis_launch_scale(const float* src, float* dst, const float* vec, long rows, long n, int divide, hipStream_t s)
+{
+    const long total = rows * n;
+    if (total <= 0) return;
+    hipLaunchKernelGGL(scale_kernel, dim3((unsigned)cdiv(total, EW_THREADS)), dim3(EW_THREADS), 0, s, src, dst, vec, total, n, divide);
+    HIP_OK(hipGetLastError());
+}
+
+__global__ void mask_relu_kernel(const float* __restrict__ src, float* __restrict__ dst, long total, long n, long tail)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const float v = src[idx];
+    dst[idx] = (idx % n >= n - tail && v < 0.f) ? 0.f : v;
+}
+void fortis_launch_mask_relu(const float* src, float* dst, long rows, long n, long tail, hipStream_t s)
+{
+    const long total = rows * n;
+    if (total <= 0) return;
+    hipLaunchKernelGGL(mask_relu_kernel, dim3((unsigned)cdiv(total, EW_THREADS)), dim3(EW_THREADS), 0, s, src, dst, total, n, tail);
+    HIP_OK(hipGetLastError());
+}
+
+// dst[c][r] = f(src[r][c], r, c) for a row-major src[R][Cc]; 32 x 32 tiles, block (32, 8).
+template <typename TI, typename TO, typename F>
+__global__ void transpose_kernel(const TI* __restrict__ src, TO* __restrict__ dst, long R, long Cc, F f)
+{
+    __shared__ TO tile[32][33];
+    const long c0 = (long)blockIdx.x * 32, r0 = (long)blockIdx.y * 32;
+    for (int y = threadIdx.y; y < 32; y += 8) {
+        const long r = r0 + y, c = c0 + threadIdx.x;
+        if (r < R && c < Cc) tile[y][threadIdx.x] = f(src[r * Cc + c], r, c);
+    }
+    __syncthreads();
+    for (int y = threadIdx.y; y < 32; y += 8) {
+        const long c = c0 + y, r = r0 + threadIdx.x;
+        if (r < R && c < Cc) dst[c * R + r] = tile[threadIdx.x][y];
+    }
+}
+template <typename TI, typename TO, typename F>
+static void launch_transpose(const TI* src, TO* dst, long R, long Cc, F f, hipStream_t s)
+{
+    if (R <= 0 || Cc <= 0) return;
+    hipLaunchKernelGGL((transpose_kernel<TI, TO, F>), dim3((unsigned)cdiv(Cc, 32), (unsigned)cdiv(R, 32)), dim3(32, 8), 0, s,
+                       src, dst, R, Cc, f);
+    HIP_OK(hipGetLastError());
+}
+
+// pre: the host array (NI, NK) column-major is the row-major matrix [NK][NI]; X = its transpose
+// with (a - mean[k]) / (max[k] - min[k]) evaluated in the host type, then cast to fp32.
+template <typename H>
+struct PreF {
+    const H* mean; const H* vmax; const H* vmin;
+    __device__ float operator()(H a, long k, long) const
+    {
+        const H m = mean ? mean[k] : (H)0, range = vmax ? (vmax[k] - (vmin ? vmin[k] : (H)0)) : (H)1;
+        return (float)((a - m) / range);
+    }
+};
+// post: Y[NI][NK] row-major -> B[NK][NI] (column-major (NI, NK)) with (H)y / scale[k].
+template <typename H>
+struct PostF {
+    const H* scale;
+    __device__ H operator()(float y, long, long k) const { return scale ? (H)y / scale[k] : (H)y; }
+};
+struct IdF { __device__ float operator()(float v, long, long) const { return v; } };
+
+void fortis_launch_boundary_pre(const void* A, float* X, long NI, long NK, const void* mean, const void* vmax,
+                                const void* vmin, int host_esz, hipStream_t s)
+{
+    if (host_esz == 8) {
+        PreF<double> f = { (const double*)mean, (const double*)vmax, (const double*)vmin };
+        launch_transpose((const double*)A, X, NK, NI, f, s);
+    } else {
+        PreF<float> f = { (const float*)mean, (const float*)vmax, (const float*)vmin };
+        launch_transpose((const float*)A, X, NK, NI, f, s);
+    }
+}
+void fortis_launch_boundary_post(const float* Y, void* B, long NI, long NK, const void* scale, int host_esz, hipStream_t s)
+{
+    if (host_esz == 8) {
+        PostF<double> f = { (const double*)scale };
+        launch_transpose(Y, (double*)B, NI, NK, f, s);
+    } else {
+        PostF<float> f = { (const float*)scale };
+        launch_transpose(Y, (float*)B, NI, NK, f, s);
+    }
+}
+void fortis_launch_permute(const float* src, float* dst, long C, long S, int to_channels_first, hipStream_t s)
+{
+    if (to_channels_first) launch_transpose(src, dst, S, C, IdF(), s);   // [S][C] -> [C][S]
+    else launch_transpose(src, dst, C, S, IdF(), s);                      // [C][S] -> [S][C]
+}

@@ -1,0 +1,710 @@
+// Model plan (what the MLIR-generated `mlp_kernel` host function is in the reference), the step
+// binding, and the host-facing entry points of the generated shim (driver/fortis_shim.py:54-135):
+// buffer ownership, upload/download choreography, pack/unpack staging, graph capture on the
+// second call and replay afterwards, with an eager fallback.
+#include <vector>
+#include "common.h"
+
+enum OpKind { OP_LINEAR, OP_SCALE, OP_MASK_RELU, OP_PRE, OP_POST, OP_CONV2D, OP_CONVT2D, OP_MAXPOOL, OP_UPSAMPLE,
+              OP_CONCAT, OP_CONV3D, OP_PERMUTE };
+
+struct Op {
+    OpKind kind;
+    int src = -1, dst = -1, res = -1;
+    long B = 0, K = 0, N = 0;                 // linear; rows/n for scale & mask
+    int act = 0; float alpha = 0.f;
+    int flag = 0;                             // scale: divide; permute: to_channels_first; boundary: host_esz
+    long tail = 0;
+    long C = 0, D = 1, H = 0, W = 0, F = 0, KD = 1, KH = 1, KW = 1, stride = 1, pad = 0, opad = 0, coff = 0, ctot = 0, sfac = 1;
+    int nd = 2;
+    std::vector<float> w, b, v0, v1, v2, v3;  // host copies: weights, bias, vectors (bn / boundary)
+    std::vector<double> d0, d1, d2;           // f64 boundary vectors
+    float eps = 1e-5f;
+    bool has_bias = false, has_bn = false, has_v[3] = { false, false, false };
+};
+
+enum ExecKind { EX_CHAIN, EX_GEMM, EX_SCALE, EX_MASK, EX_PRE, EX_POST, EX_CONV2D, EX_CONVT2D, EX_MAXPOOL, EX_UPSAMPLE,
+                EX_CONCAT, EX_CONV3D, EX_PERMUTE };
+struct Exec {
+    ExecKind kind;
+    int src = -1, dst = -1, res = -1;
+    long rows = 0, rows_cap = 0;
+    ChainDesc chain;
+    // gemm
+    const float *W = nullptr, *bias = nullptr, *out_scale = nullptr, *vec = nullptr;
+    long K = 0, N = 0, mask_tail = 0;
+    int act = 0; float alpha = 0.f;
+    int flag = 0;
+    const void *p0 = nullptr, *p1 = nullptr, *p2 = nullptr;
+    const Op* op = nullptr;
+    ConvEpi epi = { nullptr, nullptr, 0, 0.f, nullptr };
+};
+
+struct fortis_plan {
+    std::vector<long> tbytes;
+    std::vector<void*> tptr;
+    std::vector<Op> ops;
+    std::vector<Exec> exec;
+    std::vector<void*> owned;   // device allocations owned by the plan (weights, vectors)
+    bool finalized = false;
+    int in_t = -1, out_t = -1;
+    long rows0 = 0;             // rows at finalize (row-wise plans), for run-time extents
+};
+
+static void* upload(fortis_plan* p, const void* h, size_t nbytes)
+{
+    void* d = nullptr;
+    HIP_OK(hipMalloc(&d, nbytes ? nbytes : 4));
+    if (nbytes) HIP_OK(hipMemcpy(d, h, nbytes, hipMemcpyHostToDevice));
+    p->owned.push_back(d);
+    return d;
+}
+
+static int bad(const char* what) { fprintf(stderr, "fortis_plan: %s\n", what); return -1; }
+static bool tensor_ok(fortis_plan* p, int t, long need_bytes)
+{
+    return t >= 0 && t < (int)p->tbytes.size() && p->tbytes[t] >= need_bytes;
+}
+
+extern "C" {
+
+fortis_plan* fortis_plan_create(void) { return new fortis_plan(); }
+void fortis_plan_destroy(fortis_plan* p)
+{
+    if (!p) return;
+    for (void* d : p->owned) HIP_OK(hipFree(d));
+    for (void* t : p->tptr) fortis_free(t);
+    delete p;
+}
+int fortis_plan_tensor(fortis_plan* p, long nbytes)
+{
+    if (!p || p->finalized || nbytes <= 0) return -1;
+    p->tbytes.push_back(nbytes);
+    return (int)p->tbytes.size() - 1;
+}
+
+int fortis_plan_linear(fortis_plan* p, int src, int dst, const float* W, const float* bias, long B, long K, long N,
+                       int act, float alpha)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (B <= 0 || K <= 0 || N <= 0 || !W || act < 0 || act > 2) return bad("linear: bad shape or arguments");
+    if (!tensor_ok(p, src, B * K * 4) || !tensor_ok(p, dst, B * N * 4) || src == dst) return bad("linear: tensors too small or aliased");
+    Op o; o.kind = OP_LINEAR; o.src = src; o.dst = dst; o.B = B; o.K = K; o.N = N; o.act = act; o.alpha = alpha;
+    o.w.assign(W, W + N * K);
+    if (bias) { o.b.assign(bias, bias + N); o.has_bias = true; }
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_scale(fortis_plan* p, int src, int dst, const float* vec, long rows, long n, int divide)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (rows <= 0 || n <= 0 || !vec) return bad("scale: bad shape");
+    if (!tensor_ok(p, src, rows * n * 4) || !tensor_ok(p, dst, rows * n * 4)) return bad("scale: tensors too small");
+    Op o; o.kind = OP_SCALE; o.src = src; o.dst = dst; o.B = rows; o.N = n; o.K = n; o.flag = divide ? 1 : 0;
+    o.v0.assign(vec, vec + n);
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_mask_relu(fortis_plan* p, int src, int dst, long rows, long n, long tail)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (rows <= 0 || n <= 0 || tail < 0 || tail > n) return bad("mask_relu: bad shape");
+    if (!tensor_ok(p, src, rows * n * 4) || !tensor_ok(p, dst, rows * n * 4)) return bad("mask_relu: tensors too small");
+    Op o; o.kind = OP_MASK_RELU; o.src = src; o.dst = dst; o.B = rows; o.N = n; o.K = n; o.tail = tail;
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+static void take_vec(Op& o, int which, const void* v, long n, int esz)
+{
+    if (!v) return;
+    o.has_v[which] = true;
+    if (esz == 8) { std::vector<double>& d = which == 0 ? o.d0 : which == 1 ? o.d1 : o.d2; d.assign((const double*)v, (const double*)v + n); }
+    else { std::vector<float>& f = which == 0 ? o.v0 : which == 1 ? o.v1 : o.v2; f.assign((const float*)v, (const float*)v + n); }
+}
+int fortis_plan_boundary_pre(fortis_plan* p, int src, int dst, long NI, long NK, const void* mean, const void* vmax,
+                             const void* vmin, int host_esz)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (NI <= 0 || NK <= 0 || (host_esz != 4 && host_esz != 8)) return bad("boundary_pre: bad shape or element size");
+    if (!tensor_ok(p, src, NI * NK * host_esz) || !tensor_ok(p, dst, NI * NK * 4) || src == dst) return bad("boundary_pre: tensors too small or aliased");
+    Op o; o.kind = OP_PRE; o.src = src; o.dst = dst; o.B = NI; o.N = NK; o.flag = host_esz;
+    take_vec(o, 0, mean, NK, host_esz); take_vec(o, 1, vmax, NK, host_esz); take_vec(o, 2, vmin, NK, host_esz);
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_boundary_post(fortis_plan* p, int src, int dst, long NI, long NK, const void* scale, int host_esz)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (NI <= 0 || NK <= 0 || (host_esz != 4 && host_esz != 8)) return bad("boundary_post: bad shape or element size");
+    if (!tensor_ok(p, src, NI * NK * 4) || !tensor_ok(p, dst, NI * NK * host_esz) || src == dst) return bad("boundary_post: tensors too small or aliased");
+    Op o; o.kind = OP_POST; o.src = src; o.dst = dst; o.B = NI; o.N = NK; o.flag = host_esz;
+    take_vec(o, 0, scale, NK, host_esz);
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+
+int fortis_plan_conv2d(fortis_plan* p, int src, int dst, const float* W, const float* bias, const float* bn_gamma,
+                       const float* bn_beta, const float* bn_mean, const float* bn_var, float bn_eps, long C, long H,
+                       long Wd, long F, long KH, long KW, long stride, long pad, int act, float alpha, long coff, long ctot)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (C <= 0 || H <= 0 || Wd <= 0 || F <= 0 || KH <= 0 || KW <= 0 || stride <= 0 || pad < 0 || !W) return bad("conv2d: bad shape");
+    const long Ho = (H + 2 * pad - KH) / stride + 1, Wo = (Wd + 2 * pad - KW) / stride + 1;
+    if (ctot <= 0) { ctot = F; coff = 0; }
+    if (Ho <= 0 || Wo <= 0 || coff < 0 || coff + F > ctot) return bad("conv2d: bad output shape or channel offset");
+    if (!tensor_ok(p, src, C * H * Wd * 4) || !tensor_ok(p, dst, ctot * Ho * Wo * 4) || src == dst) return bad("conv2d: tensors too small or aliased");
+    const int nbn = (bn_gamma != 0) + (bn_beta != 0) + (bn_mean != 0) + (bn_var != 0);
+    if (nbn != 0 && nbn != 4) return bad("conv2d: give all four BatchNorm vectors or none");
+    Op o; o.kind = OP_CONV2D; o.src = src; o.dst = dst; o.C = C; o.H = H; o.W = Wd; o.F = F; o.KH = KH; o.KW = KW;
+    o.stride = stride; o.pad = pad; o.act = act; o.alpha = alpha; o.coff = coff; o.ctot = ctot; o.eps = bn_eps;
+    o.w.assign(W, W + F * C * KH * KW);
+    if (bias) { o.b.assign(bias, bias + F); o.has_bias = true; }
+    if (nbn) { o.has_bn = true; o.v0.assign(bn_gamma, bn_gamma + F); o.v1.assign(bn_beta, bn_beta + F); o.v2.assign(bn_mean, bn_mean + F); o.v3.assign(bn_var, bn_var + F); }
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_convt2d(fortis_plan* p, int src, int dst, const float* W, const float* bias, long C, long H, long Wd,
+                        long F, long KH, long KW, long stride, long pad, long output_padding, int act, float alpha,
+                        long coff, long ctot)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (C <= 0 || H <= 0 || Wd <= 0 || F <= 0 || KH <= 0 || KW <= 0 || stride <= 0 || pad < 0 || !W) return bad("convt2d: bad shape");
+    const long Ho = (H - 1) * stride - 2 * pad + KH + output_padding, Wo = (Wd - 1) * stride - 2 * pad + KW + output_padding;
+    if (ctot <= 0) { ctot = F; coff = 0; }
+    if (Ho <= 0 || Wo <= 0 || coff < 0 || coff + F > ctot) return bad("convt2d: bad output shape or channel offset");
+    if (!tensor_ok(p, src, C * H * Wd * 4) || !tensor_ok(p, dst, ctot * Ho * Wo * 4) || src == dst) return bad("convt2d: tensors too small or aliased");
+    Op o; o.kind = OP_CONVT2D; o.src = src; o.dst = dst; o.C = C; o.H = H; o.W = Wd; o.F = F; o.KH = KH; o.KW = KW;
+    o.stride = stride; o.pad = pad; o.opad = output_padding; o.act = act; o.alpha = alpha; o.coff = coff; o.ctot = ctot;
+    o.w.assign(W, W + C * F * KH * KW);
+    if (bias) { o.b.assign(bias, bias + F); o.has_bias = true; }
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_maxpool2d(fortis_plan* p, int src, int dst, long C, long H, long Wd, long k)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (C <= 0 || H <= 0 || Wd <= 0 || k <= 0 || H % k || Wd % k) return bad("maxpool2d: bad shape");
+    if (!tensor_ok(p, src, C * H * Wd * 4) || !tensor_ok(p, dst, C * (H / k) * (Wd / k) * 4) || src == dst) return bad("maxpool2d: tensors too small or aliased");
+    Op o; o.kind = OP_MAXPOOL; o.src = src; o.dst = dst; o.C = C; o.H = H; o.W = Wd; o.KH = k;
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_upsample(fortis_plan* p, int src, int dst, long C, long D, long H, long Wd, long s, int nd)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (C <= 0 || D <= 0 || H <= 0 || Wd <= 0 || s <= 0 || (nd != 2 && nd != 3)) return bad("upsample: bad shape");
+    const long out = C * (nd == 3 ? D * s : D) * H * s * Wd * s;
+    if (!tensor_ok(p, src, C * D * H * Wd * 4) || !tensor_ok(p, dst, out * 4) || src == dst) return bad("upsample: tensors too small or aliased");
+    Op o; o.kind = OP_UPSAMPLE; o.src = src; o.dst = dst; o.C = C; o.D = D; o.H = H; o.W = Wd; o.sfac = s; o.nd = nd;
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_concat_copy(fortis_plan* p, int src, int dst, long C, long S, long coff, long ctot)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (C <= 0 || S <= 0 || coff < 0 || coff + C > ctot) return bad("concat_copy: bad shape");
+    if (!tensor_ok(p, src, C * S * 4) || !tensor_ok(p, dst, ctot * S * 4) || src == dst) return bad("concat_copy: tensors too small or aliased");
+    Op o; o.kind = OP_CONCAT; o.src = src; o.dst = dst; o.C = C; o.H = S; o.coff = coff; o.ctot = ctot;
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_conv3d(fortis_plan* p, int src, int dst, int res, const float* W, const float* bias, long C, long D,
+                       long H, long Wd, long F, long K, long pad, int act, float alpha)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (C <= 0 || D <= 0 || H <= 0 || Wd <= 0 || F <= 0 || K <= 0 || pad < 0 || !W) return bad("conv3d: bad shape");
+    const long Do = D + 2 * pad - K + 1, Ho = H + 2 * pad - K + 1, Wo = Wd + 2 * pad - K + 1;
+    if (Do <= 0 || Ho <= 0 || Wo <= 0) return bad("conv3d: empty output");
+    if (!tensor_ok(p, src, C * D * H * Wd * 4) || !tensor_ok(p, dst, F * Do * Ho * Wo * 4) || src == dst) return bad("conv3d: tensors too small or aliased");
+    if (res >= 0 && (!tensor_ok(p, res, F * Do * Ho * Wo * 4) || res == dst)) return bad("conv3d: residual tensor too small or aliased");
+    Op o; o.kind = OP_CONV3D; o.src = src; o.dst = dst; o.res = res; o.C = C; o.D = D; o.H = H; o.W = Wd; o.F = F;
+    o.KD = o.KH = o.KW = K; o.pad = pad; o.act = act; o.alpha = alpha;
+    o.w.assign(W, W + F * C * K * K * K);
+    if (bias) { o.b.assign(bias, bias + F); o.has_bias = true; }
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+int fortis_plan_permute(fortis_plan* p, int src, int dst, long C, long S, int to_channels_first)
+{
+    if (!p || p->finalized) return bad("plan is null or already finalized");
+    if (C <= 0 || S <= 0) return bad("permute: bad shape");
+    if (!tensor_ok(p, src, C * S * 4) || !tensor_ok(p, dst, C * S * 4) || src == dst) return bad("permute: tensors too small or aliased");
+    Op o; o.kind = OP_PERMUTE; o.src = src; o.dst = dst; o.C = C; o.H = S; o.flag = to_channels_first ? 1 : 0;
+    p->ops.push_back(std::move(o));
+    return 0;
+}
+
+}  // extern "C"
+
+// ---- finalize: fusion + uploads -----------------------------------------------------------------
+static int uses_of(const fortis_plan* p, int t)
+{
+    int n = (t == p->out_t) ? 1 : 0;
+    for (const Op& o : p->ops) n += (o.src == t) + (o.res == t);
+    return n;
+}
+
+// Tries to turn ops[i..] into one LDS-resident chain.  Returns the number of ops consumed (0 if none).
+static size_t try_chain(fortis_plan* p, size_t i, Exec* ex)
+{
+    const std::vector<Op>& ops = p->ops;
+    size_t j = i;
+    const Op* in_div = nullptr;
+    if (ops[j].kind == OP_SCALE && ops[j].flag == 1 && j + 1 < ops.size() && ops[j + 1].kind == OP_LINEAR &&
+        ops[j + 1].src == ops[j].dst && uses_of(p, ops[j].dst) == 1 && ops[j].B == ops[j + 1].B && ops[j].N == ops[j + 1].K) {
+        in_div = &ops[j];
+        j++;
+    }
+    if (ops[j].kind != OP_LINEAR) return 0;
+    std::vector<const Op*> lin;
+    const long rows = ops[j].B;
+    while (j < ops.size() && ops[j].kind == OP_LINEAR && ops[j].B == rows && ops[j].K <= FORTIS_CHAIN_MAX_WIDTH &&
+           ops[j].N <= FORTIS_CHAIN_MAX_WIDTH && (int)lin.size() < FORTIS_CHAIN_MAX_LAYERS &&
+           (lin.empty() || (ops[j].src == lin.back()->dst && uses_of(p, lin.back()->dst) == 1))) {
+        lin.push_back(&ops[j]);
+        j++;
+    }
+    if (lin.empty()) return 0;
+    if (in_div && lin[0]->src != in_div->dst) return 0;
+    const Op* out_mul = nullptr;
+    const Op* mask = nullptr;
+    int last_dst = lin.back()->dst;
+    if (j < ops.size() && ops[j].kind == OP_SCALE && ops[j].flag == 0 && ops[j].src == last_dst && uses_of(p, last_dst) == 1 &&
+        ops[j].B == rows && ops[j].N == lin.back()->N) { out_mul = &ops[j]; last_dst = ops[j].dst; j++; }
+    if (!out_mul && j < ops.size() && ops[j].kind == OP_MASK_RELU && ops[j].src == last_dst && uses_of(p, last_dst) == 1 &&
+        ops[j].B == rows && ops[j].N == lin.back()->N) { mask = &ops[j]; last_dst = ops[j].dst; j++; }
+    memset(&ex->chain, 0, sizeof ex->chain);
+    ex->kind = EX_CHAIN;
+    ex->src = in_div ? in_div->src : lin[0]->src;
+    ex->dst = last_dst;
+    ex->rows = ex->rows_cap = rows;
+    ChainDesc& d = ex->chain;
+    d.nlayers = (int)lin.size();
+    for (size_t l = 0; l < lin.size(); l++) {
+        ChainLayer& L = d.L[l];
+        L.K = (int)lin[l]->K; L.N = (int)lin[l]->N; L.act = lin[l]->act; L.alpha = lin[l]->alpha;
+        float* wp = fortis_chain_pack_weights(lin[l]->w.data(), L.N, L.K, &L.Kp, &L.Np);
+        p->owned.push_back(wp);
+        float* bp = fortis_chain_pack_bias(lin[l]->has_bias ? lin[l]->b.data() : nullptr, L.N, L.Np);
+        p->owned.push_back(bp);
+        L.Wp = wp; L.bias = bp;
+    }
+    if (in_div) d.in_div = (const float*)upload(p, in_div->v0.data(), in_div->v0.size() * 4);
+    if (out_mul) d.out_mul = (const float*)upload(p, out_mul->v0.data(), out_mul->v0.size() * 4);
+    d.mask_tail = mask ? (int)mask->tail : 0;
+    d.ld = fortis_chain_ld(d);
+    return j - i;
+}
+
+extern "C" {
+
+int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
+{
+    if (!p || p->finalized) return bad("finalize: plan is null or already finalized");
+    if (in_t < 0 || in_t >= (int)p->tbytes.size() || out_t < 0 || out_t >= (int)p->tbytes.size()) return bad("finalize: bad input/output tensor");
+    if (p->ops.empty()) return bad("finalize: empty plan");
+    p->in_t = in_t; p->out_t = out_t;
+    (void)fortis_stream_get();
+    for (long nb : p->tbytes) {
+        void* d = fortis_alloc(nb);
+        if (!d) return bad("finalize: out of device memory");
+        p->tptr.push_back(d);
+    }
+    const std::vector<Op>& ops = p->ops;
+    for (size_t i = 0; i < ops.size();) {
+        Exec ex;
+        size_t took = try_chain(p, i, &ex);
+        if (took) { p->exec.push_back(ex); i += took; continue; }
+        const Op& o = ops[i];
+        ex.src = o.src; ex.dst = o.dst; ex.res = o.res; ex.op = &ops[i];
+        size_t adv = 1;
+        switch (o.kind) {
+            case OP_LINEAR: {
+                ex.kind = EX_GEMM; ex.rows = ex.rows_cap = o.B; ex.K = o.K; ex.N = o.N; ex.act = o.act; ex.alpha = o.alpha;
+                ex.W = (const float*)upload(p, o.w.data(), o.w.size() * 4);
+                ex.bias = o.has_bias ? (const float*)upload(p, o.b.data(), o.b.size() * 4) : nullptr;
+                // fold a directly following output scale or masked-ReLU head into the epilogue
+                if (i + 1 < ops.size() && ops[i + 1].src == o.dst && uses_of(p, o.dst) == 1 && ops[i + 1].B == o.B && ops[i + 1].N == o.N) {
+                    if (ops[i + 1].kind == OP_SCALE && ops[i + 1].flag == 0) {
+                        ex.out_scale = (const float*)upload(p, ops[i + 1].v0.data(), ops[i + 1].v0.size() * 4);
+                        ex.dst = ops[i + 1].dst; adv = 2;
+                    } else if (ops[i + 1].kind == OP_MASK_RELU) {
+                        ex.mask_tail = ops[i + 1].tail; ex.dst = ops[i + 1].dst; adv = 2;
+                    }
+                }
+                break;
+            }
+            case OP_SCALE:
+                ex.kind = EX_SCALE; ex.rows = ex.rows_cap = o.B; ex.N = o.N; ex.flag = o.flag;
+                ex.vec = (const float*)upload(p, o.v0.data(), o.v0.size() * 4);
+                break;
+            case OP_MASK_RELU:
+                ex.kind = EX_MASK; ex.rows = ex.rows_cap = o.B; ex.N = o.N; ex.mask_tail = o.tail;
+                break;
+            case OP_PRE:
+            case OP_POST: {
+                ex.kind = o.kind == OP_PRE ? EX_PRE : EX_POST; ex.rows = ex.rows_cap = o.B; ex.N = o.N; ex.flag = o.flag;
+                const void* hv[3]; size_t nb = (size_t)o.N * o.flag;
+                hv[0] = o.flag == 8 ? (const void*)o.d0.data() : (const void*)o.v0.data();
+                hv[1] = o.flag == 8 ? (const void*)o.d1.data() : (const void*)o.v1.data();
+                hv[2] = o.flag == 8 ? (const void*)o.d2.data() : (const void*)o.v2.data();
+                ex.p0 = o.has_v[0] ? upload(p, hv[0], nb) : nullptr;
+                ex.p1 = o.has_v[1] ? upload(p, hv[1], nb) : nullptr;
+                ex.p2 = o.has_v[2] ? upload(p, hv[2], nb) : nullptr;
+                break;
+            }
+            case OP_CONV2D:
+            case OP_CONVT2D:
+            case OP_CONV3D: {
+                ex.kind = o.kind == OP_CONV2D ? EX_CONV2D : o.kind == OP_CONVT2D ? EX_CONVT2D : EX_CONV3D;
+                ex.W = (const float*)upload(p, o.w.data(), o.w.size() * 4);
+                // y = act(scale * conv + shift): bias and BatchNorm-eval folded into two vectors.
+                // scale = gamma / sqrt(var + eps); shift = beta + (bias - mean) * scale.
+                std::vector<float> scale, shift;
+                if (o.has_bn) {
+                    scale.resize(o.F); shift.resize(o.F);
+                    for (long f = 0; f < o.F; f++) {
+                        const double sc = (double)o.v0[f] / sqrt((double)o.v3[f] + (double)o.eps);
+                        scale[f] = (float)sc;
+                        shift[f] = (float)((double)o.v1[f] + ((o.has_bias ? (double)o.b[f] : 0.0) - (double)o.v2[f]) * sc);
+                    }
+                } else if (o.has_bias) shift = o.b;
+                ex.epi.scale = scale.empty() ? nullptr : (const float*)upload(p, scale.data(), scale.size() * 4);
+                ex.epi.shift = shift.empty() ? nullptr : (const float*)upload(p, shift.data(), shift.size() * 4);
+                ex.epi.act = o.act; ex.epi.alpha = o.alpha;
+                break;
+            }
+            case OP_MAXPOOL: ex.kind = EX_MAXPOOL; break;
+            case OP_UPSAMPLE: ex.kind = EX_UPSAMPLE; break;
+            case OP_CONCAT: ex.kind = EX_CONCAT; break;
+            case OP_PERMUTE: ex.kind = EX_PERMUTE; break;
+        }
+        p->exec.push_back(ex);
+        i += adv;
+    }
+    bool rowwise = true;
+    long rows = -1;
+    for (const Exec& e : p->exec) {
+        if (e.kind > EX_MASK) { rowwise = false; break; }
+        if (rows < 0) rows = e.rows; else if (rows != e.rows) rowwise = false;
+    }
+    p->rows0 = rowwise ? rows : 0;
+    p->finalized = true;
+    HIP_OK(hipDeviceSynchronize());
+    return 0;
+}
+
+void fortis_plan_run(fortis_plan* p)
+{
+    if (!p || !p->finalized) { fprintf(stderr, "fortis_plan_run: plan not finalized\n"); return; }
+    hipStream_t s = fortis_stream_get();
+    for (const Exec& e : p->exec) {
+        const float* src = (const float*)p->tptr[e.src];
+        float* dst = (float*)p->tptr[e.dst];
+        const Op* o = e.op;
+        int rc = 0;
+        switch (e.kind) {
+            case EX_CHAIN: fortis_launch_chain(e.chain, src, dst, e.rows, s); break;
+            case EX_GEMM: rc = fortis_launch_gemm(src, e.W, e.bias, dst, e.rows, e.N, e.K, e.act, e.alpha, e.out_scale, e.mask_tail, s); break;
+            case EX_SCALE: fortis_launch_scale(src, dst, e.vec, e.rows, e.N, e.flag, s); break;
+            case EX_MASK: fortis_launch_mask_relu(src, dst, e.rows, e.N, e.mask_tail, s); break;
+            case EX_PRE: fortis_launch_boundary_pre(p->tptr[e.src], dst, e.rows, e.N, e.p0, e.p1, e.p2, e.flag, s); break;
+            case EX_POST: fortis_launch_boundary_post(src, p->tptr[e.dst], e.rows, e.N, e.p0, e.flag, s); break;
+            case EX_CONV2D: {
+                const long Ho = (o->H + 2 * o->pad - o->KH) / o->stride + 1, Wo = (o->W + 2 * o->pad - o->KW) / o->stride + 1;
+                rc = fortis_launch_conv2d(src, e.W, dst, o->C, o->H, o->W, o->F, o->KH, o->KW, Ho, Wo, o->stride, o->stride,
+                                          o->pad, o->pad, e.epi, o->coff, o->ctot, s);
+                break;
+            }
+            case EX_CONVT2D: {
+                const long Ho = (o->H - 1) * o->stride - 2 * o->pad + o->KH + o->opad, Wo = (o->W - 1) * o->stride - 2 * o->pad + o->KW + o->opad;
+                rc = fortis_launch_convt2d(src, e.W, dst, o->C, o->H, o->W, o->F, o->KH, o->KW, Ho, Wo, o->stride, o->pad, e.epi,
+                                           o->coff, o->ctot, s);
+                break;
+            }
+            case EX_CONV3D: {
+                ConvEpi epi = e.epi;
+                epi.res = e.res >= 0 ? (const float*)p->tptr[e.res] : nullptr;
+                const long Do = o->D + 2 * o->pad - o->KD + 1, Ho = o->H + 2 * o->pad - o->KH + 1, Wo = o->W + 2 * o->pad - o->KW + 1;
+                rc = fortis_launch_conv3d(src, e.W, dst, o->C, o->D, o->H, o->W, o->F, o->KD, o->KH, o->KW, Do, Ho, Wo, o->pad,
+                                          o->pad, o->pad, epi, s);
+                break;
+            }
+            case EX_MAXPOOL: fortis_launch_maxpool2d(src, dst, o->C, o->H, o->W, o->KH, s); break;
+            case EX_UPSAMPLE: fortis_launch_upsample(src, dst, o->C, o->D, o->H, o->W, o->sfac, o->nd, s); break;
+            case EX_CONCAT: fortis_launch_concat_copy(src, dst + o->coff * o->H, o->C, o->H, o->coff, s); break;
+            case EX_PERMUTE: fortis_launch_permute(src, dst, o->C, o->H, o->flag, s); break;
+        }
+        if (rc != 0) fprintf(stderr, "fortis_plan_run: an op was rejected by its kernel launcher\n");
+    }
+}
+
+void* fortis_plan_tensor_ptr(fortis_plan* p, int t)
+{
+    if (!p || !p->finalized || t < 0 || t >= (int)p->tptr.size()) return nullptr;
+    return p->tptr[t];
+}
+int fortis_plan_num_kernels(fortis_plan* p) { return p && p->finalized ? (int)p->exec.size() : -1; }
+
+}  // extern "C"
+
+int fortis_plan_as_chain(fortis_plan* p, ChainDesc* out)
+{
+    if (!p || !p->finalized || p->exec.size() != 1 || p->exec[0].kind != EX_CHAIN) return -1;
+    *out = p->exec[0].chain;
+    return 0;
+}
+
+// Run-time extents: row-wise plans can be re-run on fewer rows than they were sized for.
+static int plan_set_rows(fortis_plan* p, long rows)
+{
+    if (!p || !p->finalized || p->rows0 <= 0 || rows <= 0 || rows > p->rows0) return -1;
+    for (Exec& e : p->exec) e.rows = rows;
+    return 0;
+}
+
+// ================================ step binding and entries ========================================
+void fortis_stencil_reset_internal();
+
+struct Step {
+    fortis_plan* plan = nullptr;
+    fortis_host_t h;
+    void *din = nullptr, *dout = nullptr;
+    void *X = nullptr, *Y = nullptr;          // pinned pack/unpack staging (driver/fortis_shim.py:102-106)
+    hipGraphExec_t gexec = nullptr;
+    int ncalls = 0;
+    long count0 = 0;
+};
+static Step g_step;
+
+static void drop_graph()
+{
+    if (g_step.gexec) { HIP_OK(hipGraphExecDestroy(g_step.gexec)); g_step.gexec = nullptr; }
+    g_step.ncalls = 0;
+}
+
+extern "C" {
+
+int fortis_step_bind(fortis_plan* p, const fortis_host_t* host)
+{
+    if (!p || !p->finalized || !host) return bad("step_bind: plan not finalized or host facts missing");
+    if (host->n_in <= 0 || host->n_out <= 0 || (host->in_esz != 4 && host->in_esz != 8) || (host->out_esz != 4 && host->out_esz != 8))
+        return bad("step_bind: bad sizes");
+    if (p->tbytes[p->in_t] < host->n_in * host->in_esz || p->tbytes[p->out_t] < host->n_out * host->out_esz)
+        return bad("step_bind: model input/output tensors smaller than the host's arrays");
+    if (host->verdict == FORTIS_VERDICT_BATCHED && (host->count <= 0 || host->n_in % host->count || host->n_out % host->count))
+        return bad("step_bind: batched verdict needs a row count dividing n_in and n_out");
+    drop_graph();
+    if (g_step.X) { HIP_OK(hipHostFree(g_step.X)); g_step.X = nullptr; }
+    if (g_step.Y) { HIP_OK(hipHostFree(g_step.Y)); g_step.Y = nullptr; }
+    g_step.plan = p;
+    g_step.h = *host;
+    g_step.din = p->tptr[p->in_t];
+    g_step.dout = p->tptr[p->out_t];
+    g_step.count0 = host->count;
+    return 0;
+}
+void fortis_step_reset(void)
+{
+    drop_graph();
+    if (g_step.X) { HIP_OK(hipHostFree(g_step.X)); }
+    if (g_step.Y) { HIP_OK(hipHostFree(g_step.Y)); }
+    g_step = Step();
+    fortis_stencil_reset_internal();
+}
+int fortis_step_graph_active(void) { return g_step.gexec != nullptr; }
+
+static bool bound(const char* who)
+{
+    if (!g_step.plan) { fprintf(stderr, "%s: no step bound (fortis_step_bind was not called)\n", who); return false; }
+    return true;
+}
+
+void* fortis_model_input(void) { return g_step.din; }
+void* fortis_model_output(void) { return g_step.dout; }
+
+void mlp_forward_dev(void)
+{
+    if (!bound("mlp_forward_dev")) return;
+    hipStream_t s = fortis_stream_get();
+    if (g_step.gexec) { HIP_OK(hipGraphLaunch(g_step.gexec, s)); return; }
+    const int cap = (++g_step.ncalls == 2) && (g_step.h.graph || getenv("FORTIS_GRAPH") != 0);
+    if (cap) {
+        fortis_capturing = 1;
+        if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+            fortis_capturing = 0;
+            (void)hipGetLastError();
+            fprintf(stderr, "fortis: graph capture failed, running eagerly\n");
+            fortis_plan_run(g_step.plan);
+            return;
+        }
+    }
+    fortis_plan_run(g_step.plan);
+    if (cap) {
+        hipGraph_t g = nullptr;
+        fortis_capturing = 0;
+        if (hipStreamEndCapture(s, &g) == hipSuccess && g && hipGraphInstantiate(&g_step.gexec, g, nullptr, nullptr, 0) == hipSuccess) {
+            HIP_OK(hipGraphLaunch(g_step.gexec, s));
+        } else {
+            fprintf(stderr, "fortis: graph capture failed, running eagerly\n");
+            g_step.gexec = nullptr;
+            (void)hipGetLastError();
+            fortis_plan_run(g_step.plan);
+        }
+        if (g) HIP_OK(hipGraphDestroy(g));
+    }
+}
+
+void mlp_upload(void* in)
+{
+    if (!bound("mlp_upload")) return;
+    HIP_OK(hipMemcpyAsync(g_step.din, in, (size_t)g_step.h.n_in * g_step.h.in_esz, hipMemcpyHostToDevice, fortis_stream_get()));
+}
+void mlp_download(void* out)
+{
+    if (!bound("mlp_download")) return;
+    hipStream_t s = fortis_stream_get();
+    HIP_OK(hipMemcpyAsync(out, g_step.dout, (size_t)g_step.h.n_out * g_step.h.out_esz, hipMemcpyDeviceToHost, s));
+    HIP_OK(hipStreamSynchronize(s));
+}
+
+static void setup_xy()
+{
+    // page-locked staging is allocated, never registered over existing host memory
+    HIP_OK(hipHostMalloc(&g_step.X, (size_t)g_step.h.n_in * g_step.h.in_esz, hipHostMallocDefault));
+    HIP_OK(hipHostMalloc(&g_step.Y, (size_t)g_step.h.n_out * g_step.h.out_esz, hipHostMallocDefault));
+}
+void fortis_pack(void* row, int col)
+{
+    if (!bound("fortis_pack")) return;
+    if (!g_step.X) setup_xy();
+    const size_t nin = (size_t)(g_step.h.n_in / g_step.count0) * g_step.h.in_esz;
+    memcpy((char*)g_step.X + (size_t)col * nin, row, nin);
+}
+void fortis_unpack(void* row, int col)
+{
+    if (!bound("fortis_unpack")) return;
+    if (!g_step.Y) setup_xy();
+    const size_t nout = (size_t)(g_step.h.n_out / g_step.count0) * g_step.h.out_esz;
+    memcpy(row, (char*)g_step.Y + (size_t)col * nout, nout);
+}
+
+void mlp_forward_batched(void* in, void* out)
+{
+    if (!bound("mlp_forward_batched")) return;
+    const fortis_host_t& h = g_step.h;
+    hipStream_t s = fortis_stream_get();
+    if (h.verdict != FORTIS_VERDICT_BATCHED) { fprintf(stderr, "mlp_forward_batched: the bound step is not a batched build\n"); return; }
+    const size_t NIN = (size_t)(h.n_in / g_step.count0) * h.in_esz, NOUT = (size_t)(h.n_out / g_step.count0) * h.out_esz;
+    if (h.expanded) {
+        if (!g_step.X) setup_xy();
+        if (!h.gather) HIP_OK(hipMemcpyAsync(g_step.din, g_step.X, NIN * h.count, hipMemcpyHostToDevice, s));
+        mlp_forward_dev();
+        if (!h.scatter) {
+            HIP_OK(hipMemcpyAsync(g_step.Y, g_step.dout, NOUT * h.count, hipMemcpyDeviceToHost, s));
+            HIP_OK(hipStreamSynchronize(s));
+        }
+        return;
+    }
+    if (h.step == 1 && h.minc == 1) {
+        HIP_OK(hipMemcpyAsync(g_step.din, in, NIN * h.count, hipMemcpyHostToDevice, s));
+        mlp_forward_dev();
+        HIP_OK(hipMemcpyAsync(out, g_step.dout, NOUT * h.count, hipMemcpyDeviceToHost, s));
+        HIP_OK(hipStreamSynchronize(s));
+        return;
+    }
+    // strided / offset loop: rows minc, minc+|step|, ... of the host arrays (driver/fortis_shim.py:119-121)
+    const long st = h.step < 0 ? -h.step : h.step;
+    HIP_OK(hipMemcpy2DAsync(g_step.din, NIN, (const char*)in + (size_t)(h.minc - 1) * NIN, (size_t)st * NIN, NIN, (size_t)h.count,
+                            hipMemcpyHostToDevice, s));
+    mlp_forward_dev();
+    HIP_OK(hipMemcpy2DAsync((char*)out + (size_t)(h.minc - 1) * NOUT, (size_t)st * NOUT, g_step.dout, NOUT, NOUT, (size_t)h.count,
+                            hipMemcpyDeviceToHost, s));
+    HIP_OK(hipStreamSynchronize(s));
+}
+
+void mlp_forward(void* in, void* out)
+{
+    if (!bound("mlp_forward")) return;
+    const fortis_host_t& h = g_step.h;
+    hipStream_t s = fortis_stream_get();
+    if (h.verdict == FORTIS_VERDICT_BATCHED) {
+        // a call outside the distributed loop: one row through the batched model (driver/fortis_shim.py:122)
+        const size_t NIN = (size_t)(h.n_in / g_step.count0) * h.in_esz, NOUT = (size_t)(h.n_out / g_step.count0) * h.out_esz;
+        HIP_OK(hipMemcpyAsync(g_step.din, in, NIN, hipMemcpyHostToDevice, s));
+        mlp_forward_dev();
+        HIP_OK(hipMemcpyAsync(out, g_step.dout, NOUT, hipMemcpyDeviceToHost, s));
+        HIP_OK(hipStreamSynchronize(s));
+        return;
+    }
+    mlp_upload(in);
+    mlp_forward_dev();
+    mlp_download(out);
+}
+
+void fortis_begin(int count)
+{
+    if (!bound("fortis_begin")) return;
+    fortis_host_t& h = g_step.h;
+    if (h.verdict != FORTIS_VERDICT_BATCHED || count <= 0 || count > g_step.count0) {
+        fprintf(stderr, "fortis_begin: %d rows do not fit the bound step (at most %ld)\n", count, g_step.count0);
+        exit(1);   // the reference stub exits when it cannot specialise (driver/fortis_stub.c:23)
+    }
+    if (count == h.count) return;
+    const long per = g_step.plan->rows0 / g_step.count0;   // rows per cell (enclosing-loop distribution)
+    if (plan_set_rows(g_step.plan, (long)count * per) != 0) {
+        fprintf(stderr, "fortis_begin: the bound model is not row-wise, cannot change its extent\n");
+        exit(1);
+    }
+    h.count = count;
+    drop_graph();
+}
+
+// ---- timing ----------------------------------------------------------------------------------------
+float fortis_time_ms(void (*fn)(void*), void* arg, int iters)
+{
+    hipStream_t s = fortis_stream_get();
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1));
+    HIP_OK(hipEventRecord(e0, s));
+    for (int i = 0; i < iters; i++) fn(arg);
+    HIP_OK(hipEventRecord(e1, s));
+    HIP_OK(hipEventSynchronize(e1));
+    float ms = 0.f;
+    HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+    HIP_OK(hipEventDestroy(e0)); HIP_OK(hipEventDestroy(e1));
+    return ms;
+}
+static void run_plan_cb(void* p) { fortis_plan_run((fortis_plan*)p); }
+float fortis_plan_time_ms(fortis_plan* p, int iters, int use_graph)
+{
+    if (!p || !p->finalized || iters <= 0) return -1.f;
+    hipStream_t s = fortis_stream_get();
+    if (!use_graph) return fortis_time_ms(run_plan_cb, p, iters);
+    hipGraph_t g = nullptr;
+    hipGraphExec_t ge = nullptr;
+    fortis_plan_run(p);   // first pass eager: function attributes and lazy state settle outside capture
+    HIP_OK(hipStreamSynchronize(s));
+    if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) return -1.f;
+    fortis_plan_run(p);
+    if (hipStreamEndCapture(s, &g) != hipSuccess || !g || hipGraphInstantiate(&ge, g, nullptr, nullptr, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        if (g) HIP_OK(hipGraphDestroy(g));
+        return -1.f;
+    }
+    HIP_OK(hipGraphLaunch(ge, s));
+    HIP_OK(hipStreamSynchronize(s));
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1));
+    HIP_OK(hipEventRecord(e0, s));
+    for (int i = 0; i < iters; i++) HIP_OK(hipGraphLaunch(ge, s));
+    HIP_OK(hipEventRecord(e1, s));
+    HIP_OK(hipEventSynchronize(e1));
+    float ms = 0.f;
+    HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+    HIP_OK(hipEventDestroy(e0)); HIP_OK(hipEventDestroy(e1));
+    HIP_OK(hipGraphExecDestroy(ge)); HIP_OK(hipGraphDestroy(g));
+    return ms;
+}
+
+}  // extern "C"

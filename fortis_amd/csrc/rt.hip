@@ -1,0 +1,174 @@
+// Runtime tier: persistent stream, device buffer pool and the memref-expanded GEMM / conv entry
+// points of include/fortis_rt.h.  Replaces runtime/fortis_rt.c of the reference one for one; the
+// vendor-library calls behind those entries are replaced by the hand-written kernels of this
+// library.
+#include "common.h"
+
+// ---- stream (runtime/fortis_rt.c:5-12) ---------------------------------------------------
+static hipStream_t g_stream = nullptr;
+extern "C" {
+int fortis_capturing = 0;
+
+void* mgpuStreamCreate(void)
+{
+    if (!g_stream) {
+        int ndev = 0;
+        if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+            fprintf(stderr, "fortis: no HIP device available; this library has no CPU path\n");
+            abort();
+        }
+        HIP_OK(hipStreamCreate(&g_stream));   // default priority, blocking flag like cudaStreamCreate
+    }
+    return (void*)g_stream;
+}
+void mgpuStreamDestroy(void*) {}
+void mgpuStreamSynchronize(void*) {}
+}
+
+// ---- pool (runtime/fortis_rt.c:14-40) ------------------------------------------------------
+// Same policy as the reference: 256 slots, best fit among released buffers, allocate otherwise,
+// release-all-unused-and-retry once when the device is out of memory.  The allocator behind it is
+// switchable so the policy can be exercised on a machine with no GPU (tests set a host allocator).
+#define FORTIS_POOL 256
+typedef int (*fortis_raw_alloc_fn)(void** p, size_t n);
+typedef void (*fortis_raw_free_fn)(void* p);
+static int dev_alloc(void** p, size_t n) { return hipMalloc(p, n) == hipSuccess ? 0 : -1; }
+static void dev_free(void* p) { HIP_OK(hipFree(p)); }
+static fortis_raw_alloc_fn g_alloc = dev_alloc;
+static fortis_raw_free_fn g_free = dev_free;
+static struct { long n; void* p; int used; } g_pool[FORTIS_POOL];
+
+extern "C" {
+// Test hook: replaces the raw allocator (null restores hipMalloc/hipFree) and empties the pool table.
+void fortis_pool_set_allocator(fortis_raw_alloc_fn a, fortis_raw_free_fn f)
+{
+    g_alloc = a ? a : dev_alloc;
+    g_free = f ? f : dev_free;
+    memset(g_pool, 0, sizeof g_pool);
+}
+// Test hook: number of slots holding a buffer, and how many of them are in use.
+void fortis_pool_stats(int* held, int* used)
+{
+    int h = 0, u = 0;
+    for (int i = 0; i < FORTIS_POOL; i++) if (g_pool[i].p) { h++; u += g_pool[i].used; }
+    if (held) *held = h;
+    if (used) *used = u;
+}
+
+void* fortis_alloc(long n)
+{
+    int best = -1;
+    for (int i = 0; i < FORTIS_POOL; i++)
+        if (g_pool[i].p && !g_pool[i].used && g_pool[i].n >= n && (best < 0 || g_pool[i].n < g_pool[best].n)) best = i;
+    if (best >= 0) { g_pool[best].used = 1; return g_pool[best].p; }
+    for (int attempt = 0; attempt < 2; attempt++) {
+        for (int i = 0; i < FORTIS_POOL; i++)
+            if (!g_pool[i].p) {
+                if (g_alloc(&g_pool[i].p, (size_t)n) == 0) { g_pool[i].n = n; g_pool[i].used = 1; return g_pool[i].p; }
+                g_pool[i].p = nullptr;
+                break;
+            }
+        if (g_alloc == dev_alloc) (void)hipGetLastError();
+        for (int i = 0; i < FORTIS_POOL; i++)
+            if (g_pool[i].p && !g_pool[i].used) { g_free(g_pool[i].p); g_pool[i].p = nullptr; g_pool[i].n = 0; }
+    }
+    fprintf(stderr, "fortis_alloc: device allocation of %ld bytes failed\n", n);
+    return nullptr;
+}
+void fortis_free(void* p)
+{
+    if (!p) return;
+    for (int i = 0; i < FORTIS_POOL; i++) if (g_pool[i].p == p) { g_pool[i].used = 0; return; }
+    g_free(p);
+}
+
+// ---- GEMM entry (runtime/fortis_rt.c:45-75) ------------------------------------------------
+// The reference pre-transposes each weight once so cuBLAS can run N,N.  The MFMA kernel reads
+// W[N][K] rows directly as its B operand (k is the contiguous axis of both operands), so no
+// transpose cache exists here and FORTIS_NO_PRETRANS has nothing to switch.
+void fortis_gemm(float* Aa, float* A, long Ao, long As0, long As1, long At0, long At1,
+                 float* Wa, float* W, long Wo, long Ws0, long Ws1, long Wt0, long Wt1,
+                 float* Ca, float* C, long Co, long Cs0, long Cs1, long Ct0, long Ct1,
+                 long B, long N, long K)
+{
+    (void)Aa; (void)As0; (void)As1; (void)At0; (void)At1; (void)Wa; (void)Ws0; (void)Ws1; (void)Wt0; (void)Wt1;
+    (void)Ca; (void)Cs0; (void)Cs1; (void)Ct0; (void)Ct1;
+    if (fortis_launch_gemm(A + Ao, W + Wo, nullptr, C + Co, B, N, K, FORTIS_ACT_NONE, 0.f, nullptr, 0, fortis_stream_get()) != 0)
+        fprintf(stderr, "fortis_gemm: unsupported shape B%ld N%ld K%ld\n", B, N, K);
+}
+
+// ---- conv entries (runtime/fortis_rt.c:108-156, runtime/fortis_fft.cu:66-79, 131-146) -------
+void fortis_conv2d(float* xa, float* x, long xo, long x0, long x1, long x2, long x3, long xt0, long xt1, long xt2, long xt3,
+                   float* wa, float* w, long wo, long w0, long w1, long w2, long w3, long wt0, long wt1, long wt2, long wt3,
+                   float* ya, float* y, long yo, long y0, long y1, long y2, long y3, long yt0, long yt1, long yt2, long yt3,
+                   long N, long C, long Hin, long Win, long F, long KH, long KW, long Hout, long Wout,
+                   long sh, long sw, long ph, long pw)
+{
+    (void)xa; (void)x0; (void)x1; (void)x2; (void)x3; (void)xt0; (void)xt1; (void)xt2; (void)xt3;
+    (void)wa; (void)w0; (void)w1; (void)w2; (void)w3; (void)wt0; (void)wt1; (void)wt2; (void)wt3;
+    (void)ya; (void)y0; (void)y1; (void)y2; (void)y3; (void)yt0; (void)yt1; (void)yt2; (void)yt3;
+    ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
+    for (long n = 0; n < N; n++) {
+        int rc = fortis_launch_conv2d(x + xo + n * C * Hin * Win, w + wo, y + yo + n * F * Hout * Wout, C, Hin, Win, F,
+                                      KH, KW, Hout, Wout, sh, sw, ph, pw, e, 0, F, fortis_stream_get());
+        if (rc != 0) {
+            fprintf(stderr, "fortis_conv2d: unsupported shape  N%ld C%ld in%ldx%ld F%ld K%ldx%ld out%ldx%ld s%ld,%ld p%ld,%ld\n",
+                    N, C, Hin, Win, F, KH, KW, Hout, Wout, sh, sw, ph, pw);
+            return;
+        }
+    }
+}
+
+static void conv3d_any(const char* who, float* x, long xo, float* w, long wo, float* y, long yo, long N, long C,
+                       long Din, long Hin, long Win, long F, long KD, long KH, long KW, long Dout, long Hout,
+                       long Wout, long sd, long sh, long sw, long pd, long ph, long pw)
+{
+    if (N != 1 || sd != 1 || sh != 1 || sw != 1) { fprintf(stderr, "%s: unsupported shape\n", who); return; }
+    ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
+    if (fortis_launch_conv3d(x + xo, w + wo, y + yo, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, pd, ph, pw, e,
+                             fortis_stream_get()) != 0)
+        fprintf(stderr, "%s: unsupported shape\n", who);
+}
+#define CONV3D_FWD(who)                                                                                             \
+    (void)xa; (void)x0; (void)x1; (void)x2; (void)x3; (void)x4; (void)xt0; (void)xt1; (void)xt2; (void)xt3; (void)xt4; \
+    (void)wa; (void)w0; (void)w1; (void)w2; (void)w3; (void)w4; (void)wt0; (void)wt1; (void)wt2; (void)wt3; (void)wt4; \
+    (void)ya; (void)y0; (void)y1; (void)y2; (void)y3; (void)y4; (void)yt0; (void)yt1; (void)yt2; (void)yt3; (void)yt4; \
+    conv3d_any(who, x, xo, w, wo, y, yo, N, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, sd, sh, sw, pd, ph, pw)
+
+void fortis_conv3d(FORTIS_CONV3D_ARGS) { CONV3D_FWD("fortis_conv3d"); }
+void fortis_conv3d_direct(FORTIS_CONV3D_ARGS) { CONV3D_FWD("fortis_conv3d_direct"); }
+void fortis_conv3d_fft(FORTIS_CONV3D_ARGS)
+{
+    if (pd || ph || pw) { fprintf(stderr, "fortis_conv3d_fft: unsupported shape\n"); return; }
+    CONV3D_FWD("fortis_conv3d_fft");
+}
+
+// ---- host utilities ----------------------------------------------------------------------------
+void fortis_h2d(void* dst, const void* src, long n)
+{
+    hipStream_t s = fortis_stream_get();
+    HIP_OK(hipMemcpyAsync(dst, src, (size_t)n, hipMemcpyHostToDevice, s));
+    HIP_OK(hipStreamSynchronize(s));
+}
+void fortis_d2h(void* dst, const void* src, long n)
+{
+    hipStream_t s = fortis_stream_get();
+    HIP_OK(hipMemcpyAsync(dst, src, (size_t)n, hipMemcpyDeviceToHost, s));
+    HIP_OK(hipStreamSynchronize(s));
+}
+void fortis_d2d(void* dst, const void* src, long n)
+{
+    HIP_OK(hipMemcpyAsync(dst, src, (size_t)n, hipMemcpyDeviceToDevice, fortis_stream_get()));
+}
+void fortis_sync(void) { HIP_OK(hipStreamSynchronize(fortis_stream_get())); }
+int fortis_device_info(char* name, int len, long* total_mem)
+{
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) { (void)hipGetLastError(); return -1; }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return -1;
+    if (name && len > 0) { strncpy(name, prop.gcnArchName, (size_t)len - 1); name[len - 1] = 0; }
+    if (total_mem) *total_mem = (long)prop.totalGlobalMem;
+    return 0;
+}
+}  // extern "C"

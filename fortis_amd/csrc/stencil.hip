@@ -1,0 +1,355 @@
+// Stencil gather / scatter between the host's Fortran arrays and the batch-major model
+// input / output, driven by tables instead of generated source.
+//
+// Reference: the generator driver/fortis_gather_emit.py and its checked-in output
+// mom6_zb/gather.cu (gather kernel :14-49, host wrapper :50-57, scatter kernel :58-81, wrapper
+// :82-91).  Index arithmetic is integer-exact; slot values go through the lifted expressions in
+// explicit round-to-nearest fp32 with no contraction (the reference builds with -fmad=false).
+//
+// Kernel mapping on CDNA4 (differs from the reference's one-thread-per-row store pattern):
+//   gather : thread = row for the loads (consecutive lanes -> consecutive i, coalesced plane
+//            reads), results staged in LDS and written out as one contiguous, fully coalesced
+//            block of 256 x n floats (a row-per-thread store would touch n cache lines per lane).
+//   scatter: thread = cell; Y rows staged through LDS the same way in reverse; plane stores
+//            are coalesced along i.
+#include "stencil_dev.h"
+
+#define ST_THREADS 256
+
+__global__ __launch_bounds__(ST_THREADS) void gather_kernel(const StencilDev* __restrict__ d, PtrTab A,
+                                                            float* __restrict__ X, long rows)
+{
+    extern __shared__ float lds[];
+    const int n = d->nrefs;
+    const int tid = threadIdx.x;
+    const long row0 = (long)blockIdx.x * ST_THREADS, row = row0 + tid;
+    if (row < rows) {
+        const long col = row % d->count;
+        const int kk = (int)(row / d->count);
+        int i, j;
+        st_cell(d, col, i, j);
+        float S[FORTIS_MAX_SCAL], c[FORTIS_MAX_INS];
+        st_cell_values(d, A, i, j, kk, S, c);
+        for (int q = 0; q < n; q++) {
+            float tv = A.p[d->refs[q].array][st_elem(d, d->refs[q], i, j, kk)];
+            lds[tid * n + q] = st_chain(d, tv, S, c);
+        }
+    }
+    __syncthreads();
+    const long lim = (rows - row0 < ST_THREADS ? rows - row0 : ST_THREADS) * n;
+    float* out = X + row0 * n;
+    for (long idx = tid; idx < lim; idx += ST_THREADS) out[idx] = lds[idx];
+}
+
+__global__ __launch_bounds__(ST_THREADS) void scatter_kernel(const StencilDev* __restrict__ d, PtrTabW A,
+                                                             const float* __restrict__ Y, int kk)
+{
+    extern __shared__ float lds[];
+    const int n = d->nrefs;
+    const int tid = threadIdx.x;
+    const long col0 = (long)blockIdx.x * ST_THREADS, col = col0 + tid;
+    const long lim = (d->count - col0 < ST_THREADS ? d->count - col0 : ST_THREADS) * n;
+    const float* in = Y + col0 * n;
+    for (long idx = tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
+    __syncthreads();
+    if (col >= d->count) return;
+    int i, j;
+    st_cell(d, col, i, j);
+    float S[FORTIS_MAX_SCAL], c[FORTIS_MAX_INS];
+    st_cell_values(d, A, i, j, kk, S, c);
+    for (int q = 0; q < n; q++) {
+        const float tv = st_chain(d, lds[tid * n + q], S, c);
+        A.p[d->refs[q].array][st_elem(d, d->refs[q], i, j, kk)] = tv;
+    }
+}
+
+// ---- lowering: straight-line program -> per-cell code + tv chain -----------------------------
+int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
+{
+    memset(out, 0, sizeof *out);
+    if (in->narrays < 1 || in->narrays > FORTIS_MAX_ARRAYS || in->nrefs < 1 || in->nrefs > FORTIS_MAX_REFS ||
+        in->nscal < 0 || in->nscal > FORTIS_MAX_SCAL || in->nins < 0 || in->nins > FORTIS_MAX_INS ||
+        in->nconst < 0 || in->nconst > FORTIS_MAX_CONST || in->count < 1 || in->nk < 1) {
+        fprintf(stderr, "fortis: stencil table out of range\n");
+        return -1;
+    }
+    out->narrays = in->narrays;
+    for (int a = 0; a < in->narrays; a++) out->plane[a] = in->plane[a];
+    out->nrefs = in->nrefs;
+    out->nscal = in->nscal;
+    for (int r = 0; r < in->nrefs; r++) out->refs[r] = in->refs[r];
+    for (int r = 0; r < in->nscal; r++) out->scal[r] = in->scal[r];
+    for (int r = 0; r < in->nrefs + in->nscal; r++) {
+        const fortis_ref_t& f = r < in->nrefs ? in->refs[r] : in->scal[r - in->nrefs];
+        if (f.array < 0 || f.array >= in->narrays) { fprintf(stderr, "fortis: stencil ref names array %d\n", f.array); return -1; }
+    }
+    for (int c = 0; c < in->nconst; c++) out->consts[c] = in->consts[c];
+    out->count = in->count; out->nk = in->nk;
+    out->ilo = in->ilo; out->jlo = in->jlo; out->ni = in->ni > 0 ? in->ni : 1; out->sx = in->sx > 0 ? in->sx : 1;
+    out->cells = nullptr;
+    // dep[n]: instruction n depends on tv; map[n]: its index in the per-cell program otherwise
+    int dep[FORTIS_MAX_INS], map[FORTIS_MAX_INS], last_dep = -1;
+    for (int n = 0; n < in->nins; n++) {
+        const fortis_ins_t& I = in->ins[n];
+        int codes[2] = { I.a, I.b }, isdep[2], lowered[2];
+        for (int s = 0; s < 2; s++) {
+            const int c = codes[s];
+            bool ok = c == 0 || (c >= 1 && c <= in->nscal) || (c >= 16 && c < 16 + in->nconst) || (c >= 32 && c < 32 + n);
+            if (!ok || I.op < 0 || I.op > 3) { fprintf(stderr, "fortis: bad stencil instruction %d\n", n); return -1; }
+            if (c == 0) { isdep[s] = 1; lowered[s] = 0; if (last_dep >= 0) { fprintf(stderr, "fortis: stencil expression re-reads the slot value after transforming it\n"); return -1; } }
+            else if (c >= 32 && dep[c - 32]) { isdep[s] = 1; lowered[s] = 0; if (c - 32 != last_dep) { fprintf(stderr, "fortis: stencil expression is not a single chain on the slot value\n"); return -1; } }
+            else { isdep[s] = 0; lowered[s] = c >= 32 ? 32 + map[c - 32] : c; }
+        }
+        if (isdep[0] && isdep[1]) { fprintf(stderr, "fortis: stencil expression combines the slot value with itself\n"); return -1; }
+        if (isdep[0] || isdep[1]) {
+            dep[n] = 1; map[n] = -1; last_dep = n;
+            CellStep st = { I.op, isdep[0] ? lowered[1] : lowered[0], isdep[0] ? 1 : 0 };
+            out->chain[out->nchain++] = st;
+        } else {
+            dep[n] = 0; map[n] = out->ncell;
+            fortis_ins_t ci = { I.op, lowered[0], lowered[1] };
+            out->cell[out->ncell++] = ci;
+        }
+    }
+    if (in->nins > 0 && last_dep != in->nins - 1 && last_dep >= 0) {
+        fprintf(stderr, "fortis: the last stencil instruction must produce the slot value\n");
+        return -1;
+    }
+    if (in->nins > 0 && last_dep < 0) { fprintf(stderr, "fortis: stencil expressions never use the slot value\n"); return -1; }
+    return 0;
+}
+
+// ---- device copies of tables -----------------------------------------------------------------
+struct BoundStencil {
+    bool ok = false;
+    fortis_stencil_t host;       // as configured (cells pointer not owned)
+    StencilDev low;              // lowered, with device cell list
+    StencilDev* dev = nullptr;   // device copy of `low`
+    int* dcells = nullptr;
+    void* darr[FORTIS_MAX_ARRAYS] = {};       // device planes of the host arrays
+    const void* reg[FORTIS_MAX_ARRAYS] = {};  // last host address seen per array
+    bool written[FORTIS_MAX_ARRAYS] = {};
+    bool init = false;
+};
+static BoundStencil g_gather, g_scatter;
+
+static int upload_table(const fortis_stencil_t* t, StencilDev* low, StencilDev** dev, int** dcells)
+{
+    if (fortis_stencil_lower(t, low) != 0) return -1;
+    if (t->cells) {
+        HIP_OK(hipMalloc((void**)dcells, t->count * sizeof(int)));
+        HIP_OK(hipMemcpy(*dcells, t->cells, t->count * sizeof(int), hipMemcpyHostToDevice));
+        low->cells = *dcells;
+    }
+    HIP_OK(hipMalloc((void**)dev, sizeof(StencilDev)));
+    HIP_OK(hipMemcpy(*dev, low, sizeof(StencilDev), hipMemcpyHostToDevice));
+    return 0;
+}
+
+static void release(BoundStencil& b)
+{
+    if (b.dev) HIP_OK(hipFree(b.dev));
+    if (b.dcells) HIP_OK(hipFree(b.dcells));
+    for (int a = 0; a < FORTIS_MAX_ARRAYS; a++) if (b.darr[a]) HIP_OK(hipFree(b.darr[a]));
+    b = BoundStencil();
+}
+
+static int config(BoundStencil& b, const fortis_stencil_t* t, bool is_scatter)
+{
+    release(b);
+    if (upload_table(t, &b.low, &b.dev, &b.dcells) != 0) return -1;
+    b.host = *t;
+    b.host.cells = nullptr;
+    if (is_scatter) for (int r = 0; r < t->nrefs; r++) b.written[t->refs[r].array] = true;
+    b.ok = true;
+    return 0;
+}
+
+void fortis_stencil_reset_internal()
+{
+    release(g_gather);
+    release(g_scatter);
+}
+
+// cache of device tables for the device-resident API (keyed by table contents)
+struct CacheEnt { fortis_stencil_t key; const int* cells_key; StencilDev* dev; StencilDev low; };
+static CacheEnt g_cache[16];
+static int g_ncache = 0;
+static CacheEnt* cached(const fortis_stencil_t* t)
+{
+    for (int i = 0; i < g_ncache; i++) {
+        fortis_stencil_t a = g_cache[i].key, b = *t;
+        a.cells = b.cells = nullptr;
+        if (!memcmp(&a, &b, sizeof a) && g_cache[i].cells_key == t->cells) return &g_cache[i];
+    }
+    if (g_ncache == 16) { fprintf(stderr, "fortis: stencil table cache full\n"); return nullptr; }
+    CacheEnt* e = &g_cache[g_ncache];
+    int* dc = nullptr;
+    fortis_stencil_t clean;
+    memset(&clean, 0, sizeof clean);   // copy field by field so padding bytes compare equal
+    clean = *t;
+    if (upload_table(t, &e->low, &e->dev, &dc) != 0) return nullptr;
+    e->key = *t;
+    e->cells_key = t->cells;
+    g_ncache++;
+    return e;
+}
+
+static void launch_gather(const StencilDev* dev, const StencilDev& low, const float* const* dA, float* dX, hipStream_t s)
+{
+    PtrTab tab = {};
+    for (int a = 0; a < low.narrays; a++) tab.p[a] = dA[a];
+    const long rows = low.count * low.nk;
+    hipLaunchKernelGGL(gather_kernel, dim3((unsigned)cdiv(rows, ST_THREADS)), dim3(ST_THREADS),
+                       (size_t)ST_THREADS * low.nrefs * sizeof(float), s, dev, tab, dX, rows);
+    HIP_OK(hipGetLastError());
+}
+static void launch_scatter(const StencilDev* dev, const StencilDev& low, float* const* dA, const float* dY, int kk, hipStream_t s)
+{
+    PtrTabW tab = {};
+    for (int a = 0; a < low.narrays; a++) tab.p[a] = dA[a];
+    hipLaunchKernelGGL(scatter_kernel, dim3((unsigned)cdiv(low.count, ST_THREADS)), dim3(ST_THREADS),
+                       (size_t)ST_THREADS * low.nrefs * sizeof(float), s, dev, tab, dY, kk);
+    HIP_OK(hipGetLastError());
+}
+
+void fortis_launch_chain_stencil_dev(const ChainDesc& d, const StencilDev* g_dev, const StencilDev* sc_dev,
+                                     long rows, const float* const* dG, int nG, float* const* dS, int nS,
+                                     float* dY, hipStream_t s);
+// plan.hip: describes the plan as a chain if it is one
+int fortis_plan_as_chain(fortis_plan* p, ChainDesc* out);
+
+extern "C" {
+
+int fortis_gather_config(const fortis_stencil_t* g) { return config(g_gather, g, false); }
+int fortis_scatter_config(const fortis_stencil_t* s) { return config(g_scatter, s, true); }
+
+// A host array whose address changes between calls is a temporary: forget it once and never treat
+// it as program-scope again (driver/fortis_gather_emit.py:41-44).  Host memory is staged with plain
+// stream-ordered copies; existing host memory is never page-locked by this library.
+static void note_host(BoundStencil& b, int a, const void* H)
+{
+    if (b.reg[a] && b.reg[a] != H) b.reg[a] = (const void*)1;
+    else if (!b.reg[a]) b.reg[a] = H;
+}
+
+void fortis_gather_v(const int* a, const void* const* H)
+{
+    BoundStencil& b = g_gather;
+    if (!b.ok) { fprintf(stderr, "fortis_gather: no gather table configured\n"); return; }
+    hipStream_t s = fortis_stream_get();
+    const fortis_stencil_t& t = b.host;
+    const bool kdist = t.nk > 1;
+    if (!b.init) {
+        for (int ai = 0; ai < t.narrays; ai++)
+            HIP_OK(hipMalloc(&b.darr[ai], (size_t)t.plane[ai] * t.nk * sizeof(float)));   // gather.cu:8-11
+        b.init = true;
+    }
+    const float* dptr[FORTIS_MAX_ARRAYS];
+    for (int ai = 0; ai < t.narrays; ai++) {
+        note_host(b, ai, H[ai]);
+        // under loop distribution all nk planes starting at klo; otherwise the plane of the
+        // current enclosing-loop index (gather.cu:52-55; gather_emit.py:66-68)
+        long off = 0;
+        const bool planar3d = t.total[ai] > t.plane[ai];
+        if (planar3d) off = kdist ? (long)(t.klo - 1) * t.plane[ai] : (long)((a ? a[0] : 1) - 1) * t.plane[ai];
+        const long nelem = (kdist && planar3d) ? t.plane[ai] * t.nk : t.plane[ai];
+        HIP_OK(hipMemcpyAsync(b.darr[ai], (const float*)H[ai] + off, nelem * sizeof(float), hipMemcpyHostToDevice, s));
+        dptr[ai] = (const float*)b.darr[ai];
+    }
+    launch_gather(b.dev, b.low, dptr, (float*)fortis_model_input(), s);
+}
+
+void fortis_scatter_v(const int* a, void* const* H)
+{
+    BoundStencil& b = g_scatter;
+    if (!b.ok) { fprintf(stderr, "fortis_scatter: no scatter table configured\n"); return; }
+    hipStream_t s = fortis_stream_get();
+    const fortis_stencil_t& t = b.host;
+    if (!b.init) {
+        for (int ai = 0; ai < t.narrays; ai++) HIP_OK(hipMalloc(&b.darr[ai], (size_t)t.plane[ai] * sizeof(float)));   // gather.cu:60-64
+        b.init = true;
+    }
+    const int k1 = a ? a[0] : 1;   // 1-based enclosing-loop index
+    float* dptr[FORTIS_MAX_ARRAYS];
+    for (int ai = 0; ai < t.narrays; ai++) {
+        note_host(b, ai, H[ai]);
+        dptr[ai] = (float*)b.darr[ai];
+        if (!b.written[ai]) {
+            const long off = t.total[ai] > t.plane[ai] ? (long)(k1 - 1) * t.plane[ai] : 0;
+            HIP_OK(hipMemcpyAsync(b.darr[ai], (const float*)H[ai] + off, t.plane[ai] * sizeof(float), hipMemcpyHostToDevice, s));
+        }
+    }
+    // the device holds ONE plane per array here, so the kernel runs with plane index 0
+    const long yoff = t.nk > 1 ? (long)(k1 - t.klo) * t.count * t.nrefs : 0;   // gather.cu:86
+    launch_scatter(b.dev, b.low, dptr, (const float*)fortis_model_output() + yoff, 0, s);
+    for (int r = 0; r < t.nrefs; r++) {
+        const int ai = t.refs[r].array;
+        const long off = t.total[ai] > t.plane[ai] ? (long)(k1 - 1) * t.plane[ai] : 0;
+        float* hbase = (float*)H[ai] + off;
+        if (t.cells || t.refs[r].si != 1) {
+            // cell list or non-unit inner stride: no rectangle to copy, return the whole plane
+            HIP_OK(hipMemcpyAsync(hbase, b.darr[ai], t.plane[ai] * sizeof(float), hipMemcpyDeviceToHost, s));
+        } else {
+            // visited rectangle, pitch = stride of the j index (gather.cu:87-89; gather_emit.py:88-95)
+            const long rect = t.refs[r].base + (long)t.ilo * t.refs[r].si + (long)t.jlo * t.refs[r].sj;
+            const long pitch = t.refs[r].sj > 0 ? t.refs[r].sj : t.ni;
+            HIP_OK(hipMemcpy2DAsync(hbase + rect, pitch * sizeof(float), (float*)b.darr[ai] + rect, pitch * sizeof(float),
+                                    (size_t)t.ni * sizeof(float), (size_t)(t.nj > 0 ? t.nj : t.count / t.ni),
+                                    hipMemcpyDeviceToHost, s));
+        }
+    }
+    HIP_OK(hipStreamSynchronize(s));
+}
+
+void fortis_gather(const float* H0, const float* H1, const float* H2, const float* H3)
+{
+    const void* H[4] = { H0, H1, H2, H3 };
+    fortis_gather_v(nullptr, H);
+}
+void fortis_scatter(int a0, float* H0, float* H1, float* H2, float* H3, float* H4)
+{
+    void* H[5] = { H0, H1, H2, H3, H4 };
+    fortis_scatter_v(&a0, H);
+}
+
+void fortis_stencil_gather_dev(const fortis_stencil_t* g, const float* const* dA, float* dX)
+{
+    CacheEnt* e = cached(g);
+    if (!e) return;
+    launch_gather(e->dev, e->low, dA, dX, fortis_stream_get());
+}
+void fortis_stencil_scatter_dev(const fortis_stencil_t* sd, float* const* dA, const float* dY, int kk)
+{
+    CacheEnt* e = cached(sd);
+    if (!e) return;
+    launch_scatter(e->dev, e->low, dA, dY, kk, fortis_stream_get());
+}
+
+int fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t* sd, fortis_plan* p,
+                              const float* const* dG, float* const* dS, float* dY)
+{
+    ChainDesc d;
+    if (fortis_plan_as_chain(p, &d) != 0) {
+        fprintf(stderr, "fortis_stencil_step_fused: the plan is not a narrow MLP chain\n");
+        return -1;
+    }
+    if (d.L[0].K != g->nrefs || d.L[d.nlayers - 1].N != sd->nrefs || g->count != sd->count || g->nk != sd->nk) {
+        fprintf(stderr, "fortis_stencil_step_fused: gather/scatter tables do not match the model (%d->%d vs %d->%d)\n",
+                g->nrefs, sd->nrefs, d.L[0].K, d.L[d.nlayers - 1].N);
+        return -1;
+    }
+    // Every written array gets a plane per enclosing-loop iteration on the device, also the ones
+    // that are 2-D on the host (overwritten each iteration there).
+    fortis_stencil_t s2 = *sd;
+    for (int r = 0; r < s2.nrefs; r++)
+        if (!s2.refs[r].planar) { s2.refs[r].planar = 1; s2.plane[s2.refs[r].array] = s2.total[s2.refs[r].array]; }
+    CacheEnt* eg = cached(g);
+    CacheEnt* es = cached(&s2);
+    if (!eg || !es) return -1;
+    fortis_launch_chain_stencil_dev(d, eg->dev, es->dev, g->count * g->nk, dG, g->narrays, dS, sd->narrays, dY,
+                                    fortis_stream_get());
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,214 @@
+/*
+ * fortis_step.h -- host-facing tier of the MI355X backend: the entry points a Fortran/C host
+ * calls by bind(c) name, and the tables that parameterise them.
+ *
+ * In the reference these entries are C/CUDA text generated per build with every size baked in
+ * (driver/fortis_shim.py -> shim.c, driver/fortis_gather_emit.py -> gather.cu) and the model is
+ * MLIR-generated host code (`mlp_kernel` in model.o).  Here the same entry names live in the
+ * library and read their sizes from tables bound once at start-up:
+ *     fortis_plan_*     the model: the op list fortis-fuse would have emitted, with its weights
+ *     fortis_step_bind  the facts of the `fortis.host` attribute (driver/fortis_hostattr.py:11-28)
+ *     fortis_gather_config / fortis_scatter_config   gather.json / scatter.json / loop.json / kdist.json
+ * The per-build generated file shrinks to a table plus one bind call.
+ *
+ * Conventions kept from the reference (driver/fortis_shim.py, mom6_zb/gather.cu): host arrays
+ * belong to the host; device buffers belong to the library for the life of the process; no return
+ * codes on the bind(c) entries, diagnostics on stderr; one host thread, one stream, file-scope
+ * state.  mlp_forward, mlp_download and fortis_scatter return with results visible on the host;
+ * fortis_gather, mlp_forward_dev and the argument-less mlp_forward_batched are asynchronous.
+ * Table-building calls (fortis_plan_*, *_config, fortis_step_bind) return 0 or -1.
+ */
+#ifndef FORTIS_STEP_H
+#define FORTIS_STEP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ================================ model plan ============================================ */
+enum { FORTIS_ACT_NONE = 0, FORTIS_ACT_RELU = 1, FORTIS_ACT_LEAKY = 2 };
+
+typedef struct fortis_plan fortis_plan;
+
+fortis_plan* fortis_plan_create(void);
+void         fortis_plan_destroy(fortis_plan* p);
+/* Declares an activation tensor of `nbytes` bytes; returns its id (>= 0).  Tensors are device
+ * buffers taken from fortis_alloc at finalize. */
+int  fortis_plan_tensor(fortis_plan* p, long nbytes);
+
+/* dst[B][N] = act(src[B][K] . W[N][K]^T + bias[N]).  W, bias are host pointers, copied to the
+ * device at finalize (the role of setup() uploading w<i>, driver/fortis_shim.py:67-72).  bias may
+ * be NULL.  Replaces a fortis_gemm call plus its epilogue kernel (runtime/fortis_rt.c:45-75,
+ * compiler/FortisFuse.cpp:685-692, 721-760) with one fused kernel. */
+int  fortis_plan_linear(fortis_plan* p, int src, int dst, const float* W, const float* bias,
+                        long B, long K, long N, int act, float alpha);
+/* dst[r][c] = divide ? src[r][c] / vec[c] : src[r][c] * vec[c]; the lifted input/output
+ * normalisation chain (mom6_zb/export_zb.py:14; compiler/FortisFuse.cpp:526-573). */
+int  fortis_plan_scale(fortis_plan* p, int src, int dst, const float* vec, long rows, long n, int divide);
+/* dst = src with ReLU applied to the last `tail` of n features of every row: the
+ * `y + mask*(relu(y) - y)` head (benchmarks/climsim/export_wide.py:27-28). */
+int  fortis_plan_mask_relu(fortis_plan* p, int src, int dst, long rows, long n, long tail);
+/* Boundary verdict, pre side: src is the host's own column-major (NI, NK) array of element size
+ * host_esz (4 or 8); dst[i][k] = (float)((src[i + NI*k] - mean[k]) / (vmax[k] - vmin[k])) computed
+ * in the host type.  mean/vmax/vmin are host vectors of that type (any may be NULL: mean 0,
+ * range 1).  trt_backend/e3sm_boundary.cu:9-14; driver/fortis_emit2d.py:20-36. */
+int  fortis_plan_boundary_pre(fortis_plan* p, int src, int dst, long NI, long NK, const void* mean,
+                              const void* vmax, const void* vmin, int host_esz);
+/* Post side: dst[i + NI*k] = (H)src[i][k] / scale[k].  trt_backend/e3sm_boundary.cu:15-20. */
+int  fortis_plan_boundary_post(fortis_plan* p, int src, int dst, long NI, long NK, const void* scale,
+                               int host_esz);
+
+/* conv2d NCHW (N = 1): dst[coff .. coff+F) of a tensor holding ctot channels (so that a skip
+ * concatenation is a channel-offset write, compiler/FortisFuse.cpp:547-551) =
+ * act(bn(conv(src, W) + bias)).  W [F][C][KH][KW]; bias, and the four BatchNorm-eval vectors
+ * (gamma, beta, mean, var; all or none) are host pointers of length F or NULL.  Replaces
+ * fortis_conv2d + epilogue kernel (runtime/fortis_rt.c:108-127; FortisFuse.cpp:688-692). */
+int  fortis_plan_conv2d(fortis_plan* p, int src, int dst, const float* W, const float* bias,
+                        const float* bn_gamma, const float* bn_beta, const float* bn_mean,
+                        const float* bn_var, float bn_eps, long C, long H, long Wd, long F, long KH,
+                        long KW, long stride, long pad, int act, float alpha, long coff, long ctot);
+/* Transposed conv2d, weights [C][F][KH][KW] (PyTorch layout), output size
+ * (H-1)*stride - 2*pad + KH + output_padding.  Same epilogue and concat arguments. */
+int  fortis_plan_convt2d(fortis_plan* p, int src, int dst, const float* W, const float* bias,
+                         long C, long H, long Wd, long F, long KH, long KW, long stride, long pad,
+                         long output_padding, int act, float alpha, long coff, long ctot);
+/* k x k max pooling, stride k (compiler/FortisFuse.cpp:667-672: non-additive reduction). */
+int  fortis_plan_maxpool2d(fortis_plan* p, int src, int dst, long C, long H, long Wd, long k);
+/* Nearest-neighbour upsample by s over the trailing nd (2 or 3) spatial dims; D = 1 for nd = 2. */
+int  fortis_plan_upsample(fortis_plan* p, int src, int dst, long C, long D, long H, long Wd, long s, int nd);
+/* Copy C channels of S elements into dst at channel offset coff of ctot (concat by copy). */
+int  fortis_plan_concat_copy(fortis_plan* p, int src, int dst, long C, long S, long coff, long ctot);
+/* conv3d NCDHW, N = 1, stride 1: dst = act(conv(src, W) + bias) [+ res].  res is a tensor id
+ * added after the activation (residual skip), or -1.  W [F][C][KD][KH][KW].  Replaces
+ * fortis_conv3d(_direct) + epilogue (runtime/fortis_fft.cu:131-201). */
+int  fortis_plan_conv3d(fortis_plan* p, int src, int dst, int res, const float* W, const float* bias,
+                        long C, long D, long H, long Wd, long F, long K, long pad, int act, float alpha);
+/* Layout permutes around a channels-last host tensor: to_channels_first != 0: [S][C] -> [C][S];
+ * otherwise [C][S] -> [S][C].  S = product of the spatial dims. */
+int  fortis_plan_permute(fortis_plan* p, int src, int dst, long C, long S, int to_channels_first);
+
+/* Fixes the plan: allocates tensors, uploads weights, folds BatchNorm, fuses neighbouring ops
+ * into single kernels.  in_tensor / out_tensor are what fortis_model_input/output return. */
+int   fortis_plan_finalize(fortis_plan* p, int in_tensor, int out_tensor);
+/* Enqueues one forward pass on the persistent stream (the role of the generated
+ * mlp_kernel(...) host function, driver/fortis_shim.py:62-63, 86). */
+void  fortis_plan_run(fortis_plan* p);
+void* fortis_plan_tensor_ptr(fortis_plan* p, int tensor);
+int   fortis_plan_num_kernels(fortis_plan* p);   /* launches per forward pass after fusion */
+
+/* ================================ step binding ========================================== */
+enum { FORTIS_VERDICT_WHOLE = 0, FORTIS_VERDICT_BATCHED = 1, FORTIS_VERDICT_BOUNDARY = 2 };
+
+/* The facts the reference bakes into shim.c from the `fortis.host` attribute
+ * (driver/fortis_shim.py:9-38, 94-133). */
+typedef struct {
+    long n_in, n_out;     /* elements of the whole model input / output */
+    int  in_esz, out_esz; /* host element size: 4, or 8 under a boundary verdict on f64 arrays */
+    int  verdict;         /* FORTIS_VERDICT_* */
+    int  expanded;        /* batched: call temporaries expanded across the batch (pack/unpack form) */
+    long count;           /* batched: rows per batched call */
+    long lo, step, minc;  /* batched: loop start, stride, smallest visited column (1-based) */
+    int  graph;           /* the fortis.graph attribute; FORTIS_GRAPH in the environment also enables it */
+    int  gather, scatter; /* the build-time FORTIS_GATHER / FORTIS_SCATTER switches */
+} fortis_host_t;
+
+int  fortis_step_bind(fortis_plan* p, const fortis_host_t* host);
+/* Forgets the bound step, the stencil tables and the graph (tests; a host never calls it). */
+void fortis_step_reset(void);
+int  fortis_step_graph_active(void);    /* 1 once a captured graph is being replayed */
+
+/* ---- entry points, names and behaviour of the generated shim --------------------------- */
+void  mlp_upload(void* in);                       /* driver/fortis_shim.py:93 */
+void  mlp_forward_dev(void);                      /* :82-90  capture on call #2, replay after, eager fallback */
+void  mlp_download(void* out);                    /* :92 */
+void  mlp_forward(void* in, void* out);           /* :122 (single row, batched build) / :132-133 (whole array) */
+/* One symbol, two reference forms: the expanded form takes no arguments (:113-115) and ignores
+ * what it is passed; the slice form takes the host's whole in/out arrays (:117-121). */
+void  mlp_forward_batched(void* in, void* out);
+void  fortis_pack(void* row, int col);            /* :105  col is 0-based */
+void  fortis_unpack(void* row, int col);          /* :106 */
+void* fortis_model_input(void);                   /* :109 */
+void* fortis_model_output(void);                  /* :110 */
+/* Run-time extents: re-specialises the bound step for `count` rows per call; no JIT, the
+ * kernels take the row count at run time.                  driver/fortis_stub.c:12-31 */
+void  fortis_begin(int count);
+
+/* ================================ stencil gather / scatter ============================== */
+/* One element of one host array relative to cell (i, j) (1-based Fortran indices) and the
+ * enclosing-loop plane kk (0-based): elem = base + i*si + j*sj + (planar ? kk*plane[array] : 0).
+ * For A(i+di, j+dj, k) on a column-major (sx, sy, nk) array: si = 1, sj = sx,
+ * base = (di-1) + (dj-1)*sx.  This is what driver/fortis_gather_emit.py:27-33 (elem, plane_off)
+ * prints into the generated kernel. */
+typedef struct { int array; int planar; long base, si, sj; } fortis_ref_t;
+
+/* Lifted expressions as straight-line fp32 code: r[n] = operand(a) op operand(b).
+ * operand: 0 = tv (the slot value), 1..8 = scalar S0..S7, 16+n = consts[n], 32+n = r[n].
+ * op: 0 add, 1 sub, 2 mul, 3 div.  The last result replaces tv.  Each op is one IEEE fp32
+ * operation, never fused (the reference compiles gather.cu with -fmad=false).  tv may enter
+ * an instruction only as the running value of one chain (tv op c, c op tv). */
+typedef struct { int op, a, b; } fortis_ins_t;
+
+#define FORTIS_MAX_ARRAYS 8
+#define FORTIS_MAX_REFS 32
+#define FORTIS_MAX_SCAL 8
+#define FORTIS_MAX_INS 12
+#define FORTIS_MAX_CONST 8
+
+typedef struct {
+    int  narrays;
+    long total[FORTIS_MAX_ARRAYS];     /* elements of each host array */
+    long plane[FORTIS_MAX_ARRAYS];     /* elements per enclosing-loop iteration (== total for 2-D arrays) */
+    int  nrefs;                        /* gather: feature slots in order; scatter: one store per output slot */
+    fortis_ref_t refs[FORTIS_MAX_REFS];
+    int  nscal;
+    fortis_ref_t scal[FORTIS_MAX_SCAL];
+    int  nins;
+    fortis_ins_t ins[FORTIS_MAX_INS];
+    int  nconst;
+    float consts[FORTIS_MAX_CONST];
+    long count;                        /* cells per enclosing-loop iteration */
+    int  nk, klo;                      /* enclosing-loop distribution: trip count and first index (nk = 1: none) */
+    int  nargs;                        /* leading int arguments of the generated entry (enclosing-loop variables) */
+    int  ilo, jlo, ni, nj;             /* visited rectangle (1-based lower bounds) */
+    int  sx;                           /* leading dimension of the cell plane, for the cell list */
+    const int* cells;                  /* optional host list of `count` 0-based cell indices (i-1)+(j-1)*sx;
+                                          NULL = the rectangle.  Copied at config. */
+} fortis_stencil_t;
+
+int  fortis_gather_config(const fortis_stencil_t* g);
+int  fortis_scatter_config(const fortis_stencil_t* s);
+/* Generic forms of the generated entries.  a: the enclosing-loop index arguments (1-based
+ * Fortran values; none for the gather under loop distribution); H: the host arrays in
+ * descriptor order.  fortis_gather_v: async H2D of the planes it needs, then the gather kernel
+ * writing the model input (mom6_zb/gather.cu:50-57).  fortis_scatter_v: H2D of the arrays it
+ * only reads, scatter kernel on the model output of iteration a[0], device->host copy of the
+ * visited rectangle of every written array, stream sync (mom6_zb/gather.cu:82-91). */
+void fortis_gather_v(const int* a, const void* const* H);
+void fortis_scatter_v(const int* a, void* const* H);
+/* The checked-in ZB instance's exact signatures (mom6_zb/gather.cu:50, :82). */
+void fortis_gather(const float* H0, const float* H1, const float* H2, const float* H3);
+void fortis_scatter(int a0, float* H0, float* H1, float* H2, float* H3, float* H4);
+
+/* Device-resident forms (arrays already in HBM; nothing is copied).  dA: device pointers in
+ * descriptor order.  Asynchronous on the persistent stream. */
+void fortis_stencil_gather_dev(const fortis_stencil_t* g, const float* const* dA, float* dX);
+void fortis_stencil_scatter_dev(const fortis_stencil_t* s, float* const* dA, const float* dY, int kk);
+/* The whole lifted step in ONE kernel: gather (g) -> MLP chain (plan p, every op a linear or a
+ * feature scale) -> scatter (s) for all nk iterations at once.  Arrays the scatter writes need a
+ * plane per iteration on the device: an array that is 2-D on the host (written once per
+ * iteration, like Txy_h) is given nk planes of `plane` elements.  dY (optional) also receives the
+ * raw model output.  Returns -1 if the plan is not such a chain or is too wide for the kernel. */
+int  fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t* s, fortis_plan* p,
+                               const float* const* dG, float* const* dS, float* dY);
+
+/* ================================ timing helper ========================================= */
+/* Runs fn(arg) `iters` times on the persistent stream between two HIP events on that stream and
+ * returns the elapsed milliseconds (the benchmark's per-kernel clock). */
+float fortis_time_ms(void (*fn)(void*), void* arg, int iters);
+/* Same clock around `iters` enqueues of a plan / the fused stencil step / a graph replay. */
+float fortis_plan_time_ms(fortis_plan* p, int iters, int use_graph);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
