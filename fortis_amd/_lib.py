@@ -49,7 +49,8 @@ PROTOTYPES = {
     "fortis_conv3d_direct": (None, ([vp, vp] + [l] * 11) * 3 + [l] * 18),
     "fortis_conv3d_fft": (None, ([vp, vp] + [l] * 11) * 3 + [l] * 18),
     "fortis_h2d": (None, [vp, vp, l]), "fortis_d2h": (None, [vp, vp, l]), "fortis_d2d": (None, [vp, vp, l]),
-    "fortis_sync": (None, []), "fortis_device_info": (i, [C.c_char_p, i, C.POINTER(l)]),
+    "fortis_sync": (None, []), "fortis_pool_stats": (None, [C.POINTER(i), C.POINTER(i)]),
+    "fortis_pool_set_allocator": (None, [vp, vp]), "fortis_device_info": (i, [C.c_char_p, i, C.POINTER(l)]),
     # fortis_step.h: plan
     "fortis_plan_create": (vp, []), "fortis_plan_destroy": (None, [vp]), "fortis_plan_tensor": (i, [vp, l]),
     "fortis_plan_linear": (i, [vp, i, i, vp, vp, l, l, l, i, f]),
@@ -74,6 +75,7 @@ PROTOTYPES = {
     "fortis_pack": (None, [vp, i]), "fortis_unpack": (None, [vp, i]),
     "fortis_model_input": (vp, []), "fortis_model_output": (vp, []), "fortis_begin": (None, [i]),
     # stencil
+    "fortis_stencil_check": (i, [C.POINTER(Stencil)]),
     "fortis_gather_config": (i, [C.POINTER(Stencil)]), "fortis_scatter_config": (i, [C.POINTER(Stencil)]),
     "fortis_gather_v": (None, [C.POINTER(i), C.POINTER(vp)]), "fortis_scatter_v": (None, [C.POINTER(i), C.POINTER(vp)]),
     "fortis_gather": (None, [vp, vp, vp, vp]), "fortis_scatter": (None, [i, vp, vp, vp, vp, vp]),

@@ -185,9 +185,6 @@ static CacheEnt* cached(const fortis_stencil_t* t)
     if (g_ncache == 16) { fprintf(stderr, "fortis: stencil table cache full\n"); return nullptr; }
     CacheEnt* e = &g_cache[g_ncache];
     int* dc = nullptr;
-    fortis_stencil_t clean;
-    memset(&clean, 0, sizeof clean);   // copy field by field so padding bytes compare equal
-    clean = *t;
     if (upload_table(t, &e->low, &e->dev, &dc) != 0) return nullptr;
     e->key = *t;
     e->cells_key = t->cells;
@@ -221,6 +218,11 @@ int fortis_plan_as_chain(fortis_plan* p, ChainDesc* out);
 
 extern "C" {
 
+int fortis_stencil_check(const fortis_stencil_t* t)
+{
+    StencilDev tmp;
+    return t ? fortis_stencil_lower(t, &tmp) : -1;
+}
 int fortis_gather_config(const fortis_stencil_t* g) { return config(g_gather, g, false); }
 int fortis_scatter_config(const fortis_stencil_t* s) { return config(g_scatter, s, true); }
 

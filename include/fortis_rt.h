@@ -37,6 +37,12 @@ void* fortis_alloc(long nbytes);
  * freed for real.                                                   runtime/fortis_rt.c:37-40 */
 void  fortis_free(void* p);
 
+/* Test hooks, no reference counterpart: swap the raw allocator under the pool (NULL, NULL restores
+ * the device allocator) and empty the pool table; count held / in-use slots.  They let the pool
+ * policy be exercised on a machine without a GPU. */
+void  fortis_pool_set_allocator(int (*raw_alloc)(void** p, unsigned long nbytes), void (*raw_free)(void* p));
+void  fortis_pool_stats(int* held, int* used);
+
 /* ---- GEMM -------------------------------------------------------------------------------- */
 /* C[B][N] = A[B][K] . W[N][K]^T, fp32, beta = 0.                     runtime/fortis_rt.c:45-75 */
 void fortis_gemm(float* Aa, float* A, long Ao, long As0, long As1, long At0, long At1,

@@ -175,6 +175,9 @@ typedef struct {
                                           NULL = the rectangle.  Copied at config. */
 } fortis_stencil_t;
 
+/* Validates a table without touching the GPU (ranges, and that the expressions form one chain on
+ * the slot value); what *_config and the device-resident forms check first. */
+int  fortis_stencil_check(const fortis_stencil_t* t);
 int  fortis_gather_config(const fortis_stencil_t* g);
 int  fortis_scatter_config(const fortis_stencil_t* s);
 /* Generic forms of the generated entries.  a: the enclosing-loop index arguments (1-based

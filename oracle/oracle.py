@@ -210,7 +210,7 @@ def mlp_native(Ws, bs, X, in_norms=None, out_norms=None):
     return Y
 
 
-ACT = {"none": 0, "relu": 1, "leaky": 2}
+ACT = {None: 0, "none": 0, "relu": 1, "leaky": 2}
 
 
 def mlp_f64(Ws, bs, acts, X, alphas=None, in_norms=None, out_norms=None, mask_tail=0):
@@ -219,7 +219,7 @@ def mlp_f64(Ws, bs, acts, X, alphas=None, in_norms=None, out_norms=None, mask_ta
     X, xp = _f(X)
     rows = X.shape[0]
     Y = np.empty((rows, widths[-1]), dtype=np.float32)
-    act = (C.c_int * len(Ws))(*[ACT[a] if isinstance(a, str) else a for a in acts])
+    act = (C.c_int * len(Ws))(*[a if isinstance(a, int) else ACT[a] for a in acts])
     al = np.ascontiguousarray(alphas if alphas is not None else np.zeros(len(Ws)), dtype=np.float32)
     inn = _f(in_norms) if in_norms is not None else (None, None)
     outn = _f(out_norms) if out_norms is not None else (None, None)

@@ -1,0 +1,40 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an MI355X; run with -m gpu on the GPU box")
+
+
+@pytest.fixture(scope="session")
+def golden():
+    return GOLDEN
+
+
+@pytest.fixture(scope="session")
+def L():
+    """The product library, loaded once.  GPU tests fail (not skip) if it is missing."""
+    import fortis_amd
+    return fortis_amd.load()
+
+
+@pytest.fixture(scope="session")
+def gpu(L):
+    import ctypes as C
+    name = C.create_string_buffer(64)
+    assert L.fortis_device_info(name, 64, None) == 0, "no GPU visible to libfortis_rt"
+    return name.value.decode()
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    # names the case before it runs, flushed, so a run that dies on the GPU still says where
+    print(f"\n[case] {request.node.nodeid}", flush=True)
+    yield

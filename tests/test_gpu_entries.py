@@ -1,0 +1,200 @@
+"""The host-facing entry points (the generated shim's names, driver/fortis_shim.py:54-135, and the
+generated gather/scatter wrappers, mom6_zb/gather.cu:50-57, 82-91) driven the way a Fortran host
+drives them."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+from fortis_amd import configs, plan as P, stencil as S, step as ST
+from oracle import oracle as O
+from util import TOL, bits_equal, maxrel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _fresh_step(L):
+    yield
+    ST.reset()
+
+
+def _toy(rows=256):
+    case = configs.toy_mlp(rows)
+    return case, configs.mlp_case_plan(case), O.mlp_f64(case["Ws"], case["bs"], case["acts"], case["X"])
+
+
+def test_whole_array_call_and_resident_entries(L, gpu):
+    """mlp_forward(x, y) and the upload / forward_dev / download triple of benchmarks/toy/bench_dev.f90:4-11."""
+    case, plan, ref = _toy()
+    ST.bind(plan, case["X"].size, ref.size)
+    y = np.empty_like(ref)
+    ST.mlp_forward(case["X"], y)
+    assert maxrel(y, ref) < TOL
+    y2 = np.zeros_like(ref)
+    ST.mlp_upload(case["X"])
+    for _ in range(3):
+        ST.mlp_forward_dev()
+    ST.mlp_download(y2)
+    assert bits_equal(y, y2)
+
+
+def test_graph_capture_on_second_call_and_replay(L, gpu):
+    """fortis.graph set: call 1 eager, call 2 captures and launches, later calls replay
+    (driver/fortis_shim.py:82-90).  Every replay must equal the eager result, with eager work and
+    synchronisations in between."""
+    case, plan, ref = _toy()
+    ST.bind(plan, case["X"].size, ref.size, graph=True)
+    outs = []
+    rng = np.random.default_rng(3)
+    for n in range(6):
+        x = case["X"] if n in (0, 5) else rng.uniform(-1, 1, case["X"].shape).astype(np.float32)
+        y = np.empty_like(ref)
+        ST.mlp_forward(x, y)
+        assert ST.graph_active() == (n >= 1)
+        assert maxrel(y, O.mlp_f64(case["Ws"], case["bs"], case["acts"], x)) < TOL
+        outs.append(y)
+        plan.run()                                   # eager work between replays
+        L.fortis_sync()
+    assert bits_equal(outs[0], outs[5])              # eager call == replayed call on the same input
+
+
+def test_graph_env_switch(L, gpu, monkeypatch):
+    case, plan, ref = _toy()
+    ST.bind(plan, case["X"].size, ref.size, graph=False)
+    y = np.empty_like(ref)
+    ST.mlp_forward(case["X"], y)
+    ST.mlp_forward(case["X"], y)
+    assert not ST.graph_active()
+    ST.reset()
+    monkeypatch.setenv("FORTIS_GRAPH", "1")
+    ST.bind(plan, case["X"].size, ref.size, graph=False)
+    ST.mlp_forward(case["X"], y)
+    ST.mlp_forward(case["X"], y)
+    assert ST.graph_active() and maxrel(y, ref) < TOL
+
+
+def test_pack_batched_unpack(L, gpu):
+    """Fissioned per-column loop: fortis_pack x B -> mlp_forward_batched() -> fortis_unpack x B
+    (driver/fortis_shim.py:99-115)."""
+    case, plan, ref = _toy(200)
+    ST.bind(plan, case["X"].size, ref.size, verdict="batched", expanded=True, count=200)
+    for col in range(200):
+        ST.fortis_pack(case["X"][col], col)
+    ST.mlp_forward_batched()
+    y = np.empty_like(ref)
+    row = np.empty(32, np.float32)
+    for col in range(200):
+        ST.fortis_unpack(row, col)
+        y[col] = row
+    assert maxrel(y, ref) < TOL
+    # a per-row call outside the loop goes through the same batched model (fortis_shim.py:122)
+    ST.mlp_forward(case["X"][7], row)
+    assert maxrel(row, ref[7]) < TOL * np.abs(ref).max() / np.abs(ref[7]).max()
+
+
+def test_batched_slice_forms(L, gpu):
+    """Slice form on the host's whole arrays: unit stride (fortis_shim.py:117-118) and the strided
+    upload with step 2, first visited column 3 (fortis_shim.py:119-121)."""
+    case, plan, ref = _toy(100)
+    ST.bind(plan, case["X"].size, ref.size, verdict="batched", count=100, lo=1, step=1, minc=1)
+    y = np.empty_like(ref)
+    ST.mlp_forward_batched(case["X"], y)
+    assert maxrel(y, ref) < TOL
+    ST.reset()
+    big = np.random.default_rng(9).uniform(-1, 1, (210, 64)).astype(np.float32)
+    out = np.zeros((210, 32), np.float32)
+    ST.bind(plan, 100 * 64, 100 * 32, verdict="batched", count=100, lo=3, step=2, minc=3)
+    ST.mlp_forward_batched(big, out)
+    rows = np.arange(100) * 2 + 2                                  # 0-based rows 2, 4, ...
+    full = O.mlp_f64(case["Ws"], case["bs"], case["acts"], big[rows])
+    assert maxrel(out[rows], full) < TOL
+    untouched = np.setdiff1d(np.arange(210), rows)
+    assert not out[untouched].any()
+
+
+def test_boundary_verdict_f64_host_arrays(L, gpu):
+    """Boundary verdict: mlp_forward takes the host's own f64 column-major arrays (benchmarks/cam host,
+    driver/fortis_emit2d.py:20-52; trt_backend/e3sm_boundary.cu)."""
+    rng = np.random.default_rng(4)
+    NI, NIN, NOUT = 384, 124, 128
+    Ws = [(rng.standard_normal((128, NIN)) / 11).astype(np.float32), (rng.standard_normal((NOUT, 128)) / 11).astype(np.float32)]
+    bs = [rng.standard_normal(128).astype(np.float32), rng.standard_normal(NOUT).astype(np.float32)]
+    A = np.asfortranarray(rng.standard_normal((NI, NIN)))
+    mean, vmax, vmin, scale = rng.standard_normal(NIN), rng.uniform(2, 3, NIN), rng.uniform(0, 1, NIN), rng.uniform(0.5, 2, NOUT)
+    p = P.Plan()
+    t0, t1, t2, t3, t4 = p.tensor(NI * NIN, 8), p.tensor(NI * NIN), p.tensor(NI * 128), p.tensor(NI * NOUT), p.tensor(NI * NOUT, 8)
+    p.boundary_pre(t0, t1, NI, NIN, mean, vmax, vmin, np.float64)
+    p.linear(t1, t2, Ws[0], bs[0], NI, "leaky", 0.15)
+    p.linear(t2, t3, Ws[1], bs[1], NI, None)
+    p.boundary_post(t3, t4, NI, NOUT, scale, np.float64)
+    p.finalize(t0, t4)
+    assert p.num_kernels == 3                                       # pre, fused 2-layer chain, post
+    ST.bind(p, NI * NIN, NI * NOUT, verdict="boundary", in_dtype=np.float64, out_dtype=np.float64)
+    B = np.empty((NI, NOUT), np.float64, order="F")
+    ST.mlp_forward(A, B)
+    X = O.boundary_pre(A, mean, vmax, vmin)
+    ref = O.boundary_post(O.mlp_f64(Ws, bs, ["leaky", "none"], X, alphas=[0.15, 0]), scale, np.float64)
+    assert maxrel(B, ref) < TOL
+
+
+def test_run_time_extents(L, gpu):
+    """fortis_begin(count) (driver/fortis_stub.c:12-31): the step bound for 200 rows serves 120."""
+    case, plan, ref = _toy(200)
+    ST.bind(plan, case["X"].size, ref.size, verdict="batched", expanded=True, count=200)
+    ST.fortis_begin(120)
+    for col in range(120):
+        ST.fortis_pack(case["X"][col], col)
+    ST.mlp_forward_batched()
+    row = np.empty(32, np.float32)
+    for col in (0, 57, 119):
+        ST.fortis_unpack(row, col)
+        assert maxrel(row, ref[col]) < 5 * TOL
+
+
+def _corner_interp(Txy_h, maskBu, sx=68, sy=78):
+    """Txy(I,J) = 0.25*((Txy_h(i+1,j+1)+Txy_h(i,j)) + (Txy_h(i+1,j)+Txy_h(i,j+1))) * mask2dBu over
+    J=3..75, I=3..65 (mom6_zb/zb_host.f90:102-105), fp32 in the host's operation order."""
+    h, m = Txy_h.reshape(sy, sx), maskBu.reshape(sy, sx)
+    out = np.zeros((sy, sx), np.float32)
+    J, I = slice(2, 75), slice(2, 65)
+    J1, I1 = slice(3, 76), slice(3, 66)
+    out[J, I] = np.float32(0.25) * ((h[J1, I1] + h[J, I]) + (h[J, I1] + h[J1, I])) * m[J, I]
+    return out
+
+
+def test_zb_host_step_through_gather_batched_scatter(L, gpu, golden):
+    """The fissioned ZB host's step (mom6_zb/host_fissioned.fir:732-740): fortis_gather(4 arrays) ->
+    mlp_forward_batched() -> do k: fortis_scatter(k, 5 arrays) + host corner interpolation; results
+    against the fixture written by the reference's own CPU build."""
+    gt, st, gd, sd, lp, kd = S.load_tables(*[os.path.join(golden, f"zb_{n}.json") for n in ("gather", "scatter", "loop", "kdist")])
+    W = np.load(os.path.join(golden, "zb_nn.npz"))
+    G = np.load(os.path.join(golden, "zb_native_golden.npz"))
+    F = O.zb_fields()
+    Pp = O.zb_prep(F)
+    plan = P.mlp_plan([W["A0"], W["A1"]], [W["b0"], W["b1"]], ["relu", None], 71040, in_norms=W["in_norms"], out_norms=W["out_norms"])
+    ST.bind(plan, 71040 * 27, 71040 * 3, verdict="batched", expanded=True, count=71040, gather=True, scatter=True, graph=True)
+    ST.gather_config(gt)
+    ST.scatter_config(st)
+    n3 = 68 * 78 * 15
+    for step in range(3):                                            # step 2 captures the graph, step 3 replays
+        Txy_h, Txx, Tyy, Txy = np.zeros(68 * 78, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)
+        L.fortis_gather(*[a.ctypes.data for a in (Pp["sh_xy_h"], F["sh_xx"], Pp["vort_xy_h"], Pp["norm_h"])])
+        ST.mlp_forward_batched()
+        for k in range(1, 16):
+            L.fortis_scatter(k, *[a.ctypes.data for a in (Pp["norm_h"], F["kappa_h"], Txy_h, Txx, Tyy)])
+            Txy.reshape(15, 78, 68)[k - 1] = _corner_interp(Txy_h, F["mask2dBu"])
+        lay = G["layers"] - 1
+        assert maxrel(Txx.reshape(15, 78, 68)[lay], G["Txx"]) < TOL
+        assert maxrel(Tyy.reshape(15, 78, 68)[lay], G["Tyy"]) < TOL
+        assert maxrel(Txy.reshape(15, 78, 68)[lay], G["Txy"]) < TOL
+        for n, a in enumerate((Txx, Tyy, Txy)):
+            assert abs(a.astype(np.float64).sum() - G["checksum"][n]) < 1e-5 * np.abs(a).sum()
+        # cells outside the visited rectangle are never written
+        assert not Txx.reshape(15, 78, 68)[:, :2].any() and not Txx.reshape(15, 78, 68)[:, :, 66:].any()
+    assert ST.graph_active()
+    # the gather wrote the model input exactly as the oracle's gather does
+    X = np.empty((71040, 27), np.float32)
+    L.fortis_d2h(X.ctypes.data, L.fortis_model_input(), X.nbytes)
+    assert bits_equal(X, O.stencil_gather(gd, [Pp["sh_xy_h"], F["sh_xx"], Pp["vort_xy_h"], Pp["norm_h"]], 4736, 15, 3, 3, 64))

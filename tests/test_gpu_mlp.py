@@ -1,0 +1,152 @@
+"""Column MLPs on the GPU through the C ABI: LDS-resident fused chain (narrow networks), MFMA
+GEMM + fused epilogue (wide networks), the memref-expanded fortis_gemm entry, boundary pre/post."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+from fortis_amd import configs, plan as P
+from oracle import oracle as O
+from util import TOL, DevBuf, maxrel
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config1_toy_mlp(L, gpu):
+    case = configs.toy_mlp()
+    plan = configs.mlp_case_plan(case)
+    assert plan.num_kernels == 1                     # whole 64-256-256-32 stack in one kernel
+    Y = plan.forward(case["X"], (1024, 32))
+    ref = O.mlp_f64(case["Ws"], case["bs"], case["acts"], case["X"])
+    assert maxrel(Y, ref) < TOL
+    assert abs(float(Y.astype(np.float64).sum()) - float(ref.astype(np.float64).sum())) < 1e-5 * np.abs(ref).sum()
+    plan.close()
+
+
+def test_reference_toy_model_readme_stamp(L, gpu):
+    """The reference's own toy: batch 1, Linear(1024,256) ReLU Linear(256,1024), seed 42, z-scored ramp;
+    checksum stamp 7.775037 (README.md:25, frontend/export_mlp.py, benchmarks/toy/bench_fortis.f90)."""
+    import torch
+    torch.manual_seed(42)
+    net = torch.nn.Sequential(torch.nn.Linear(1024, 256), torch.nn.ReLU(), torch.nn.Linear(256, 1024)).eval()
+    x = torch.arange(1, 1025, dtype=torch.float32) / 1024
+    x = ((x - x.mean()) / x.std(unbiased=False)).numpy()[None]
+    Ws = [net[0].weight.detach().numpy(), net[2].weight.detach().numpy()]
+    bs = [net[0].bias.detach().numpy(), net[2].bias.detach().numpy()]
+    plan = P.mlp_plan(Ws, bs, ["relu", None], 1)
+    y = plan.forward(x, (1, 1024))
+    assert abs(float(y.astype(np.float64).sum()) - 7.775037) / 7.775037 < 1e-5
+    assert maxrel(y, O.mlp_f64(Ws, bs, ["relu", "none"], x)) < TOL
+    plan.close()
+
+
+def test_zb_known_answer_vector(L, gpu, golden):
+    W = np.load(os.path.join(golden, "zb_nn.npz"))
+    plan = P.mlp_plan([W["A0"], W["A1"]], [W["b0"], W["b1"]], ["relu", None], 100, in_norms=W["in_norms"], out_norms=W["out_norms"])
+    y = plan.forward(np.tile(W["x_test"], (100, 1)), (100, 3))
+    assert maxrel(y[0], W["y_test"]) < TOL and maxrel(y[99], W["y_test"]) < TOL
+    plan.close()
+
+
+@pytest.mark.parametrize("rows", [1, 63, 64, 65, 1000])
+def test_chain_ragged_rows(L, gpu, rows):
+    """SAM-shaped 61 -> 128 x4 -> 148 network (benchmarks/sam/fwd_native.f90:5, 34-42), row counts around
+    the 64-row tile."""
+    rng = np.random.default_rng(0)
+    widths = [61, 128, 128, 128, 128, 148]
+    Ws = [(rng.standard_normal((widths[i + 1], widths[i])) / np.sqrt(widths[i])).astype(np.float32) for i in range(5)]
+    bs = [rng.standard_normal(widths[i + 1]).astype(np.float32) * 0.1 for i in range(5)]
+    X = rng.standard_normal((rows, 61)).astype(np.float32)
+    plan = P.mlp_plan(Ws, bs, ["relu"] * 4 + [None], rows)
+    assert plan.num_kernels == 1
+    Y = plan.forward(X, (rows, 148))
+    assert maxrel(Y, O.mlp_f64(Ws, bs, ["relu"] * 4 + ["none"], X)) < TOL
+    plan.close()
+
+
+def test_config3_climsim_shape_reduced_rows(L, gpu):
+    """556 -> 768 x5 LeakyReLU(0.15) -> 368 with the column-major gather/scatter around it, 1024 rows."""
+    case = configs.climsim(rows=1024)
+    plan = configs.climsim_plan(case)
+    B = plan.forward(case["A"].reshape(-1, order="F"), (368, 1024)).T      # column-major (1024, 368)
+    X = O.boundary_pre(case["A"], case["mean"], case["vmax"], case["vmin"])
+    Yref = O.mlp_f64(case["Ws"], case["bs"], case["acts"], X, alphas=case["alphas"])
+    ref = O.boundary_post(Yref, case["scale"])
+    assert maxrel(B, ref) < TOL
+    plan.close()
+
+
+def test_config3_climsim_full_size_row_sample(L, gpu):
+    """All 24576 columns on the GPU; rows are independent, so a seeded sample of 192 rows is checked
+    against the oracle at full width."""
+    case = configs.climsim()
+    plan = configs.climsim_plan(case, boundary=False)
+    X = np.ascontiguousarray(case["A"])                                   # row-major [24576][556]
+    Y = plan.forward(X, (24576, 368))
+    idx = np.random.default_rng(5).choice(24576, 192, replace=False)
+    ref = O.mlp_f64(case["Ws"], case["bs"], case["acts"], X[idx], alphas=case["alphas"])
+    assert maxrel(Y[idx], ref) < TOL
+    assert np.isfinite(Y).all()
+    plan.close()
+
+
+def test_masked_relu_head_and_output_scale_fold_into_gemm(L, gpu):
+    """124 -> 512 -> 128 with ReLU on the last 8 outputs (benchmarks/climsim/export_wide.py:24-28)."""
+    rng = np.random.default_rng(1)
+    Ws = [(rng.standard_normal((512, 124)) / 11).astype(np.float32), (rng.standard_normal((128, 512)) / 22).astype(np.float32)]
+    bs = [rng.standard_normal(512).astype(np.float32), rng.standard_normal(128).astype(np.float32)]
+    X = rng.standard_normal((384, 124)).astype(np.float32)
+    plan = P.mlp_plan(Ws, bs, ["leaky", None], 384, alphas=[0.15, 0.0], mask_tail=8)
+    assert plan.num_kernels == 2                    # mask head folded into the second GEMM's epilogue
+    Y = plan.forward(X, (384, 128))
+    assert maxrel(Y, O.mlp_f64(Ws, bs, ["leaky", "none"], X, alphas=[0.15, 0.0], mask_tail=8)) < TOL
+    assert (Y[:, 120:] >= 0).all() and (Y[:, :120] < 0).any()
+    plan.close()
+    out_norms = rng.uniform(0.5, 2, 128).astype(np.float32)
+    plan = P.mlp_plan(Ws, bs, ["leaky", None], 384, alphas=[0.15, 0.0], out_norms=out_norms)
+    assert plan.num_kernels == 2
+    Y = plan.forward(X, (384, 128))
+    assert maxrel(Y, O.mlp_f64(Ws, bs, ["leaky", "none"], X, alphas=[0.15, 0.0], out_norms=out_norms)) < TOL
+    plan.close()
+
+
+@pytest.mark.parametrize("B,N,K", [(1, 1, 4), (64, 64, 32), (100, 70, 36), (33, 17, 7), (512, 768, 556), (300, 368, 768)])
+def test_fortis_gemm_entry(L, gpu, B, N, K):
+    """The memref-expanded entry (runtime/fortis_rt.c:45-48): C = A . W^T, offsets honoured, any shape
+    (K = 7 takes the guarded non-vector path)."""
+    rng = np.random.default_rng(2)
+    pad = 8                                           # elements of offset into each allocation
+    A = rng.standard_normal(B * K + pad).astype(np.float32)
+    W = rng.standard_normal(N * K + pad).astype(np.float32)
+    dA, dW, dC = DevBuf(L, A), DevBuf(L, W), DevBuf(L, nbytes=(B * N + pad) * 4)
+    L.fortis_gemm(dA.ptr, dA.ptr, pad, B, K, K, 1, dW.ptr, dW.ptr, pad, N, K, K, 1, dC.ptr, dC.ptr, pad, B, N, N, 1, B, N, K)
+    Cc = dC.get((B * N + pad,))[pad:].reshape(B, N)
+    assert maxrel(Cc, O.gemm(A[pad:].reshape(B, K), W[pad:].reshape(N, K))) < TOL
+    for d in (dA, dW, dC):
+        d.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("NI,NK", [(384, 124), (50, 33), (1, 1)])
+def test_boundary_pre_post_bit_exact(L, gpu, dtype, NI, NK):
+    """E3SM boundary shapes (384 x 124 f64 in, trt_backend/e3sm_boundary.cu:9-20) and ragged ones;
+    host-type arithmetic then cast, bit-exact against the oracle."""
+    rng = np.random.default_rng(3)
+    A = np.asfortranarray(rng.standard_normal((NI, NK)).astype(dtype))
+    mean, vmax, vmin = rng.standard_normal(NK).astype(dtype), rng.uniform(2, 3, NK).astype(dtype), rng.uniform(0, 1, NK).astype(dtype)
+    scale = rng.uniform(0.5, 2, NK).astype(dtype)
+    esz = np.dtype(dtype).itemsize
+    p = P.Plan()
+    t0, t1, t2 = p.tensor(NI * NK, esz), p.tensor(NI * NK), p.tensor(NI * NK, esz)
+    p.boundary_pre(t0, t1, NI, NK, mean, vmax, vmin, dtype)
+    p.boundary_post(t1, t2, NI, NK, scale, dtype)
+    p.finalize(t0, t2)
+    p.write(t0, A.reshape(-1, order="F"))
+    p.run()
+    X = p.read(t1, (NI, NK))
+    Bm = p.read(t2, (NK, NI), dtype).T
+    Xref = O.boundary_pre(A, mean, vmax, vmin)
+    assert np.array_equal(X.view(np.uint32), Xref.view(np.uint32))
+    assert np.array_equal(Bm, O.boundary_post(Xref, scale, dtype))
+    p.close()

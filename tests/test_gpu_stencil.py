@@ -1,0 +1,167 @@
+"""Stencil gather / scatter and the fused gather->MLP->scatter step on the GPU, through the C ABI,
+against the CPU oracle.  Index maps and expression arithmetic: bit-exact.  Model outputs: 1e-5."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+from fortis_amd import configs, plan as P, stencil as S
+from oracle import oracle as O
+from util import TOL, DevBuf, bits_equal, maxrel, ptrs
+
+pytestmark = pytest.mark.gpu
+
+
+def golden_tables(golden, cells=None):
+    return S.load_tables(*[os.path.join(golden, f"zb_{n}.json") for n in ("gather", "scatter", "loop", "kdist")], cells=cells)
+
+
+@pytest.fixture(scope="module")
+def zbhost(golden):
+    W = np.load(os.path.join(golden, "zb_nn.npz"))
+    F = O.zb_fields()
+    Pp = O.zb_prep(F)
+    return dict(W=W, F=F, P=Pp, Ws=[W["A0"], W["A1"]], bs=[W["b0"], W["b1"]],
+                garr=[Pp["sh_xy_h"], F["sh_xx"], Pp["vort_xy_h"], Pp["norm_h"]])
+
+
+def test_gather_reference_geometry_bit_exact(L, gpu, golden, zbhost):
+    gt, st, gd, sd, lp, kd = golden_tables(golden)
+    bufs = [DevBuf(L, a) for a in zbhost["garr"]]
+    dX = DevBuf(L, nbytes=71040 * 27 * 4)
+    L.fortis_stencil_gather_dev(C.byref(gt), ptrs(bufs), dX.ptr)
+    X = dX.get((71040, 27))
+    ref = O.stencil_gather(gd, zbhost["garr"], 4736, 15, 3, 3, 64)
+    assert bits_equal(X, ref)
+    for b in bufs + [dX]:
+        b.free()
+
+
+@pytest.mark.parametrize("sx,sy,nz", [(48, 58, 10), (9, 7, 1), (133, 70, 3)])
+def test_gather_scatter_other_grids_bit_exact(L, gpu, sx, sy, nz):
+    """48x58x10 -> 44x54 = 2376 cells per layer is the reference's second specialisation size
+    (mom6_zb/README.md:37); the others are ragged (count not a multiple of the block) and tiny."""
+    gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    gt, st = S.build_table(gd, lp, kd, "gather"), S.build_table(sd, lp, kd, "scatter")
+    A = configs.zb_arrays(sx, sy, nz)
+    garr = [A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"]]
+    count = (sx - 4) * (sy - 4)
+    bufs = [DevBuf(L, a) for a in garr]
+    dX = DevBuf(L, nbytes=count * nz * 27 * 4)
+    L.fortis_stencil_gather_dev(C.byref(gt), ptrs(bufs), dX.ptr)
+    X = dX.get((count * nz, 27))
+    assert bits_equal(X, O.stencil_gather(gd, garr, count, nz, 3, 3, sx - 4))
+    # scatter of a random Y, one enclosing-loop iteration at a time, onto full-depth device arrays
+    Y = np.random.default_rng(4).standard_normal((count * nz, 3)).astype(np.float32)
+    host = [A["norm_h"], A["kappa_h"], np.zeros(sx * sy, np.float32), np.zeros(sx * sy * nz, np.float32), np.zeros(sx * sy * nz, np.float32)]
+    ref = [a.copy() for a in host]
+    sb = [DevBuf(L, a) for a in host]
+    dY = DevBuf(L, Y)
+    for kk in range(nz):
+        L.fortis_stencil_scatter_dev(C.byref(st), ptrs(sb), C.c_void_p(dY.ptr + kk * count * 3 * 4), kk)
+        O.stencil_scatter(sd, ref, Y[kk * count:(kk + 1) * count], count, kk, 3, 3, sx - 4)
+    for b, r in zip(sb[2:], ref[2:]):
+        assert bits_equal(b.get(r.shape), r)
+    for b in bufs + sb + [dX, dY]:
+        b.free()
+
+
+@pytest.mark.parametrize("ncells", [4736, 2376])
+def test_gather_scatter_masked_cell_list_bit_exact(L, gpu, ncells):
+    """480 x 240 grid with a 1-cell halo and a seeded ~30 % land mask; the first 4736 (2376) usable
+    ocean cells form the active list."""
+    sx, sy, nz = 482, 242, 2
+    gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    A = configs.zb_arrays(sx, sy, nz, mask_land=0.3)
+    cells = configs.zb_cells_from_mask(A["mask"], sx, sy, ncells)
+    gt, st = S.build_table(gd, lp, kd, "gather", cells), S.build_table(sd, lp, kd, "scatter", cells)
+    garr = [A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"]]
+    bufs = [DevBuf(L, a) for a in garr]
+    dX = DevBuf(L, nbytes=ncells * nz * 27 * 4)
+    L.fortis_stencil_gather_dev(C.byref(gt), ptrs(bufs), dX.ptr)
+    X = dX.get((ncells * nz, 27))
+    assert bits_equal(X, O.stencil_gather(gd, garr, ncells, nz, cells=cells))
+    Y = np.random.default_rng(4).standard_normal((ncells * nz, 3)).astype(np.float32)
+    host = [A["norm_h"], A["kappa_h"], np.zeros(sx * sy, np.float32), np.zeros(sx * sy * nz, np.float32), np.zeros(sx * sy * nz, np.float32)]
+    ref = [a.copy() for a in host]
+    sb = [DevBuf(L, a) for a in host]
+    dY = DevBuf(L, Y)
+    for kk in range(nz):
+        L.fortis_stencil_scatter_dev(C.byref(st), ptrs(sb), C.c_void_p(dY.ptr + kk * ncells * 3 * 4), kk)
+        O.stencil_scatter(sd, ref, Y[kk * ncells:(kk + 1) * ncells], ncells, kk, cells=cells)
+    for b, r in zip(sb[2:], ref[2:]):
+        assert bits_equal(b.get(r.shape), r)
+    for b in bufs + sb + [dX, dY]:
+        b.free()
+
+
+def _fused(L, gt, st, plan, garr, sarr_host, rows, nout=3):
+    gb = [DevBuf(L, a) for a in garr]
+    sb = [DevBuf(L, a) for a in sarr_host]
+    dY = DevBuf(L, nbytes=rows * nout * 4)
+    rc = L.fortis_stencil_step_fused(C.byref(gt), C.byref(st), plan.handle, ptrs(gb), ptrs(sb), dY.ptr)
+    assert rc == 0
+    L.fortis_sync()
+    out = [b.get(a.shape) for b, a in zip(sb, sarr_host)]
+    Y = dY.get((rows, nout))
+    for b in gb + sb + [dY]:
+        b.free()
+    return out, Y
+
+
+def test_fused_step_reference_network_vs_native_host(L, gpu, golden, zbhost):
+    """One kernel for gather -> 27-20-3 ANN -> scatter over all 15 layers, against the cell-by-cell
+    host loop (which the oracle tests tie bit-for-bit to the reference's own Fortran build)."""
+    gt, st, gd, sd, lp, kd = golden_tables(golden)
+    W = zbhost["W"]
+    plan = P.mlp_plan(zbhost["Ws"], zbhost["bs"], ["relu", None], 71040, in_norms=W["in_norms"], out_norms=W["out_norms"])
+    assert plan.num_kernels == 1
+    F, Pp = zbhost["F"], zbhost["P"]
+    n3 = 68 * 78 * 15
+    host = [Pp["norm_h"], F["kappa_h"], np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+    out, Y = _fused(L, gt, st, plan, zbhost["garr"], host, 71040)
+    T = O.zb_step_native(F, Pp, zbhost["Ws"], zbhost["bs"], W["in_norms"], W["out_norms"])
+    assert maxrel(out[3], T["Txx"]) < TOL and maxrel(out[4], T["Tyy"]) < TOL
+    assert maxrel(out[2].reshape(15, -1)[14], T["Txy_h"]) < TOL       # the host's 2-D Txy_h holds the last layer
+    # golden fixture layers written by the reference build
+    G = np.load(os.path.join(golden, "zb_native_golden.npz"))
+    assert maxrel(out[3].reshape(15, 78, 68)[G["layers"] - 1], G["Txx"]) < TOL
+    # the scatter applied to the kernel's own raw outputs is bit-exact
+    ref = [a.copy() for a in host[:2]] + [np.zeros(68 * 78, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+    for kk in range(15):
+        O.stencil_scatter(sd, ref, Y[kk * 4736:(kk + 1) * 4736], 4736, kk, 3, 3, 64)
+    assert bits_equal(out[3], ref[3]) and bits_equal(out[4], ref[4])
+    plan.close()
+
+
+@pytest.mark.parametrize("hidden", [(64, 64), (20,), (128, 32, 8)])
+def test_fused_step_config2_network(L, gpu, golden, hidden):
+    """Config 2's 27->64->64->3 network (and two other shapes) on the reference geometry, against the
+    fp64-accumulated chain run on the oracle's gathered rows."""
+    gt, st, gd, sd, lp, kd = golden_tables(golden)
+    A = configs.zb_arrays(68, 78, 15)
+    net = configs.zb_mlp(hidden)
+    plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], 71040)
+    garr = [A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"]]
+    n3 = 68 * 78 * 15
+    host = [A["norm_h"], A["kappa_h"], np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+    out, Y = _fused(L, gt, st, plan, garr, host, 71040)
+    X = O.stencil_gather(gd, garr, 4736, 15, 3, 3, 64)
+    Yref = O.mlp_f64(net["Ws"], net["bs"], net["acts"], X)
+    assert maxrel(Y, Yref) < TOL
+    ref = [a.copy() for a in host[:2]] + [np.zeros(68 * 78, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+    for kk in range(15):
+        O.stencil_scatter(sd, ref, Yref[kk * 4736:(kk + 1) * 4736], 4736, kk, 3, 3, 64)
+    assert maxrel(out[3], ref[3]) < TOL and maxrel(out[4], ref[4]) < TOL
+    plan.close()
+
+
+def test_fused_step_rejects_mismatched_tables(L, gpu, golden, capfd):
+    gt, st, gd, sd, lp, kd = golden_tables(golden)
+    net = configs.toy_mlp(64)
+    plan = configs.mlp_case_plan(net)               # 64 inputs, not 27
+    assert L.fortis_stencil_step_fused(C.byref(gt), C.byref(st), plan.handle, None, None, None) == -1
+    assert "do not match" in capfd.readouterr().err
+    plan.close()

@@ -1,0 +1,166 @@
+"""Host-side logic that needs no GPU: pool policy, plan argument checks, table building and
+expression lowering."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+from fortis_amd import stencil as S
+from fortis_amd._lib import Ins, Stencil
+
+# ---- pool: the reference's policy (runtime/fortis_rt.c:14-40) on a host allocator ---------------
+ALLOC = C.CFUNCTYPE(C.c_int, C.POINTER(C.c_void_p), C.c_size_t)
+FREE = C.CFUNCTYPE(None, C.c_void_p)
+
+
+class FakeDevice:
+    def __init__(self, capacity):
+        self.capacity, self.live, self.next = capacity, {}, 0x1000
+        self.allocs = self.frees = 0
+
+        def a(pp, n):
+            if sum(self.live.values()) + n > self.capacity:
+                return -1
+            self.next += 0x100000
+            self.live[self.next] = n
+            pp[0] = self.next
+            self.allocs += 1
+            return 0
+
+        def f(p):
+            del self.live[p]
+            self.frees += 1
+
+        self.a, self.f = ALLOC(a), FREE(f)
+
+
+@pytest.fixture
+def pool(L):
+    dev = FakeDevice(1000)
+    L.fortis_pool_set_allocator(C.cast(dev.a, C.c_void_p), C.cast(dev.f, C.c_void_p))
+    yield L, dev
+    L.fortis_pool_set_allocator(None, None)
+
+
+def stats(L):
+    h, u = C.c_int(), C.c_int()
+    L.fortis_pool_stats(C.byref(h), C.byref(u))
+    return h.value, u.value
+
+
+def test_pool_best_fit_reuse(pool):
+    L, dev = pool
+    a, b, c = L.fortis_alloc(100), L.fortis_alloc(300), L.fortis_alloc(200)
+    assert dev.allocs == 3 and stats(L) == (3, 3)
+    for p in (a, b, c):
+        L.fortis_free(p)
+    assert stats(L) == (3, 0) and dev.frees == 0          # released buffers stay allocated
+    assert L.fortis_alloc(150) == c                        # smallest released buffer that fits
+    assert L.fortis_alloc(150) == b
+    assert L.fortis_alloc(50) == a
+    assert dev.allocs == 3
+
+
+def test_pool_release_all_and_retry_on_oom(pool):
+    L, dev = pool
+    a, b = L.fortis_alloc(400), L.fortis_alloc(400)
+    L.fortis_free(a)
+    L.fortis_free(b)
+    c = L.fortis_alloc(900)                                # does not fit beside 800 held bytes
+    assert c and dev.frees == 2 and stats(L) == (1, 1)
+    assert not L.fortis_alloc(200)                         # genuinely out of memory: NULL, no crash
+    L.fortis_free(c)
+    assert L.fortis_alloc(900) == c
+
+
+def test_pool_unknown_pointer_is_really_freed(pool):
+    L, dev = pool
+    p = C.c_void_p()
+    assert dev.a(C.byref(p), 10) == 0
+    L.fortis_free(p.value)
+    assert dev.frees == 1
+
+
+# ---- plan argument checks (no device work before finalize) ------------------------------------------
+def test_plan_rejects_bad_arguments(L):
+    p = L.fortis_plan_create()
+    t0, t1 = L.fortis_plan_tensor(p, 64 * 27 * 4), L.fortis_plan_tensor(p, 64 * 3 * 4)
+    W = np.zeros((3, 27), np.float32)
+    vp = W.ctypes.data_as(C.c_void_p)
+    assert L.fortis_plan_tensor(p, 0) == -1
+    assert L.fortis_plan_linear(p, t0, t1, vp, None, 64, 27, 3, 0, 0.0) == 0
+    assert L.fortis_plan_linear(p, t0, t1, vp, None, 65, 27, 3, 0, 0.0) == -1      # tensor too small
+    assert L.fortis_plan_linear(p, t0, t0, vp, None, 64, 27, 27, 0, 0.0) == -1     # aliased
+    assert L.fortis_plan_linear(p, t0, 7, vp, None, 64, 27, 3, 0, 0.0) == -1       # unknown tensor
+    assert L.fortis_plan_linear(p, t0, t1, vp, None, 64, 27, 3, 9, 0.0) == -1      # unknown activation
+    assert L.fortis_plan_linear(p, t0, t1, None, None, 64, 27, 3, 0, 0.0) == -1
+    assert L.fortis_plan_mask_relu(p, t1, t1, 64, 3, 4) == -1                       # tail > n
+    assert L.fortis_plan_conv2d(p, t0, t1, vp, None, vp, None, None, None, 1e-5, 1, 8, 8, 1, 3, 3, 1, 1, 0, 0.0, 0, 0) == -1  # partial BN
+    assert L.fortis_plan_num_kernels(p) == -1                                       # not finalized
+    L.fortis_plan_destroy(p)
+
+
+def test_entries_without_a_bound_step_do_not_crash(L, capfd):
+    L.fortis_step_reset()
+    L.mlp_forward_dev()
+    assert "no step bound" in capfd.readouterr().err
+
+
+# ---- tables ---------------------------------------------------------------------------------------------
+def test_zb_tables_from_the_reference_descriptors(golden, L):
+    g, s, gd, sd, lp, kd = S.load_tables(*[os.path.join(golden, f"zb_{n}.json") for n in ("gather", "scatter", "loop", "kdist")])
+    assert (g.count, g.nk, g.klo, g.ilo, g.jlo, g.ni, g.nj, g.nargs) == (4736, 15, 1, 3, 3, 64, 74, 0)
+    assert (s.count, s.nk, s.nrefs, s.nscal, s.nargs) == (4736, 15, 3, 2, 1)
+    # slot q = f*9 + (dj+1)*3 + (di+1) reads A_f[(i+di-1) + (j+dj-1)*68] (mom6_zb/gather.cu:21-48)
+    for q in range(27):
+        f, dj, di = q // 9, (q % 9) // 3 - 1, q % 3 - 1
+        r = g.refs[q]
+        assert (r.array, r.planar, r.base, r.si, r.sj) == (f, 1, (di - 1) + (dj - 1) * 68, 1, 68)
+    assert [g.plane[a] for a in range(4)] == [5304] * 4 and [g.total[a] for a in range(4)] == [79560] * 4
+    assert [s.plane[a] for a in range(5)] == [5304] * 5 and [s.total[a] for a in range(5)] == [79560, 5304, 5304, 79560, 79560]
+    assert [(s.refs[q].array, s.refs[q].planar) for q in range(3)] == [(2, 0), (3, 1), (4, 1)]
+    assert L.fortis_stencil_check(C.byref(g)) == 0 and L.fortis_stencil_check(C.byref(s)) == 0
+
+
+def test_batch_already_multiplied_by_nk_is_accepted(golden):
+    paths = [os.path.join(golden, f"zb_{n}.json") for n in ("gather", "scatter", "loop", "kdist")]
+    gd, lp, kd = json.load(open(paths[0])), json.load(open(paths[2])), json.load(open(paths[3]))
+    lp["batch"] *= kd["nk"]                                 # what driver/fortisc.sh:44 does before emitting
+    assert S.build_table(gd, lp, kd, "gather").count == 4736
+
+
+def test_expression_compiler():
+    assert S.compile_exprs(["(((tv * S0) * S0) * S1)"])[0] == [(2, 0, 1), (2, 32, 1), (2, 33, 2)]
+    ins, consts = S.compile_exprs(["(tv / (S0 + 1.000000e-30f))"])
+    assert ins == [(0, 1, 16), (3, 0, 32)] and consts == [float(np.float32(1e-30))]
+    ins, _ = S.compile_exprs(["(tv * S0)", "(tv - 2.0f)"])   # two expressions in order, each replacing tv
+    assert ins == [(2, 0, 1), (1, 32, 16)]
+    with pytest.raises(ValueError):
+        S.compile_exprs(["sqrtf(tv)"])
+
+
+def _table_with(ins, nscal=2, nconst=1):
+    t = Stencil()
+    t.narrays, t.nrefs, t.nscal, t.count, t.nk, t.ni, t.sx = 1, 1, nscal, 4, 1, 2, 4
+    t.total[0] = t.plane[0] = 16
+    t.nins, t.nconst = len(ins), nconst
+    for n, i3 in enumerate(ins):
+        t.ins[n] = Ins(*i3)
+    return t
+
+
+def test_lowering_accepts_chains_and_rejects_the_rest(L, capfd):
+    ok = [[(0, 1, 16), (3, 0, 32)], [(2, 0, 1), (2, 32, 1), (2, 33, 2)], [(1, 16, 0)], []]
+    for ins in ok:
+        assert L.fortis_stencil_check(C.byref(_table_with(ins))) == 0
+    bad = [[(2, 0, 0)],                      # tv * tv
+           [(2, 0, 1), (0, 32, 0)],          # re-reads tv after transforming it
+           [(2, 0, 1), (0, 1, 2)],           # last instruction does not produce the slot value
+           [(0, 1, 2)],                      # never uses tv
+           [(7, 0, 1)],                      # unknown op
+           [(0, 0, 5)]]                      # scalar out of range
+    for ins in bad:
+        assert L.fortis_stencil_check(C.byref(_table_with(ins))) == -1
+    capfd.readouterr()
