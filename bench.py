@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused inference step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload climsim|zb|zb_ref|toy] [--no-cpu]
+
+One "step" is one pass of the hot path over one batch of synthetic input that is already resident
+in HBM.  Prints ONE JSON line: columns/s for the whole job, the roofline figure of the dominant
+kernel (duration measured with HIP events on the library's own stream inside the timed region) and
+a CPU baseline (the oracle's port of the reference's native Fortran forward, timed on this host on a
+bounded sample of the same workload).  Only the cpu_baseline leg touches oracle/.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_F32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# same command (see profiles/), or None where no counter run has been made for the workload.
+MEASURED_TRAFFIC = {"climsim": (122875 + 68525) * 1024, "zb": None, "zb_ref": None, "toy": None}
+
+
+def omp_threads():
+    try:
+        return int(os.environ.get("OMP_NUM_THREADS", "")) or os.cpu_count()
+    except ValueError:
+        return os.cpu_count()
+
+
+def cpu_baseline_mlp(case, sample_rows, X, min_seconds=8.0, **kw):
+    """Times oracle.mlp_native_t (native Fortran loop nest, OpenMP over columns) on `sample_rows` rows."""
+    from oracle import oracle as O   # checker / baseline only
+    Xs = np.ascontiguousarray(X[:sample_rows])
+    O.mlp_native_t(case["Ws"], case["bs"], case["acts"], Xs[:64], alphas=case.get("alphas"), **kw)   # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        O.mlp_native_t(case["Ws"], case["bs"], case["acts"], Xs, alphas=case.get("alphas"), **kw)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds or reps >= 100000:
+            break
+    return dict(value=sample_rows * reps / dt, unit="columns/s", cores=omp_threads(), kind="port",
+                sample=f"{sample_rows} of {case['rows']} rows x {reps} passes of oracle mlp_native_t "
+                       f"(native Fortran loop order, fp32, OpenMP over columns), {dt:.1f} s")
+
+
+def run_climsim(L, args):
+    from fortis_amd import configs
+    case = configs.climsim()
+    plan = configs.climsim_plan(case, boundary=True)
+    plan.write(plan.in_tensor, case["A"].reshape(-1, order="F"))
+    for _ in range(args.warmup):
+        plan.run()
+    L.fortis_sync()
+    plan.profile(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        plan.run()
+    L.fortis_sync()
+    dt = time.perf_counter() - t0
+    passes, per = plan.profile_read()
+    plan.profile(False)
+    assert passes == args.steps
+    gemm_ms = sum(ms for name, ms in per if name == "gemm_bias_act")
+    ngemm = sum(1 for name, _ in per if name == "gemm_bias_act")
+    avg_launch_ms = gemm_ms / (ngemm * passes)
+    flops_per_launch = case["flops"] / ngemm
+    achieved = flops_per_launch / (avg_launch_ms * 1e-3) / 1e12
+    kern = {name: 0.0 for name, _ in per}
+    for name, ms in per:
+        kern[name] += ms / passes
+    out = dict(rows=case["rows"], dt=dt, dtype="f32",
+               config={"workload": "climsim_mlp_24576x556_768x5_368", "columns": case["rows"],
+                       "widths": case["widths"], "step": "colmajor gather -> 6 fused GEMM+bias+LeakyReLU -> colmajor scatter",
+                       "launches_per_step": plan.num_kernels, "ms_per_step_by_kernel": {k: round(v, 4) for k, v in kern.items()}},
+               roofline=dict(bound="mfma", kernel="gemm_bias_act (fp32 MFMA 32x32x2)", achieved=round(achieved, 3),
+                             peak=PEAK_F32_MFMA_TFLOPS, unit="TFLOP/s", frac=round(achieved / PEAK_F32_MFMA_TFLOPS, 4),
+                             avg_launch_ms=round(avg_launch_ms, 5), flop_per_launch=flops_per_launch,
+                             traffic=MEASURED_TRAFFIC["climsim"]))
+    if not args.no_cpu:
+        X = np.ascontiguousarray(case["A"][:2048])
+        out["cpu_baseline"] = cpu_baseline_mlp(case, 2048, X)
+    plan.close()
+    return out
+
+
+def run_copy(L, args):
+    """Plain device copy of 256 MiB (concat-by-copy kernel): the known-size kernel the HBM counters are
+    calibrated against, and the achievable-bandwidth yardstick for the memory-bound kernels."""
+    from fortis_amd import plan as P
+    n = 64 * 1024 * 1024
+    p = P.Plan()
+    a, b = p.tensor(n), p.tensor(n)
+    p.concat_copy(a, b, 1, n, 0, 1)
+    p.finalize(a, b)
+    p.write(a, np.ones(n, np.float32))
+    p.time_ms(max(1, args.warmup))
+    L.fortis_sync()
+    t0 = time.perf_counter()
+    ms = p.time_ms(args.steps)
+    L.fortis_sync()
+    dt = time.perf_counter() - t0
+    avg = ms / args.steps
+    gbs = 2 * n * 4 / (avg * 1e-3) / 1e9
+    out = dict(rows=n, dt=dt, dtype="f32", config={"workload": "device_copy_256MiB", "columns": n, "launches_per_step": 1},
+               roofline=dict(bound="hbm", kernel="copy_kernel", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                             frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(avg, 5), bytes_per_launch=2 * n * 4, traffic=None))
+    p.close()
+    return out
+
+
+def run_toy(L, args):
+    from fortis_amd import configs
+    case = configs.toy_mlp()
+    plan = configs.mlp_case_plan(case)
+    plan.write(plan.in_tensor, case["X"])
+    plan.time_ms(max(1, args.warmup))
+    L.fortis_sync()
+    t0 = time.perf_counter()
+    ms = plan.time_ms(args.steps, graph=False)
+    L.fortis_sync()
+    dt = time.perf_counter() - t0
+    avg = ms / args.steps
+    achieved = case["flops"] / (avg * 1e-3) / 1e12
+    out = dict(rows=case["rows"], dt=dt, dtype="f32",
+               config={"workload": "toy_mlp_1024x64_256_256_32", "columns": case["rows"], "launches_per_step": plan.num_kernels},
+               roofline=dict(bound="mfma", kernel="mlp_chain (LDS-resident, fp32 MFMA)", achieved=round(achieved, 4),
+                             peak=PEAK_F32_MFMA_TFLOPS, unit="TFLOP/s", frac=round(achieved / PEAK_F32_MFMA_TFLOPS, 5),
+                             avg_launch_ms=round(avg, 5), flop_per_launch=case["flops"], traffic=MEASURED_TRAFFIC["toy"]))
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_mlp(case, case["rows"], case["X"], min_seconds=3.0)
+    plan.close()
+    return out
+
+
+def run_zb(L, args, reference_net=False):
+    """gather -> MLP -> scatter for all 15 layers of the reference geometry in one kernel."""
+    from fortis_amd import configs, plan as P, stencil as S
+    sx, sy, nz = 68, 78, 15
+    g = os.path.join(ROOT, "tests", "golden")
+    gt, st, gd, sd, lp, kd = S.load_tables(f"{g}/zb_gather.json", f"{g}/zb_scatter.json", f"{g}/zb_loop.json", f"{g}/zb_kdist.json")
+    A = configs.zb_arrays(sx, sy, nz)
+    rows = gt.count * gt.nk
+    if reference_net:
+        W = np.load(f"{g}/zb_nn.npz")
+        net = dict(Ws=[W["A0"], W["A1"]], bs=[W["b0"], W["b1"]], acts=["relu", None], widths=[27, 20, 3])
+        plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows, in_norms=W["in_norms"], out_norms=W["out_norms"])
+        extra = dict(in_norms=W["in_norms"], out_norms=W["out_norms"])
+    else:
+        net = configs.zb_mlp()
+        plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows)
+        extra = {}
+    garr = [A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"]]
+    n3 = sx * sy * nz
+    sarr = [A["norm_h"], A["kappa_h"], np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+
+    def dev(a):
+        d = L.fortis_alloc(a.nbytes)
+        L.fortis_h2d(d, a.ctypes.data, a.nbytes)
+        return d
+    dG = (C.c_void_p * 4)(*[dev(a) for a in garr])
+    dS = (C.c_void_p * 5)(*[dev(a) for a in sarr])
+    L.fortis_stencil_step_fused_time_ms(C.byref(gt), C.byref(st), plan.handle, dG, dS, None, max(1, args.warmup))
+    L.fortis_sync()
+    t0 = time.perf_counter()
+    ms = L.fortis_stencil_step_fused_time_ms(C.byref(gt), C.byref(st), plan.handle, dG, dS, None, args.steps)
+    L.fortis_sync()
+    dt = time.perf_counter() - t0
+    avg = ms / args.steps          # the helper runs one validating launch before the clocked ones
+    widths = net["widths"]
+    flops = 2 * rows * sum(widths[i] * widths[i + 1] for i in range(len(widths) - 1))
+    # algorithmic bytes: 4 input planes + kappa read once, 3 output values per cell written, weights once
+    nbytes = 4 * (4 * n3 + sx * sy + 3 * rows + sum(w.size + b.size for w, b in zip(net["Ws"], net["bs"])))
+    tf, gbs = flops / (avg * 1e-3) / 1e12, nbytes / (avg * 1e-3) / 1e9
+    # the fused kernel's arithmetic intensity decides the bound: flop/byte against 157.3e12 / 8e12 = 19.7
+    bound = "mfma" if flops / nbytes > PEAK_F32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9) else "hbm"
+    roof = dict(bound=bound, kernel="mlp_chain<stencil> (gather -> MLP -> scatter, one launch)",
+                achieved=round(tf if bound == "mfma" else gbs, 3), peak=PEAK_F32_MFMA_TFLOPS if bound == "mfma" else PEAK_HBM_GBS,
+                unit="TFLOP/s" if bound == "mfma" else "GB/s",
+                frac=round((tf / PEAK_F32_MFMA_TFLOPS) if bound == "mfma" else (gbs / PEAK_HBM_GBS), 5),
+                avg_launch_ms=round(avg, 5), flop_per_launch=flops, bytes_per_launch=nbytes,
+                hbm_GBs=round(gbs, 2), mfma_TFLOPs=round(tf, 3), traffic=MEASURED_TRAFFIC["zb_ref" if reference_net else "zb"])
+    # dt covers the validating launch too; whole-job throughput uses the clocked launches only
+    out = dict(rows=rows, dt=ms * 1e-3, wall_dt=dt, dtype="f32",
+               config={"workload": "zb_gather_mlp_scatter_%s_68x78x15" % ("27_20_3" if reference_net else "27_64_64_3"),
+                       "columns": rows, "cells_per_layer": int(gt.count), "layers": int(gt.nk), "widths": widths,
+                       "launches_per_step": 1},
+               roofline=roof)
+    if not args.no_cpu:
+        from oracle import oracle as O
+        X = O.stencil_gather(gd, garr, int(gt.count), int(gt.nk), 3, 3, 64)
+        case = dict(net, rows=rows)
+        out["cpu_baseline"] = cpu_baseline_mlp(case, rows, X, min_seconds=5.0, **extra)
+        out["cpu_baseline"]["sample"] += " (MLP part only; the gather and scatter loops of the host are not included)"
+    plan.close()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="climsim", choices=["climsim", "zb", "zb_ref", "toy", "copy"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the fused step on ONE GPU; --gpus %d is not supported "
+              "(the path has no inter-GPU exchange to measure)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import fortis_amd
+    L = fortis_amd.load()
+    name = C.create_string_buffer(64)
+    if L.fortis_device_info(name, 64, None) != 0:
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    if args.workload == "climsim":
+        r = run_climsim(L, args)
+    elif args.workload == "toy":
+        r = run_toy(L, args)
+    elif args.workload == "copy":
+        r = run_copy(L, args)
+    else:
+        r = run_zb(L, args, reference_net=(args.workload == "zb_ref"))
+    ms_per_step = r["dt"] / args.steps * 1e3
+    line = {"metric": "columns/sec per fused forward step", "value": r["rows"] * args.steps / r["dt"], "unit": "columns/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "device": name.value.decode(),
+            "config": r["config"], "roofline": r["roofline"]}
+    if "cpu_baseline" in r:
+        line["cpu_baseline"] = r["cpu_baseline"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -49,6 +49,9 @@ struct fortis_plan {
     bool finalized = false;
     int in_t = -1, out_t = -1;
     long rows0 = 0;             // rows at finalize (row-wise plans), for run-time extents
+    bool prof = false;          // per-kernel event timing (fortis_plan_profile)
+    std::vector<hipEvent_t> ev; // events of the recorded passes: (nexec + 1) per pass
+    size_t ev_used = 0;
 };
 
 static void* upload(fortis_plan* p, const void* h, size_t nbytes)
@@ -398,6 +401,12 @@ void fortis_plan_run(fortis_plan* p)
 {
     if (!p || !p->finalized) { fprintf(stderr, "fortis_plan_run: plan not finalized\n"); return; }
     hipStream_t s = fortis_stream_get();
+    auto mark = [&]() {
+        if (!p->prof || fortis_capturing) return;
+        if (p->ev_used == p->ev.size()) { hipEvent_t e; HIP_OK(hipEventCreate(&e)); p->ev.push_back(e); }
+        HIP_OK(hipEventRecord(p->ev[p->ev_used++], s));
+    };
+    mark();
     for (const Exec& e : p->exec) {
         const float* src = (const float*)p->tptr[e.src];
         float* dst = (float*)p->tptr[e.dst];
@@ -436,7 +445,40 @@ void fortis_plan_run(fortis_plan* p)
             case EX_PERMUTE: fortis_launch_permute(src, dst, o->C, o->H, o->flag, s); break;
         }
         if (rc != 0) fprintf(stderr, "fortis_plan_run: an op was rejected by its kernel launcher\n");
+        mark();
     }
+}
+
+static const char* const kExecNames[] = { "mlp_chain", "gemm_bias_act", "scale", "mask_relu", "boundary_pre", "boundary_post",
+                                          "conv2d", "convt2d", "maxpool2d", "upsample", "concat_copy", "conv3d", "permute" };
+const char* fortis_plan_kernel_name(fortis_plan* p, int idx)
+{
+    if (!p || !p->finalized || idx < 0 || idx >= (int)p->exec.size()) return "";
+    return kExecNames[p->exec[idx].kind];
+}
+void fortis_plan_profile(fortis_plan* p, int enable)
+{
+    if (!p) return;
+    p->prof = enable != 0;
+    p->ev_used = 0;
+    if (!enable) { for (hipEvent_t e : p->ev) HIP_OK(hipEventDestroy(e)); p->ev.clear(); }
+}
+int fortis_plan_profile_read(fortis_plan* p, float* ms_per_kernel)
+{
+    if (!p || !p->finalized) return -1;
+    const size_t per = p->exec.size() + 1;
+    const int passes = (int)(p->ev_used / per);
+    for (size_t k = 0; k < p->exec.size(); k++) ms_per_kernel[k] = 0.f;
+    if (passes == 0) return 0;
+    HIP_OK(hipEventSynchronize(p->ev[p->ev_used - 1]));
+    for (int n = 0; n < passes; n++)
+        for (size_t k = 0; k < p->exec.size(); k++) {
+            float ms = 0.f;
+            HIP_OK(hipEventElapsedTime(&ms, p->ev[n * per + k], p->ev[n * per + k + 1]));
+            ms_per_kernel[k] += ms;
+        }
+    p->ev_used = 0;
+    return passes;
 }
 
 void* fortis_plan_tensor_ptr(fortis_plan* p, int t)

@@ -354,4 +354,18 @@ int fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t*
     return 0;
 }
 
+
+struct FusedArgs { const fortis_stencil_t* g; const fortis_stencil_t* s; fortis_plan* p; const float* const* dG; float* const* dS; float* dY; };
+static void fused_cb(void* a)
+{
+    FusedArgs* f = (FusedArgs*)a;
+    fortis_stencil_step_fused(f->g, f->s, f->p, f->dG, f->dS, f->dY);
+}
+float fortis_stencil_step_fused_time_ms(const fortis_stencil_t* g, const fortis_stencil_t* sd, fortis_plan* p,
+                                        const float* const* dG, float* const* dS, float* dY, int iters)
+{
+    FusedArgs a = { g, sd, p, dG, dS, dY };
+    if (fortis_stencil_step_fused(g, sd, p, dG, dS, dY) != 0) return -1.f;   // validates, warms the table cache
+    return fortis_time_ms(fused_cb, &a, iters);
+}
 }  // extern "C"

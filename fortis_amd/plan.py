@@ -142,6 +142,16 @@ class Plan:
     def num_kernels(self):
         return self._L.fortis_plan_num_kernels(self._p)
 
+    def profile(self, enable=True):
+        self._L.fortis_plan_profile(self._p, 1 if enable else 0)
+
+    def profile_read(self):
+        """-> (passes, [(kernel name, total ms over the passes)])"""
+        n = self.num_kernels
+        ms = (C.c_float * n)()
+        passes = self._L.fortis_plan_profile_read(self._p, ms)
+        return passes, [(self._L.fortis_plan_kernel_name(self._p, k).decode(), float(ms[k])) for k in range(n)]
+
     def time_ms(self, iters, graph=False):
         return self._L.fortis_plan_time_ms(self._p, iters, 1 if graph else 0)
 

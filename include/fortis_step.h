@@ -208,8 +208,18 @@ int  fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t
 /* Runs fn(arg) `iters` times on the persistent stream between two HIP events on that stream and
  * returns the elapsed milliseconds (the benchmark's per-kernel clock). */
 float fortis_time_ms(void (*fn)(void*), void* arg, int iters);
-/* Same clock around `iters` enqueues of a plan / the fused stencil step / a graph replay. */
+/* Same clock around `iters` enqueues of a plan (use_graph: captured once, then replayed) and of
+ * the fused stencil step. */
 float fortis_plan_time_ms(fortis_plan* p, int iters, int use_graph);
+float fortis_stencil_step_fused_time_ms(const fortis_stencil_t* g, const fortis_stencil_t* s, fortis_plan* p,
+                                        const float* const* dG, float* const* dS, float* dY, int iters);
+/* Per-kernel clock: while enabled, every fortis_plan_run records a HIP event on the persistent
+ * stream before its first and after each of its kernels.  fortis_plan_profile_read adds up the
+ * elapsed milliseconds per kernel over the passes recorded since the last read, returns the
+ * number of passes and starts over.  fortis_plan_kernel_name names kernel idx of the pass. */
+void  fortis_plan_profile(fortis_plan* p, int enable);
+int   fortis_plan_profile_read(fortis_plan* p, float* ms_per_kernel);
+const char* fortis_plan_kernel_name(fortis_plan* p, int idx);
 
 #ifdef __cplusplus
 }

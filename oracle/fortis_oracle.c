@@ -14,7 +14,7 @@
  *        bit-compared against the output of the reference's own Fortran host + native forward
  *        (mom6_zb/zb_host.f90 + fwd_native_zb.f90, built by oracle/build_ref.sh with flang),
  *        via tests/golden/zb_native_golden.npz.
- *   orc_mlp_native / orc_mlp_f64
+ *   orc_mlp_native / orc_mlp_native_t / orc_mlp_f64
  *        reference-held known answer x_test -> y_test in mom6_zb/zb_nn.npz (copied as a data
  *        fixture to tests/golden/zb_nn.npz); README stamp 7.775037 for the toy MLP.
  *   orc_stencil_gather / orc_stencil_scatter
@@ -136,6 +136,49 @@ void orc_mlp_native(int nlayers, const int* widths, const float* const* W, const
                 for (int j = 0; j < no; j++) {
                     x2[j] = x2[j] + b[l][j];
                     if (l < nlayers - 1) x2[j] = x2[j] > 0.0f ? x2[j] : 0.0f;
+                }
+                float* t = x1; x1 = x2; x2 = t;
+            }
+            float* y = Y + (size_t)r * widths[nlayers];
+            for (int j = 0; j < widths[nlayers]; j++) y[j] = out_norms ? x1[j] * out_norms[j] : x1[j];
+        }
+        free(x1); free(x2);
+    }
+}
+
+/* The same native loop nest with the weights held as the Fortran code holds them, A(out, in)
+ * column-major, i.e. Wt[l] is [n_in][n_out] with the output index contiguous, so the inner j loop
+ * is unit stride exactly as in Layer_apply (mom6_zb/fwd_native_zb.f90:37-41).  Same arithmetic and
+ * order as orc_mlp_native (bit-identical for ReLU networks; the test suite checks that), plus
+ * LeakyReLU for the ClimSim-shaped network.  This is the CPU baseline the benchmark times:
+ * columns in parallel over OpenMP threads, one column through all layers at a time. */
+void orc_mlp_native_t(int nlayers, const int* widths, const float* const* Wt, const float* const* b,
+                      const int* act, const float* alpha, const float* in_norms, const float* out_norms,
+                      long rows, const float* X, float* Y)
+{
+    int maxw = 0;
+    for (int l = 0; l <= nlayers; l++) if (widths[l] > maxw) maxw = widths[l];
+#pragma omp parallel if (rows > 64)
+    {
+        float* x1 = (float*)malloc(sizeof(float) * maxw);
+        float* x2 = (float*)malloc(sizeof(float) * maxw);
+#pragma omp for schedule(static)
+        for (long r = 0; r < rows; r++) {
+            const float* x = X + (size_t)r * widths[0];
+            for (int i = 0; i < widths[0]; i++) x1[i] = in_norms ? x[i] / in_norms[i] : x[i];
+            for (int l = 0; l < nlayers; l++) {
+                const int ni = widths[l], no = widths[l + 1];
+                for (int j = 0; j < no; j++) x2[j] = 0.0f;
+                for (int i = 0; i < ni; i++) {
+                    const float xi = x1[i];
+                    const float* w = Wt[l] + (size_t)i * no;
+                    for (int j = 0; j < no; j++) x2[j] = x2[j] + (xi * w[j]);
+                }
+                for (int j = 0; j < no; j++) {
+                    float v = x2[j] + b[l][j];
+                    if (act[l] == 1) v = v > 0.0f ? v : 0.0f;
+                    else if (act[l] == 2) v = v > 0.0f ? v : alpha[l] * v;
+                    x2[j] = v;
                 }
                 float* t = x1; x1 = x2; x2 = t;
             }

@@ -210,6 +210,23 @@ def mlp_native(Ws, bs, X, in_norms=None, out_norms=None):
     return Y
 
 
+def mlp_native_t(Ws, bs, acts, X, alphas=None, in_norms=None, out_norms=None):
+    """Native loop nest on Fortran-ordered weights (the timed CPU baseline); see orc_mlp_native_t."""
+    widths, kw, kb, wp, bp, wid = _mlp_args(Ws, bs)
+    Wt = [np.ascontiguousarray(w.T) for w in kw]
+    wtp = (f32p * len(Ws))(*[w.ctypes.data_as(f32p) for w in Wt])
+    X, xp = _f(X)
+    rows = X.shape[0]
+    Y = np.empty((rows, widths[-1]), dtype=np.float32)
+    act = (C.c_int * len(Ws))(*[a if isinstance(a, int) else ACT[a] for a in acts])
+    al = np.ascontiguousarray(alphas if alphas is not None else np.zeros(len(Ws)), dtype=np.float32)
+    inn = _f(in_norms) if in_norms is not None else (None, None)
+    outn = _f(out_norms) if out_norms is not None else (None, None)
+    lib().orc_mlp_native_t(len(Ws), wid, wtp, bp, act, al.ctypes.data_as(f32p), inn[1], outn[1], C.c_long(rows), xp,
+                           Y.ctypes.data_as(f32p))
+    return Y
+
+
 ACT = {None: 0, "none": 0, "relu": 1, "leaky": 2}
 
 

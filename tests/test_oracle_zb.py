@@ -99,3 +99,20 @@ def test_expression_compiler_order():
     ins, n, consts = O.compile_exprs(["(tv / (S0 + 1.000000e-30f))"])
     assert n == 2 and (ins[0].op, ins[0].a, ins[0].b) == (0, 1, 16) and (ins[1].op, ins[1].a, ins[1].b) == (3, 0, 32)
     assert consts[0] == np.float32(1e-30)
+
+
+def test_native_t_is_the_same_arithmetic(zb):
+    """The Fortran-ordered-weights variant timed as the CPU baseline equals the pinned native
+    forward bit for bit on the ZB network, and the fp64 chain within rounding on a LeakyReLU net."""
+    W = zb["W"]
+    X = O.stencil_gather(__import__("json").load(open(os.path.join(os.path.dirname(__file__), "golden", "zb_gather.json"))),
+                         [zb["P"]["sh_xy_h"], zb["F"]["sh_xx"], zb["P"]["vort_xy_h"], zb["P"]["norm_h"]], 4736, 1, 3, 3, 64)
+    a = O.mlp_native(zb["Ws"], zb["bs"], X, W["in_norms"], W["out_norms"])
+    b = O.mlp_native_t(zb["Ws"], zb["bs"], ["relu", None], X, in_norms=W["in_norms"], out_norms=W["out_norms"])
+    assert bits_equal(a, b)
+    rng = np.random.default_rng(1)
+    Ws = [rng.standard_normal((40, 30)).astype(np.float32) / 5, rng.standard_normal((10, 40)).astype(np.float32) / 6]
+    bs = [rng.standard_normal(40).astype(np.float32), rng.standard_normal(10).astype(np.float32)]
+    Xs = rng.standard_normal((100, 30)).astype(np.float32)
+    assert maxrel(O.mlp_native_t(Ws, bs, ["leaky", None], Xs, alphas=[0.15, 0]),
+                  O.mlp_f64(Ws, bs, ["leaky", None], Xs, alphas=[0.15, 0])) < 2e-6
