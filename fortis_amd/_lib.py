@@ -53,6 +53,7 @@ PROTOTYPES = {
     "fortis_pool_set_allocator": (None, [vp, vp]), "fortis_device_info": (i, [C.c_char_p, i, C.POINTER(l)]),
     # fortis_step.h: plan
     "fortis_plan_create": (vp, []), "fortis_plan_destroy": (None, [vp]), "fortis_plan_tensor": (i, [vp, l]),
+    "fortis_plan_view": (i, [vp, i, l, l]),
     "fortis_plan_linear": (i, [vp, i, i, vp, vp, l, l, l, i, f]),
     "fortis_plan_scale": (i, [vp, i, i, vp, l, l, i]),
     "fortis_plan_mask_relu": (i, [vp, i, i, l, l, l]),

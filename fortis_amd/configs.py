@@ -144,3 +144,128 @@ def climsim_plan(case, boundary=True):
     return p.finalize(t_in, cur)
 
 
+
+
+# ---------------------------------------------------------------------------------------------
+def _conv_bn(rw, rb, ci, co):
+    return dict(W=_w(rw, co, ci, 3, 3), b=np.zeros(co, np.float32),
+                bn=(np.ones(co, np.float32), np.zeros(co, np.float32), (0.1 * rb.standard_normal(co)).astype(np.float32),
+                    rb.uniform(0.5, 1.5, co).astype(np.float32)))
+
+
+def unet(H=256, cin=4, chans=(32, 64, 128, 256), cout=4):
+    """Config 4: x 1 x cin x H x H ~ N(0,1).  Encoder: (conv3x3 + BN + ReLU) x2 at chans[:-1], 2x2 maxpool
+    after each; bottleneck (conv3x3 + BN + ReLU) x2 at chans[-1]; decoder: 2x2 stride-2 transposed conv,
+    concat [skip, up], (conv3x3 + BN + ReLU) x2; final 1x1 conv to cout.  BN eval: running mean N(0, 0.1),
+    var U(0.5, 1.5), gamma 1, beta 0, eps 1e-5; conv biases 0."""
+    rw, ri, rb = np.random.default_rng(0), np.random.default_rng(1), np.random.default_rng(3)
+    x = ri.standard_normal((cin, H, H)).astype(np.float32)
+    enc, ci = [], cin
+    for c in chans[:-1]:
+        enc.append([_conv_bn(rw, rb, ci, c), _conv_bn(rw, rb, c, c)])
+        ci = c
+    bott = [_conv_bn(rw, rb, ci, chans[-1]), _conv_bn(rw, rb, chans[-1], chans[-1])]
+    dec, ci = [], chans[-1]
+    for c in reversed(chans[:-1]):
+        up = dict(W=(rw.standard_normal((ci, c, 2, 2)) / np.sqrt(ci)).astype(np.float32), b=np.zeros(c, np.float32))
+        dec.append(dict(up=up, convs=[_conv_bn(rw, rb, 2 * c, c), _conv_bn(rw, rb, c, c)]))
+        ci = c
+    final = dict(W=_w(rw, cout, ci, 1, 1), b=np.zeros(cout, np.float32))
+    macs, h, cp = 0, H, cin
+    for c in chans[:-1]:
+        macs += h * h * 9 * (cp * c + c * c)
+        cp, h = c, h // 2
+    macs += h * h * 9 * (cp * chans[-1] + chans[-1] ** 2)
+    cp = chans[-1]
+    for c in reversed(chans[:-1]):
+        h *= 2
+        macs += h * h * cp * c + h * h * 9 * (2 * c * c + c * c)
+        cp = c
+    macs += h * h * cp * cout
+    return dict(name="unet", x=x, enc=enc, bott=bott, dec=dec, final=final, H=H, cin=cin, chans=list(chans), cout=cout,
+                flops=2 * macs, voxels=H * H)
+
+
+def unet_plan(case):
+    H, chans = case["H"], case["chans"]
+    p = P.Plan()
+    t_in = p.tensor(case["cin"] * H * H)
+    # one buffer per decoder level holds [skip | up]; the encoder's last conv of the level writes the
+    # first window, the transposed conv writes the second: the concatenation costs no copy
+    cat, skip_v, up_v = {}, {}, {}
+    for lvl, c in enumerate(chans[:-1]):
+        hh = H >> lvl
+        cat[lvl] = p.tensor(2 * c * hh * hh)
+        skip_v[lvl] = p.view(cat[lvl], 0, c * hh * hh)
+        up_v[lvl] = p.view(cat[lvl], c * hh * hh, c * hh * hh)
+
+    def conv(src, dst, cv, ci, h):
+        p.conv2d(src, dst, cv["W"], cv["b"], ci, h, h, 1, 1, "relu", 0.0, cv["bn"], 1e-5)
+
+    cur, ci, h = t_in, case["cin"], H
+    for lvl, (blk, c) in enumerate(zip(case["enc"], chans[:-1])):
+        t = p.tensor(c * h * h)
+        conv(cur, t, blk[0], ci, h)
+        conv(t, skip_v[lvl], blk[1], c, h)
+        t = p.tensor(c * (h // 2) * (h // 2))
+        p.maxpool2d(skip_v[lvl], t, c, h, h, 2)
+        cur, ci, h = t, c, h // 2
+    cb = chans[-1]
+    t1, t2 = p.tensor(cb * h * h), p.tensor(cb * h * h)
+    conv(cur, t1, case["bott"][0], ci, h)
+    conv(t1, t2, case["bott"][1], cb, h)
+    cur, ci = t2, cb
+    for lvl, d in zip(reversed(range(len(chans) - 1)), case["dec"]):
+        c = chans[lvl]
+        p.convt2d(cur, up_v[lvl], d["up"]["W"], d["up"]["b"], ci, h, h, 2, 0, 0, None, 0.0)
+        h *= 2
+        t1, t2 = p.tensor(c * h * h), p.tensor(c * h * h)
+        conv(cat[lvl], t1, d["convs"][0], 2 * c, h)
+        conv(t1, t2, d["convs"][1], c, h)
+        cur, ci = t2, c
+    t_out = p.tensor(case["cout"] * h * h)
+    p.conv2d(cur, t_out, case["final"]["W"], case["final"]["b"], ci, h, h, 1, 0, None, 0.0)
+    return p.finalize(t_in, t_out)
+
+
+def tsrgan(D=33, cin=3, ch=64, nblocks=8, cout=3, alpha=0.2):
+    """Config 5: x NDHWC 1 x D^3 x 3 ~ U(0,1), permuted to NCDHW inside the step; conv3d 3^3 3->64 +
+    LeakyReLU(0.2); 8 residual blocks (conv 64->64, ReLU, conv 64->64, + skip); nearest x2 upsample;
+    conv 64->64 + LeakyReLU(0.2); conv 64->3; output permuted back to NDHWC.  All pad 1, stride 1, bias 0."""
+    rw, ri = np.random.default_rng(0), np.random.default_rng(1)
+    x = ri.uniform(0, 1, (D, D, D, cin)).astype(np.float32)
+    z = lambda n: np.zeros(n, np.float32)
+    head = dict(W=_w(rw, ch, cin, 3, 3, 3), b=z(ch))
+    blocks = [dict(W1=_w(rw, ch, ch, 3, 3, 3), b1=z(ch), W2=_w(rw, ch, ch, 3, 3, 3), b2=z(ch)) for _ in range(nblocks)]
+    upc = dict(W=_w(rw, ch, ch, 3, 3, 3), b=z(ch))
+    tail = dict(W=_w(rw, cout, ch, 3, 3, 3), b=z(cout))
+    v1, v2 = D ** 3, (2 * D) ** 3
+    macs = v1 * 27 * (cin * ch + 2 * nblocks * ch * ch) + v2 * 27 * (ch * ch + ch * cout)
+    return dict(name="tsrgan", x=x, head=head, blocks=blocks, upc=upc, tail=tail, D=D, cin=cin, ch=ch, cout=cout,
+                alpha=alpha, flops=2 * macs, voxels=v2)
+
+
+def tsrgan_plan(case):
+    D, ch, cin, cout, a = case["D"], case["ch"], case["cin"], case["cout"], case["alpha"]
+    v1, D2 = D ** 3, 2 * D
+    v2 = D2 ** 3
+    p = P.Plan()
+    t_in = p.tensor(v1 * cin)
+    t = p.tensor(v1 * cin)
+    p.permute(t_in, t, cin, v1, True)
+    cur = p.tensor(ch * v1)
+    p.conv3d(t, cur, case["head"]["W"], case["head"]["b"], cin, D, D, D, 1, "leaky", a)
+    for blk in case["blocks"]:
+        h1, out = p.tensor(ch * v1), p.tensor(ch * v1)
+        p.conv3d(cur, h1, blk["W1"], blk["b1"], ch, D, D, D, 1, "relu", 0.0)
+        p.conv3d(h1, out, blk["W2"], blk["b2"], ch, D, D, D, 1, None, 0.0, res=cur)
+        cur = out
+    up = p.tensor(ch * v2)
+    p.upsample(cur, up, ch, D, D, D, 2, 3)
+    c1 = p.tensor(ch * v2)
+    p.conv3d(up, c1, case["upc"]["W"], case["upc"]["b"], ch, D2, D2, D2, 1, "leaky", a)
+    c2 = p.tensor(cout * v2)
+    p.conv3d(c1, c2, case["tail"]["W"], case["tail"]["b"], ch, D2, D2, D2, 1, None, 0.0)
+    t_out = p.tensor(cout * v2)
+    p.permute(c2, t_out, cout, v2, False)
+    return p.finalize(t_in, t_out)

@@ -42,6 +42,8 @@ struct Exec {
 
 struct fortis_plan {
     std::vector<long> tbytes;
+    std::vector<int> view_of;   // -1: owns a buffer; otherwise the tensor this one is a window of
+    std::vector<long> view_off; // byte offset of the window
     std::vector<void*> tptr;
     std::vector<Op> ops;
     std::vector<Exec> exec;
@@ -76,13 +78,27 @@ void fortis_plan_destroy(fortis_plan* p)
 {
     if (!p) return;
     for (void* d : p->owned) HIP_OK(hipFree(d));
-    for (void* t : p->tptr) fortis_free(t);
+    for (size_t t = 0; t < p->tptr.size(); t++) if (p->view_of[t] < 0) fortis_free(p->tptr[t]);
     delete p;
 }
 int fortis_plan_tensor(fortis_plan* p, long nbytes)
 {
     if (!p || p->finalized || nbytes <= 0) return -1;
     p->tbytes.push_back(nbytes);
+    p->view_of.push_back(-1);
+    p->view_off.push_back(0);
+    return (int)p->tbytes.size() - 1;
+}
+int fortis_plan_view(fortis_plan* p, int base, long byte_offset, long nbytes)
+{
+    if (!p || p->finalized || base < 0 || base >= (int)p->tbytes.size() || byte_offset < 0 || nbytes <= 0 ||
+        byte_offset % 16 || byte_offset + nbytes > p->tbytes[base]) {
+        fprintf(stderr, "fortis_plan_view: window outside tensor %d or not 16-byte aligned\n", base);
+        return -1;
+    }
+    p->tbytes.push_back(nbytes);
+    p->view_of.push_back(p->view_of[base] >= 0 ? p->view_of[base] : base);
+    p->view_off.push_back(p->view_off[base] + byte_offset);
     return (int)p->tbytes.size() - 1;
 }
 
@@ -308,8 +324,9 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
     if (p->ops.empty()) return bad("finalize: empty plan");
     p->in_t = in_t; p->out_t = out_t;
     (void)fortis_stream_get();
-    for (long nb : p->tbytes) {
-        void* d = fortis_alloc(nb);
+    for (size_t t = 0; t < p->tbytes.size(); t++) {
+        if (p->view_of[t] >= 0) { p->tptr.push_back((char*)p->tptr[p->view_of[t]] + p->view_off[t]); continue; }
+        void* d = fortis_alloc(p->tbytes[t]);
         if (!d) return bad("finalize: out of device memory");
         p->tptr.push_back(d);
     }

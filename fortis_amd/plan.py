@@ -50,6 +50,12 @@ class Plan:
             raise ValueError("fortis_plan_tensor failed")
         return t
 
+    def view(self, base, elem_offset, nelem, esz=4):
+        t = self._L.fortis_plan_view(self._p, base, int(elem_offset) * esz, int(nelem) * esz)
+        if t < 0:
+            raise ValueError("fortis_plan_view failed (see stderr)")
+        return t
+
     def linear(self, src, dst, W, bias, B, act=None, alpha=0.0):
         W = _f32(W)
         N, K = W.shape

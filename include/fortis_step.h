@@ -35,6 +35,11 @@ void         fortis_plan_destroy(fortis_plan* p);
 /* Declares an activation tensor of `nbytes` bytes; returns its id (>= 0).  Tensors are device
  * buffers taken from fortis_alloc at finalize. */
 int  fortis_plan_tensor(fortis_plan* p, long nbytes);
+/* Declares a window [byte_offset, byte_offset + nbytes) of tensor `base` as a tensor of its own
+ * (16-byte aligned).  A channel concatenation is then two producers writing the two windows of
+ * one buffer (what the reference does with memref.copy into a subview,
+ * compiler/FortisFuse.cpp:547-551, 122-133) and costs no copy. */
+int  fortis_plan_view(fortis_plan* p, int base, long byte_offset, long nbytes);
 
 /* dst[B][N] = act(src[B][K] . W[N][K]^T + bias[N]).  W, bias are host pointers, copied to the
  * device at finalize (the role of setup() uploading w<i>, driver/fortis_shim.py:67-72).  bias may
