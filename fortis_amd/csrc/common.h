@@ -95,6 +95,11 @@ int fortis_launch_convt2d(const float* x, const float* w, float* y, long C, long
 int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long D, long H, long Wd, long F,
                          long KD, long KH, long KW, long Do, long Ho, long Wo, long pd, long ph, long pw,
                          const ConvEpi& e, hipStream_t s);
+// MFMA implicit-GEMM path (conv_mfma.hip).  kind 0: KD x KS x KS conv, pad KS/2, stride 1; kind 1: 2x2
+// stride-2 transposed conv.  wp: weights packed by fortis_conv_mfma_pack.  -1: shape not taken.
+float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats);
+int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, long D, long H, long Wd, long F, int KD,
+                            int KS, int kind, const ConvEpi& e, hipStream_t s);
 void fortis_launch_maxpool2d(const float* x, float* y, long C, long H, long Wd, long k, hipStream_t s);
 void fortis_launch_upsample(const float* x, float* y, long C, long D, long H, long Wd, long sfac, int nd, hipStream_t s);
 void fortis_launch_concat_copy(const float* x, float* y, long C, long S, long coff, hipStream_t s);

@@ -1,0 +1,231 @@
+// Implicit-GEMM convolution on the fp32 matrix cores (v_mfma_f32_32x32x2f32), stride 1, N = 1:
+// conv3d 3x3x3 pad 1, conv2d 3x3 pad 1, conv 1x1, and the 2x2 stride-2 transposed conv (as a 1x1
+// conv with 4F output channels whose epilogue scatters to (2y+a, 2x+b)).  Bias / folded
+// BatchNorm / activation / residual are applied in the epilogue.
+//
+// Replaces k_conv3d_direct3 (runtime/fortis_fft.cu:148-201: scalar FMA from shared memory, 32
+// accumulators per thread) and the cuDNN calls of runtime/fortis_rt.c:108-156.
+//
+// GEMM view: rows = output channels (MFMA A operand = weights), columns = output positions (B operand
+// = input patches), k = (input channel, tap).  One MFMA step multiplies two input channels (the two
+// lane halves) at one tap.
+// Positions are linearised inside one z-plane with pitch P = W + 1: m = y*P + x.  On the virtual
+// zero-padded plane of the same pitch (the right pad of a row is the left pad of the next), tap
+// (kh, kw) of position m is element m + kh*P + kw: a lane-independent offset.  A workgroup therefore
+// stages, per input channel and per kd, ONE contiguous run of MT + 2P + 2 virtual elements into LDS
+// (zero-filled outside the image), and every B operand is a single ds_read at lane base + constant.
+// Weights are re-packed once at plan time in exactly the order the kernel consumes them, so their
+// staging is a straight 16-byte copy.  Both are double buffered through registers.
+#include "common.h"
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+#define CM_THREADS 256
+#define CM_CC 4        // input channels per staged chunk (two MFMA channel pairs)
+#define CM_FT 64       // output channels per workgroup
+#define CM_NXMAX 16    // staged input elements per thread per chunk, at most
+
+struct ConvMShape {
+    int C, D, H, W, F;         // F = output channels of the GEMM (4x the real ones in transposed mode)
+    int P, plane, tiles, nchunks, R;
+    int mode;                  // 0: convolution, 1: 2x2 stride-2 transposed conv scatter
+};
+
+template <int KD, int KS, int MT>
+__global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
+                                                               float* __restrict__ y, ConvMShape s, ConvEpi e)
+{
+    constexpr int T = KD * KS * KS;
+    constexpr int WCH = 2 * T * 2 * CM_FT;                       // floats of packed weights per chunk
+    constexpr int NW = (WCH / 4 + CM_THREADS - 1) / CM_THREADS;  // float4 per thread
+    constexpr int NMT = MT / 64;                                 // m-tiles per wave
+    constexpr int PADK = KS / 2;
+    extern __shared__ float4 smem4[];
+    float* sW = (float*)smem4;                                    // [2][WCH]
+    float* sX = sW + 2 * WCH;                                     // [2][CM_CC * KD * R]
+    const int XCH = CM_CC * KD * s.R;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int z = blockIdx.x / s.tiles, tile = blockIdx.x - z * s.tiles;
+    const int fg = blockIdx.y;
+    const int m0 = tile * MT;
+    const long HW = (long)s.H * s.W, chan = (long)s.D * HW;
+
+    // per-thread staging map of the input run (same for every chunk): global offset inside a 4-channel group
+    int goff[CM_NXMAX];
+    int gch[CM_NXMAX];
+#pragma unroll
+    for (int i = 0; i < CM_NXMAX; i++) {
+        const int el = tid + i * CM_THREADS;
+        goff[i] = -1;
+        gch[i] = 0;
+        if (el < XCH) {
+            const int c = el / (KD * s.R), rem = el - c * (KD * s.R), kd = rem / s.R, r = rem - kd * s.R;
+            const int v = m0 + r, yp = v / s.P, xp = v - yp * s.P;
+            const int zz = z + kd - (KD / 2), yy = yp - PADK, xx = xp - PADK;
+            gch[i] = c;
+            if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W)
+                goff[i] = (int)(c * chan + zz * HW + (long)yy * s.W + xx);
+        }
+    }
+
+    float4 rw[NW];
+    float rx[CM_NXMAX];
+    auto load_chunk = [&](int ch) {
+        const float4* wsrc = (const float4*)(wp + ((long)fg * s.nchunks + ch) * WCH);
+#pragma unroll
+        for (int i = 0; i < NW; i++) {
+            const int f4 = tid + i * CM_THREADS;
+            if (f4 < WCH / 4) rw[i] = wsrc[f4];
+        }
+        const float* xsrc = x + (long)ch * CM_CC * chan;
+#pragma unroll
+        for (int i = 0; i < CM_NXMAX; i++)
+            rx[i] = (goff[i] >= 0 && ch * CM_CC + gch[i] < s.C) ? xsrc[goff[i]] : 0.f;
+    };
+    auto store_chunk = [&](int buf) {
+        float4* wdst = (float4*)(sW + buf * WCH);
+#pragma unroll
+        for (int i = 0; i < NW; i++) {
+            const int f4 = tid + i * CM_THREADS;
+            if (f4 < WCH / 4) wdst[f4] = rw[i];
+        }
+        float* xdst = sX + buf * XCH;
+#pragma unroll
+        for (int i = 0; i < CM_NXMAX; i++) {
+            const int el = tid + i * CM_THREADS;
+            if (el < XCH) xdst[el] = rx[i];
+        }
+    };
+
+    const int ft = wave & 1, mt0 = (wave >> 1) * NMT;
+    const int wbase = (lane >> 5) * CM_FT + ft * 32 + (lane & 31);
+    const int xbase = (lane >> 5) * KD * s.R + mt0 * 32 + (lane & 31);
+    v16f acc[NMT];
+#pragma unroll
+    for (int j = 0; j < NMT; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+
+    load_chunk(0);
+    store_chunk(0);
+    __syncthreads();
+    for (int ch = 0; ch < s.nchunks; ch++) {
+        const int buf = ch & 1;
+        if (ch + 1 < s.nchunks) load_chunk(ch + 1);
+        const float* w = sW + buf * WCH + wbase;
+        const float* xs = sX + buf * XCH + xbase;
+#pragma unroll
+        for (int cp = 0; cp < 2; cp++)
+#pragma unroll
+            for (int kd = 0; kd < KD; kd++)
+#pragma unroll
+                for (int kh = 0; kh < KS; kh++)
+#pragma unroll
+                    for (int kw = 0; kw < KS; kw++) {
+                        const int tap = (kd * KS + kh) * KS + kw;
+                        const float a = w[(cp * T + tap) * 2 * CM_FT];
+                        const int xoff = (2 * cp * KD + kd) * s.R + kh * s.P + kw;
+#pragma unroll
+                        for (int j = 0; j < NMT; j++)
+                            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, xs[j * 32 + xoff], acc[j], 0, 0, 0);
+                    }
+        if (ch + 1 < s.nchunks) store_chunk(buf ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: a lane holds one position and 16 output channels per m-tile
+    const long ospatial = s.mode ? 4 * chan : chan;
+#pragma unroll
+    for (int j = 0; j < NMT; j++) {
+        const int m = m0 + (mt0 + j) * 32 + (lane & 31);
+        if (m >= s.plane) continue;
+        const int yy = m / s.P, xx = m - yy * s.P;
+        if (xx >= s.W) continue;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int f = fg * CM_FT + ft * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (f >= s.F) continue;
+            int fo = f;
+            long opos = ((long)z * s.H + yy) * s.W + xx;
+            if (s.mode) {
+                fo = f >> 2;
+                opos = (long)(2 * yy + ((f >> 1) & 1)) * (2 * s.W) + 2 * xx + (f & 1);
+            }
+            float v = acc[j][r];
+            if (e.scale) v = v * e.scale[fo];
+            if (e.shift) v = v + e.shift[fo];
+            if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
+            else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
+            if (e.res) v = v + e.res[fo * ospatial + opos];
+            y[fo * ospatial + opos] = v;
+        }
+    }
+}
+
+// ---- host side ---------------------------------------------------------------------------------------
+// Packs conv weights W[F][C][T] (T taps, row-major) into the kernel's order
+//   [F/64][ceil(C/4)][channel pair 2][tap T][half 2][64 channels], zero padded.
+// Transposed 2x2 conv: W is [C][F][2][2]; GEMM channel f' = f*4 + a*2 + b.
+float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats)
+{
+    const long Fg = transposed ? 4 * F : F;
+    const long nfg = cdiv(Fg, CM_FT), nch = cdiv(C, CM_CC);
+    const long wch = 2L * T * 2 * CM_FT;
+    const long n = nfg * nch * wch;
+    float* h = (float*)calloc(n, sizeof(float));
+    for (long fgi = 0; fgi < nfg; fgi++)
+        for (long ch = 0; ch < nch; ch++)
+            for (int cp = 0; cp < 2; cp++)
+                for (int t = 0; t < T; t++)
+                    for (int hh = 0; hh < 2; hh++)
+                        for (int fl = 0; fl < CM_FT; fl++) {
+                            const long f = fgi * CM_FT + fl, c = ch * CM_CC + cp * 2 + hh;
+                            if (f >= Fg || c >= C) continue;
+                            const float v = transposed ? W[(c * F + (f >> 2)) * 4 + (f & 3)] : W[(f * C + c) * T + t];
+                            h[((fgi * nch + ch) * 2 + cp) * T * 2 * CM_FT + ((long)t * 2 + hh) * CM_FT + fl] = v;
+                        }
+    float* d = nullptr;
+    HIP_OK(hipMalloc((void**)&d, n * sizeof(float)));
+    HIP_OK(hipMemcpy(d, h, n * sizeof(float), hipMemcpyHostToDevice));
+    free(h);
+    if (nfloats) *nfloats = n;
+    return d;
+}
+
+template <int KD, int KS, int MT>
+static int launch(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
+{
+    constexpr int T = KD * KS * KS;
+    s.P = KS == 3 ? s.W + 1 : s.W;
+    s.plane = s.H * s.P;
+    s.tiles = (int)cdiv(s.plane, MT);
+    s.nchunks = (int)cdiv(s.C, CM_CC);
+    s.R = MT + (KS == 3 ? 2 * s.P + 2 : 0);
+    if ((long)CM_CC * KD * s.R > (long)CM_THREADS * CM_NXMAX) return -1;     // run too long to stage
+    const size_t shmem = (size_t)2 * (2 * T * 2 * CM_FT + CM_CC * KD * s.R) * sizeof(float);
+    if (shmem > 160 * 1024) return -1;
+    static size_t attr = 0;
+    if (shmem > attr) {
+        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        attr = shmem;
+    }
+    dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, CM_FT));
+    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+    HIP_OK(hipGetLastError());
+    return 0;
+}
+
+// kind: 0 conv (KD x KS x KS, pad KS/2), 1 transposed 2x2 stride 2.  Returns -1 if the shape is not
+// one the MFMA kernel takes (the caller then uses the direct kernel).
+int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, long D, long H, long Wd, long F, int KD,
+                            int KS, int kind, const ConvEpi& e, hipStream_t st)
+{
+    if (C * D * H * Wd >= 2147483647L || F * D * H * Wd * (kind ? 4 : 1) >= 2147483647L) return -1;
+    ConvMShape s = { (int)C, (int)D, (int)H, (int)Wd, (int)(kind ? 4 * F : F), 0, 0, 0, 0, 0, kind };
+    if (kind == 1) return D == 1 ? launch<1, 1, 256>(x, wp, y, s, e, st) : -1;
+    if (KD == 3 && KS == 3) return launch<3, 3, 128>(x, wp, y, s, e, st);
+    if (KD == 1 && KS == 3) return launch<1, 3, 256>(x, wp, y, s, e, st);
+    if (KD == 1 && KS == 1) return launch<1, 1, 256>(x, wp, y, s, e, st);
+    return -1;
+}

@@ -38,6 +38,7 @@ struct Exec {
     const void *p0 = nullptr, *p1 = nullptr, *p2 = nullptr;
     const Op* op = nullptr;
     ConvEpi epi = { nullptr, nullptr, 0, 0.f, nullptr };
+    const float* Wmfma = nullptr;   // weights packed for the MFMA implicit-GEMM kernel, when the shape qualifies
 };
 
 struct fortis_plan {
@@ -392,6 +393,20 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                 ex.epi.scale = scale.empty() ? nullptr : (const float*)upload(p, scale.data(), scale.size() * 4);
                 ex.epi.shift = shift.empty() ? nullptr : (const float*)upload(p, shift.data(), shift.size() * 4);
                 ex.epi.act = o.act; ex.epi.alpha = o.alpha;
+                // matrix-core path for the shapes it takes; narrow outputs stay on the direct kernel
+                static int direct_only = -1;
+                if (direct_only < 0) direct_only = getenv("FORTIS_CONV_DIRECT") != 0;
+                const bool wide = o.F >= 16;
+                bool ok = false;
+                int T = 0, tr = 0;
+                if (o.kind == OP_CONV2D) { ok = o.stride == 1 && o.KH == o.KW && (o.KH == 1 || o.KH == 3) && o.pad == o.KH / 2; T = (int)(o.KH * o.KW); }
+                else if (o.kind == OP_CONV3D) { ok = o.KD == 3 && o.pad == 1; T = 27; }
+                else { ok = o.KH == 2 && o.KW == 2 && o.stride == 2 && o.pad == 0 && o.opad == 0; T = 1; tr = 1; }
+                if (ok && wide && !direct_only) {
+                    float* wp = fortis_conv_mfma_pack(o.w.data(), o.F, o.C, T, tr, nullptr);
+                    p->owned.push_back(wp);
+                    ex.Wmfma = wp;
+                }
                 break;
             }
             case OP_MAXPOOL: ex.kind = EX_MAXPOOL; break;
@@ -438,22 +453,28 @@ void fortis_plan_run(fortis_plan* p)
             case EX_POST: fortis_launch_boundary_post(src, p->tptr[e.dst], e.rows, e.N, e.p0, e.flag, s); break;
             case EX_CONV2D: {
                 const long Ho = (o->H + 2 * o->pad - o->KH) / o->stride + 1, Wo = (o->W + 2 * o->pad - o->KW) / o->stride + 1;
-                rc = fortis_launch_conv2d(src, e.W, dst, o->C, o->H, o->W, o->F, o->KH, o->KW, Ho, Wo, o->stride, o->stride,
-                                          o->pad, o->pad, e.epi, o->coff, o->ctot, s);
+                rc = e.Wmfma ? fortis_launch_conv_mfma(src, e.Wmfma, dst + o->coff * Ho * Wo, o->C, 1, o->H, o->W, o->F, 1, (int)o->KH, 0, e.epi, s) : -1;
+                if (rc != 0)
+                    rc = fortis_launch_conv2d(src, e.W, dst, o->C, o->H, o->W, o->F, o->KH, o->KW, Ho, Wo, o->stride, o->stride,
+                                              o->pad, o->pad, e.epi, o->coff, o->ctot, s);
                 break;
             }
             case EX_CONVT2D: {
                 const long Ho = (o->H - 1) * o->stride - 2 * o->pad + o->KH + o->opad, Wo = (o->W - 1) * o->stride - 2 * o->pad + o->KW + o->opad;
-                rc = fortis_launch_convt2d(src, e.W, dst, o->C, o->H, o->W, o->F, o->KH, o->KW, Ho, Wo, o->stride, o->pad, e.epi,
-                                           o->coff, o->ctot, s);
+                rc = e.Wmfma ? fortis_launch_conv_mfma(src, e.Wmfma, dst + o->coff * Ho * Wo, o->C, 1, o->H, o->W, o->F, 1, 1, 1, e.epi, s) : -1;
+                if (rc != 0)
+                    rc = fortis_launch_convt2d(src, e.W, dst, o->C, o->H, o->W, o->F, o->KH, o->KW, Ho, Wo, o->stride, o->pad, e.epi,
+                                               o->coff, o->ctot, s);
                 break;
             }
             case EX_CONV3D: {
                 ConvEpi epi = e.epi;
                 epi.res = e.res >= 0 ? (const float*)p->tptr[e.res] : nullptr;
                 const long Do = o->D + 2 * o->pad - o->KD + 1, Ho = o->H + 2 * o->pad - o->KH + 1, Wo = o->W + 2 * o->pad - o->KW + 1;
-                rc = fortis_launch_conv3d(src, e.W, dst, o->C, o->D, o->H, o->W, o->F, o->KD, o->KH, o->KW, Do, Ho, Wo, o->pad,
-                                          o->pad, o->pad, epi, s);
+                rc = e.Wmfma ? fortis_launch_conv_mfma(src, e.Wmfma, dst, o->C, o->D, o->H, o->W, o->F, 3, 3, 0, epi, s) : -1;
+                if (rc != 0)
+                    rc = fortis_launch_conv3d(src, e.W, dst, o->C, o->D, o->H, o->W, o->F, o->KD, o->KH, o->KW, Do, Ho, Wo, o->pad,
+                                              o->pad, o->pad, epi, s);
                 break;
             }
             case EX_MAXPOOL: fortis_launch_maxpool2d(src, dst, o->C, o->H, o->W, o->KH, s); break;

@@ -6,8 +6,22 @@ import torch
 import torch.nn.functional as TF
 
 
+_DT = [torch.float64]
+
+
 def _t(a):
-    return torch.tensor(np.asarray(a), dtype=torch.float64)
+    return torch.tensor(np.asarray(a), dtype=_DT[0])
+
+
+def _with_dtype(fn):
+    def wrapped(case, dtype=torch.float64):
+        _DT[0] = dtype
+        try:
+            with torch.no_grad():
+                return fn(case)
+        finally:
+            _DT[0] = torch.float64
+    return wrapped
 
 
 def _conv_bn_relu(x, cv):
@@ -16,6 +30,7 @@ def _conv_bn_relu(x, cv):
     return torch.relu(TF.batch_norm(y, m, v, g, b, False, 0.0, 1e-5))
 
 
+@_with_dtype
 def unet_ref(case):
     x = _t(case["x"])[None]
     skips = []
@@ -31,6 +46,7 @@ def unet_ref(case):
     return TF.conv2d(x, _t(case["final"]["W"]), _t(case["final"]["b"]))[0].numpy()
 
 
+@_with_dtype
 def tsrgan_ref(case):
     a = case["alpha"]
     x = _t(case["x"]).permute(3, 0, 1, 2)[None]                      # NDHWC -> NCDHW
