@@ -28,24 +28,25 @@ int fortis_launch_gemm(const float* A, const float* W, const float* bias, float*
 #define FORTIS_CHAIN_MAX_LAYERS 8
 #define FORTIS_CHAIN_MAX_WIDTH 256
 struct ChainLayer {
-    const float* Wp;    // packed weights: [Np/32][Kp/8][64 lanes][4]
-    const float* bias;  // [Np], zero padded
-    int K, N, Kp, Np;
+    int K, N, Kp, Np;   // real and padded (to 16) widths
+    int woff, boff;     // float offsets of the packed weights / bias inside the blob
     int act;
     float alpha;
 };
 struct ChainDesc {
     int nlayers;
     ChainLayer L[FORTIS_CHAIN_MAX_LAYERS];
+    const float* wall;     // device blob: every layer's packed weights and zero-padded bias
+    int wfloats;           // its length in floats (multiple of 4)
     const float* in_div;   // x / in_div[c] before layer 0, or null
     const float* out_mul;  // y * out_mul[c] after the last layer, or null
     int mask_tail;         // ReLU on the last mask_tail outputs
     int ld;                // LDS row pitch in floats
 };
-// Packs W[N][K] for the chain kernel into a freshly allocated device buffer (stream-ordered).
-float* fortis_chain_pack_weights(const float* W_host, long N, long K, int* Kp, int* Np);
-float* fortis_chain_pack_bias(const float* b_host, long N, int Np);
-int  fortis_chain_ld(const ChainDesc& d);
+// Packs the layers (W[l] is [N][K] row-major, b[l] may be null) into one device blob and fills the
+// descriptor's shape fields; act/alpha/in_div/out_mul/mask_tail are left to the caller.
+int fortis_chain_build(ChainDesc* d, int nlayers, const float* const* W, const float* const* b, const int* K,
+                       const int* N, float** blob_out);
 void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows, hipStream_t s);
 // ---- stencil tables as the kernels see them (stencil.hip) --------------------------------
 struct CellStep { int op, code, tv_left; };

@@ -299,20 +299,23 @@ static size_t try_chain(fortis_plan* p, size_t i, Exec* ex)
     ex->dst = last_dst;
     ex->rows = ex->rows_cap = rows;
     ChainDesc& d = ex->chain;
-    d.nlayers = (int)lin.size();
-    for (size_t l = 0; l < lin.size(); l++) {
-        ChainLayer& L = d.L[l];
-        L.K = (int)lin[l]->K; L.N = (int)lin[l]->N; L.act = lin[l]->act; L.alpha = lin[l]->alpha;
-        float* wp = fortis_chain_pack_weights(lin[l]->w.data(), L.N, L.K, &L.Kp, &L.Np);
-        p->owned.push_back(wp);
-        float* bp = fortis_chain_pack_bias(lin[l]->has_bias ? lin[l]->b.data() : nullptr, L.N, L.Np);
-        p->owned.push_back(bp);
-        L.Wp = wp; L.bias = bp;
+    {
+        const float* Wh[FORTIS_CHAIN_MAX_LAYERS];
+        const float* bh[FORTIS_CHAIN_MAX_LAYERS];
+        int Ks[FORTIS_CHAIN_MAX_LAYERS], Ns[FORTIS_CHAIN_MAX_LAYERS];
+        for (size_t l = 0; l < lin.size(); l++) {
+            Wh[l] = lin[l]->w.data();
+            bh[l] = lin[l]->has_bias ? lin[l]->b.data() : nullptr;
+            Ks[l] = (int)lin[l]->K; Ns[l] = (int)lin[l]->N;
+        }
+        float* blob = nullptr;
+        if (fortis_chain_build(&d, (int)lin.size(), Wh, bh, Ks, Ns, &blob) != 0) return 0;
+        p->owned.push_back(blob);
+        for (size_t l = 0; l < lin.size(); l++) { d.L[l].act = lin[l]->act; d.L[l].alpha = lin[l]->alpha; }
     }
     if (in_div) d.in_div = (const float*)upload(p, in_div->v0.data(), in_div->v0.size() * 4);
     if (out_mul) d.out_mul = (const float*)upload(p, out_mul->v0.data(), out_mul->v0.size() * 4);
     d.mask_tail = mask ? (int)mask->tail : 0;
-    d.ld = fortis_chain_ld(d);
     return j - i;
 }
 

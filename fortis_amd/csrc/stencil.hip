@@ -16,50 +16,68 @@
 
 #define ST_THREADS 256
 
-__global__ __launch_bounds__(ST_THREADS) void gather_kernel(const StencilDev* __restrict__ d, PtrTab A,
-                                                            float* __restrict__ X, long rows)
+__global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, float* __restrict__ X, unsigned rows)
 {
+    __shared__ GatherArgs d;
     extern __shared__ float lds[];
-    const int n = d->nrefs;
+    params_to_lds(&d, ST_THREADS);
+    const int n = st_u(d.nrefs);
     const int tid = threadIdx.x;
-    const long row0 = (long)blockIdx.x * ST_THREADS, row = row0 + tid;
+    const unsigned row0 = blockIdx.x * ST_THREADS, row = row0 + tid;
     if (row < rows) {
-        const long col = row % d->count;
-        const int kk = (int)(row / d->count);
+        const unsigned col = row % d.count;
+        const int kk = (int)(row / d.count);
         int i, j;
         st_cell(d, col, i, j);
-        float S[FORTIS_MAX_SCAL], c[FORTIS_MAX_INS];
-        st_cell_values(d, A, i, j, kk, S, c);
-        for (int q = 0; q < n; q++) {
-            float tv = A.p[d->refs[q].array][st_elem(d, d->refs[q], i, j, kk)];
-            lds[tid * n + q] = st_chain(d, tv, S, c);
+        // all slot loads are issued before any of them is consumed
+        float tv[FORTIS_MAX_REFS];
+#pragma unroll
+        for (int q = 0; q < FORTIS_MAX_REFS; q++) {
+            const StSlotT<const float*> sl = d.refs[q < n ? q : 0];
+            tv[q] = st_g(sl.p)[st_off(sl, i, j, kk)];
         }
+        StCell cell;
+        st_prepare(d, i, j, kk, cell);
+        st_chain_apply(d, cell, tv);
+#pragma unroll
+        for (int q = 0; q < FORTIS_MAX_REFS; q++)
+            if (q < n) lds[tid * n + q] = tv[q];
     }
     __syncthreads();
-    const long lim = (rows - row0 < ST_THREADS ? rows - row0 : ST_THREADS) * n;
-    float* out = X + row0 * n;
-    for (long idx = tid; idx < lim; idx += ST_THREADS) out[idx] = lds[idx];
+    const unsigned lim = (rows - row0 < ST_THREADS ? rows - row0 : ST_THREADS) * n;
+    float* out = X + (size_t)row0 * n;
+    for (unsigned idx = tid; idx < lim; idx += ST_THREADS) out[idx] = lds[idx];
 }
 
-__global__ __launch_bounds__(ST_THREADS) void scatter_kernel(const StencilDev* __restrict__ d, PtrTabW A,
-                                                             const float* __restrict__ Y, int kk)
+__global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, const float* __restrict__ Y, int kk)
 {
+    __shared__ ScatterArgs d;
     extern __shared__ float lds[];
-    const int n = d->nrefs;
+    params_to_lds(&d, ST_THREADS);
+    const int n = st_u(d.nrefs);
     const int tid = threadIdx.x;
-    const long col0 = (long)blockIdx.x * ST_THREADS, col = col0 + tid;
-    const long lim = (d->count - col0 < ST_THREADS ? d->count - col0 : ST_THREADS) * n;
-    const float* in = Y + col0 * n;
-    for (long idx = tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
+    const unsigned col0 = blockIdx.x * ST_THREADS, col = col0 + tid;
+    const unsigned lim = (d.count - col0 < ST_THREADS ? d.count - col0 : ST_THREADS) * n;
+    const float* in = Y + (size_t)col0 * n;
+    for (unsigned idx = tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
     __syncthreads();
-    if (col >= d->count) return;
+    if (col >= d.count) return;
     int i, j;
     st_cell(d, col, i, j);
-    float S[FORTIS_MAX_SCAL], c[FORTIS_MAX_INS];
-    st_cell_values(d, A, i, j, kk, S, c);
-    for (int q = 0; q < n; q++) {
-        const float tv = st_chain(d, lds[tid * n + q], S, c);
-        A.p[d->refs[q].array][st_elem(d, d->refs[q], i, j, kk)] = tv;
+    StCell cell;
+    st_prepare(d, i, j, kk, cell);
+    // outputs are few (one per model output); handled eight at a time
+    for (int q0 = 0; q0 < n; q0 += 8) {
+        float tv[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) tv[t] = q0 + t < n ? lds[tid * n + q0 + t] : 0.f;
+        st_chain_apply(d, cell, tv);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+            if (q0 + t < n) {
+                const StSlotT<float*> sl = d.refs[q0 + t];
+                st_g(sl.p)[st_off(sl, i, j, kk)] = tv[t];
+            }
     }
 }
 
@@ -68,8 +86,9 @@ int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
 {
     memset(out, 0, sizeof *out);
     if (in->narrays < 1 || in->narrays > FORTIS_MAX_ARRAYS || in->nrefs < 1 || in->nrefs > FORTIS_MAX_REFS ||
-        in->nscal < 0 || in->nscal > FORTIS_MAX_SCAL || in->nins < 0 || in->nins > FORTIS_MAX_INS ||
-        in->nconst < 0 || in->nconst > FORTIS_MAX_CONST || in->count < 1 || in->nk < 1) {
+        in->nscal < 0 || in->nscal > ST_SCAL_MAX || in->nins < 0 || in->nins > FORTIS_MAX_INS ||
+        in->nconst < 0 || in->nconst > FORTIS_MAX_CONST || in->count < 1 || in->nk < 1 ||
+        in->count * in->nk >= 4294967295L / FORTIS_MAX_REFS) {
         fprintf(stderr, "fortis: stencil table out of range\n");
         return -1;
     }
@@ -82,6 +101,7 @@ int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
     for (int r = 0; r < in->nrefs + in->nscal; r++) {
         const fortis_ref_t& f = r < in->nrefs ? in->refs[r] : in->scal[r - in->nrefs];
         if (f.array < 0 || f.array >= in->narrays) { fprintf(stderr, "fortis: stencil ref names array %d\n", f.array); return -1; }
+        if (f.si > 2147483647L || f.sj > 2147483647L || f.si < -2147483647L || f.sj < -2147483647L) { fprintf(stderr, "fortis: stencil stride out of range\n"); return -1; }
     }
     for (int c = 0; c < in->nconst; c++) out->consts[c] = in->consts[c];
     out->count = in->count; out->nk = in->nk;
@@ -104,9 +124,11 @@ int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
         if (isdep[0] || isdep[1]) {
             dep[n] = 1; map[n] = -1; last_dep = n;
             CellStep st = { I.op, isdep[0] ? lowered[1] : lowered[0], isdep[0] ? 1 : 0 };
+            if (out->nchain == ST_CHAIN_MAX) { fprintf(stderr, "fortis: stencil expression chains more than %d operations on the slot value\n", ST_CHAIN_MAX); return -1; }
             out->chain[out->nchain++] = st;
         } else {
             dep[n] = 0; map[n] = out->ncell;
+            if (out->ncell == ST_CELL_MAX) { fprintf(stderr, "fortis: more than %d per-cell stencil instructions\n", ST_CELL_MAX); return -1; }
             fortis_ins_t ci = { I.op, lowered[0], lowered[1] };
             out->cell[out->ncell++] = ci;
         }
@@ -123,9 +145,8 @@ int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
 struct BoundStencil {
     bool ok = false;
     fortis_stencil_t host;       // as configured (cells pointer not owned)
-    StencilDev low;              // lowered, with device cell list
-    StencilDev* dev = nullptr;   // device copy of `low`
-    int* dcells = nullptr;
+    StencilDev low;              // lowered table
+    int* dcells = nullptr;       // device copy of the cell list
     void* darr[FORTIS_MAX_ARRAYS] = {};       // device planes of the host arrays
     const void* reg[FORTIS_MAX_ARRAYS] = {};  // last host address seen per array
     bool written[FORTIS_MAX_ARRAYS] = {};
@@ -133,7 +154,7 @@ struct BoundStencil {
 };
 static BoundStencil g_gather, g_scatter;
 
-static int upload_table(const fortis_stencil_t* t, StencilDev* low, StencilDev** dev, int** dcells)
+static int upload_table(const fortis_stencil_t* t, StencilDev* low, int** dcells)
 {
     if (fortis_stencil_lower(t, low) != 0) return -1;
     if (t->cells) {
@@ -141,14 +162,11 @@ static int upload_table(const fortis_stencil_t* t, StencilDev* low, StencilDev**
         HIP_OK(hipMemcpy(*dcells, t->cells, t->count * sizeof(int), hipMemcpyHostToDevice));
         low->cells = *dcells;
     }
-    HIP_OK(hipMalloc((void**)dev, sizeof(StencilDev)));
-    HIP_OK(hipMemcpy(*dev, low, sizeof(StencilDev), hipMemcpyHostToDevice));
     return 0;
 }
 
 static void release(BoundStencil& b)
 {
-    if (b.dev) HIP_OK(hipFree(b.dev));
     if (b.dcells) HIP_OK(hipFree(b.dcells));
     for (int a = 0; a < FORTIS_MAX_ARRAYS; a++) if (b.darr[a]) HIP_OK(hipFree(b.darr[a]));
     b = BoundStencil();
@@ -157,7 +175,7 @@ static void release(BoundStencil& b)
 static int config(BoundStencil& b, const fortis_stencil_t* t, bool is_scatter)
 {
     release(b);
-    if (upload_table(t, &b.low, &b.dev, &b.dcells) != 0) return -1;
+    if (upload_table(t, &b.low, &b.dcells) != 0) return -1;
     b.host = *t;
     b.host.cells = nullptr;
     if (is_scatter) for (int r = 0; r < t->nrefs; r++) b.written[t->refs[r].array] = true;
@@ -172,7 +190,7 @@ void fortis_stencil_reset_internal()
 }
 
 // cache of device tables for the device-resident API (keyed by table contents)
-struct CacheEnt { fortis_stencil_t key; const int* cells_key; StencilDev* dev; StencilDev low; };
+struct CacheEnt { fortis_stencil_t key; const int* cells_key; int* dcells; StencilDev low; };
 static CacheEnt g_cache[16];
 static int g_ncache = 0;
 static CacheEnt* cached(const fortis_stencil_t* t)
@@ -184,35 +202,34 @@ static CacheEnt* cached(const fortis_stencil_t* t)
     }
     if (g_ncache == 16) { fprintf(stderr, "fortis: stencil table cache full\n"); return nullptr; }
     CacheEnt* e = &g_cache[g_ncache];
-    int* dc = nullptr;
-    if (upload_table(t, &e->low, &e->dev, &dc) != 0) return nullptr;
+    e->dcells = nullptr;
+    if (upload_table(t, &e->low, &e->dcells) != 0) return nullptr;
     e->key = *t;
     e->cells_key = t->cells;
     g_ncache++;
     return e;
 }
 
-static void launch_gather(const StencilDev* dev, const StencilDev& low, const float* const* dA, float* dX, hipStream_t s)
+static void launch_gather(const StencilDev& low, const float* const* dA, float* dX, hipStream_t s)
 {
-    PtrTab tab = {};
-    for (int a = 0; a < low.narrays; a++) tab.p[a] = dA[a];
-    const long rows = low.count * low.nk;
+    GatherArgs a;
+    st_make_args<const float*>(low, low.cells, dA, &a);
+    const unsigned rows = (unsigned)(low.count * low.nk);
     hipLaunchKernelGGL(gather_kernel, dim3((unsigned)cdiv(rows, ST_THREADS)), dim3(ST_THREADS),
-                       (size_t)ST_THREADS * low.nrefs * sizeof(float), s, dev, tab, dX, rows);
+                       (size_t)ST_THREADS * low.nrefs * sizeof(float), s, a, dX, rows);
     HIP_OK(hipGetLastError());
 }
-static void launch_scatter(const StencilDev* dev, const StencilDev& low, float* const* dA, const float* dY, int kk, hipStream_t s)
+static void launch_scatter(const StencilDev& low, float* const* dA, const float* dY, int kk, hipStream_t s)
 {
-    PtrTabW tab = {};
-    for (int a = 0; a < low.narrays; a++) tab.p[a] = dA[a];
+    ScatterArgs a;
+    st_make_args<float*>(low, low.cells, dA, &a);
     hipLaunchKernelGGL(scatter_kernel, dim3((unsigned)cdiv(low.count, ST_THREADS)), dim3(ST_THREADS),
-                       (size_t)ST_THREADS * low.nrefs * sizeof(float), s, dev, tab, dY, kk);
+                       (size_t)ST_THREADS * low.nrefs * sizeof(float), s, a, dY, kk);
     HIP_OK(hipGetLastError());
 }
 
-void fortis_launch_chain_stencil_dev(const ChainDesc& d, const StencilDev* g_dev, const StencilDev* sc_dev,
-                                     long rows, const float* const* dG, int nG, float* const* dS, int nS,
-                                     float* dY, hipStream_t s);
+void fortis_launch_chain_stencil(const ChainDesc& d, const StencilDev& g, const StencilDev& sc, long rows,
+                                 const float* const* dG, float* const* dS, float* dY, hipStream_t s);
 // plan.hip: describes the plan as a chain if it is one
 int fortis_plan_as_chain(fortis_plan* p, ChainDesc* out);
 
@@ -259,7 +276,7 @@ void fortis_gather_v(const int* a, const void* const* H)
         HIP_OK(hipMemcpyAsync(b.darr[ai], (const float*)H[ai] + off, nelem * sizeof(float), hipMemcpyHostToDevice, s));
         dptr[ai] = (const float*)b.darr[ai];
     }
-    launch_gather(b.dev, b.low, dptr, (float*)fortis_model_input(), s);
+    launch_gather(b.low, dptr, (float*)fortis_model_input(), s);
 }
 
 void fortis_scatter_v(const int* a, void* const* H)
@@ -284,7 +301,7 @@ void fortis_scatter_v(const int* a, void* const* H)
     }
     // the device holds ONE plane per array here, so the kernel runs with plane index 0
     const long yoff = t.nk > 1 ? (long)(k1 - t.klo) * t.count * t.nrefs : 0;   // gather.cu:86
-    launch_scatter(b.dev, b.low, dptr, (const float*)fortis_model_output() + yoff, 0, s);
+    launch_scatter(b.low, dptr, (const float*)fortis_model_output() + yoff, 0, s);
     for (int r = 0; r < t.nrefs; r++) {
         const int ai = t.refs[r].array;
         const long off = t.total[ai] > t.plane[ai] ? (long)(k1 - 1) * t.plane[ai] : 0;
@@ -319,13 +336,13 @@ void fortis_stencil_gather_dev(const fortis_stencil_t* g, const float* const* dA
 {
     CacheEnt* e = cached(g);
     if (!e) return;
-    launch_gather(e->dev, e->low, dA, dX, fortis_stream_get());
+    launch_gather(e->low, dA, dX, fortis_stream_get());
 }
 void fortis_stencil_scatter_dev(const fortis_stencil_t* sd, float* const* dA, const float* dY, int kk)
 {
     CacheEnt* e = cached(sd);
     if (!e) return;
-    launch_scatter(e->dev, e->low, dA, dY, kk, fortis_stream_get());
+    launch_scatter(e->low, dA, dY, kk, fortis_stream_get());
 }
 
 int fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t* sd, fortis_plan* p,
@@ -349,8 +366,7 @@ int fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t*
     CacheEnt* eg = cached(g);
     CacheEnt* es = cached(&s2);
     if (!eg || !es) return -1;
-    fortis_launch_chain_stencil_dev(d, eg->dev, es->dev, g->count * g->nk, dG, g->narrays, dS, sd->narrays, dY,
-                                    fortis_stream_get());
+    fortis_launch_chain_stencil(d, eg->low, es->low, g->count * g->nk, dG, dS, dY, fortis_stream_get());
     return 0;
 }
 

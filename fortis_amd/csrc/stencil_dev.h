@@ -1,22 +1,66 @@
 // Device-side helpers shared by the stencil gather/scatter kernels and the fused
-// gather -> MLP -> scatter kernel.  The tables (StencilDev) live in device memory and are read
-// with wave-uniform addresses; all expression arithmetic is explicit round-to-nearest fp32 with
-// no contraction, matching the reference's `-fmad=false` gather.cu.
+// gather -> MLP -> scatter kernel.
+//
+// The tables travel as kernel arguments (StencilArgs, ~1.3 KB) and every kernel first copies its
+// argument block from the kernarg segment into LDS with one 16-byte vector load per thread
+// (params_to_lds); after that a table read is an LDS read.  Reading the tables in place (scalar loads
+// from the kernarg segment, each followed by a wait) cost a wave ~80 serialized round trips and was
+// what bounded the first versions of these kernels.  Each slot carries its final device pointer
+// (array base + element offset folded in on the host), so slot loads need no second table.
+// All expression arithmetic is explicit round-to-nearest fp32 with no contraction, matching the
+// reference's `-fmad=false` gather.cu.
 #pragma once
 #include "common.h"
 
-struct PtrTab { const float* p[FORTIS_MAX_ARRAYS]; };
-struct PtrTabW { float* p[FORTIS_MAX_ARRAYS]; };
+#define ST_CHAIN_MAX 6   // operations chained on the slot value
+#define ST_CELL_MAX 6    // per-cell instructions (no slot value involved)
+#define ST_SCAL_MAX 4    // same-cell scalars the kernels load
+
+template <typename P>
+struct StSlotT { P p; int si, sj; long plane; };      // elem = p[i*si + j*sj + kk*plane]
+
+// Copies the kernel's first (by-value, 16-byte aligned) argument from the kernarg segment into LDS.
+template <typename T>
+__device__ __forceinline__ void params_to_lds(T* dst, int nthreads)
+{
+    static_assert(sizeof(T) % 16 == 0, "parameter block must be a multiple of 16 bytes");
+    const float4* src = (const float4*)__builtin_amdgcn_kernarg_segment_ptr();
+    for (int i = threadIdx.x; i < (int)(sizeof(T) / 16); i += nthreads) ((float4*)dst)[i] = src[i];
+    __syncthreads();
+}
+// A pointer read back from LDS has lost its address space; device arrays are global memory.
+typedef __attribute__((address_space(1))) float gfloat;
+__device__ __forceinline__ const gfloat* st_g(const float* p) { return (const gfloat*)p; }
+__device__ __forceinline__ gfloat* st_g(float* p) { return (gfloat*)p; }
+__device__ __forceinline__ int st_u(int v) { return __builtin_amdgcn_readfirstlane(v); }   // wave-uniform value
+struct StIns { int op, a, b; float ca, cb; };          // per-cell instruction, constants inlined
+struct StStep { int op, code, tv_left; float cv; };    // tv chain step, constant inlined
+
+template <typename P>
+struct alignas(16) StencilArgsT {
+    int nrefs, nscal, ncell, nchain;
+    StSlotT<P> refs[FORTIS_MAX_REFS];
+    StSlotT<P> scal[ST_SCAL_MAX];
+    StIns cell[ST_CELL_MAX];
+    StStep chain[ST_CHAIN_MAX];
+    unsigned count;
+    int ilo, jlo, ni, sx;
+    const int* cells;
+};
+typedef StencilArgsT<const float*> GatherArgs;
+typedef StencilArgsT<float*> ScatterArgs;
 
 // cell number -> 1-based (i, j): the rectangle of mom6_zb/gather.cu:15-16, or the cell list.
-__device__ __forceinline__ void st_cell(const StencilDev* d, long col, int& i, int& j)
+template <typename A>
+__device__ __forceinline__ void st_cell(const A& d, unsigned col, int& i, int& j)
 {
-    if (d->cells) { int c = d->cells[col]; i = 1 + c % d->sx; j = 1 + c / d->sx; }
-    else { i = d->ilo + (int)(col % d->ni); j = d->jlo + (int)(col / d->ni); }
+    if (d.cells) { const unsigned c = (unsigned)((const __attribute__((address_space(1))) int*)d.cells)[col]; i = 1 + (int)(c % (unsigned)d.sx); j = 1 + (int)(c / (unsigned)d.sx); }
+    else { i = d.ilo + (int)(col % (unsigned)d.ni); j = d.jlo + (int)(col / (unsigned)d.ni); }
 }
-__device__ __forceinline__ long st_elem(const StencilDev* d, const fortis_ref_t& r, int i, int j, int kk)
+template <typename S>
+__device__ __forceinline__ long st_off(const S& r, int i, int j, int kk)
 {
-    return r.base + (long)i * r.si + (long)j * r.sj + (r.planar ? (long)kk * d->plane[r.array] : 0L);
+    return (long)i * r.si + (long)j * r.sj + (long)kk * r.plane;
 }
 __device__ __forceinline__ float st_arith(int op, float a, float b)
 {
@@ -27,45 +71,110 @@ __device__ __forceinline__ float st_arith(int op, float a, float b)
         default: return __fdiv_rn(a, b);
     }
 }
-// operand of per-cell code: 1..8 scalar, 16+ constant, 32+ earlier per-cell result
-__device__ __forceinline__ float st_operand(const StencilDev* d, int code, const float (&S)[FORTIS_MAX_SCAL],
-                                            const float (&c)[FORTIS_MAX_INS])
+// operand of per-cell code: 1..8 scalar, 16+ constant (value inlined as cv), 32+ earlier result
+__device__ __forceinline__ float st_operand(int code, float cv, const float (&S)[ST_SCAL_MAX],
+                                            const float (&c)[ST_CELL_MAX])
 {
-    float v = 0.f;
-    if (code >= 32) {
+    float v = cv;
 #pragma unroll
-        for (int m = 0; m < FORTIS_MAX_INS; m++) if (code - 32 == m) v = c[m];
-    } else if (code >= 16) {
-        v = d->consts[code - 16];
-    } else {
+    for (int m = 0; m < ST_CELL_MAX; m++) v = (code == 32 + m) ? c[m] : v;
 #pragma unroll
-        for (int s = 0; s < FORTIS_MAX_SCAL; s++) if (code - 1 == s) v = S[s];
-    }
+    for (int s = 0; s < ST_SCAL_MAX; s++) v = (code == 1 + s) ? S[s] : v;
     return v;
 }
-// Loads the same-cell scalars and evaluates the per-cell instructions.
-template <typename Tab>
-__device__ __forceinline__ void st_cell_values(const StencilDev* d, const Tab& A, int i, int j, int kk,
-                                               float (&S)[FORTIS_MAX_SCAL], float (&c)[FORTIS_MAX_INS])
+// Same-cell scalars and per-cell instruction results of one cell.
+struct StCell { float S[ST_SCAL_MAX]; float c[ST_CELL_MAX]; };
+
+// Evaluates the per-cell instructions on scalars already in cell.S.
+template <typename A>
+__device__ __forceinline__ void st_cell_program(const A& d, StCell& cell)
 {
+    const int ncell = st_u(d.ncell);
 #pragma unroll
-    for (int s = 0; s < FORTIS_MAX_SCAL; s++) {
-        S[s] = 0.f;
-        if (s < d->nscal) S[s] = A.p[d->scal[s].array][st_elem(d, d->scal[s], i, j, kk)];
-    }
-#pragma unroll
-    for (int n = 0; n < FORTIS_MAX_INS; n++) {
-        c[n] = 0.f;
-        if (n < d->ncell) c[n] = st_arith(d->cell[n].op, st_operand(d, d->cell[n].a, S, c), st_operand(d, d->cell[n].b, S, c));
+    for (int n = 0; n < ST_CELL_MAX; n++) {
+        cell.c[n] = 0.f;
+        if (n < ncell) {
+            const StIns ci = d.cell[n];
+            cell.c[n] = st_arith(st_u(ci.op), st_operand(st_u(ci.a), ci.ca, cell.S, cell.c), st_operand(st_u(ci.b), ci.cb, cell.S, cell.c));
+        }
     }
 }
-// Runs the tv chain on one slot value.
-__device__ __forceinline__ float st_chain(const StencilDev* d, float tv, const float (&S)[FORTIS_MAX_SCAL],
-                                          const float (&c)[FORTIS_MAX_INS])
+// Loads the same-cell scalars and evaluates the per-cell instructions.
+template <typename A>
+__device__ __forceinline__ void st_prepare(const A& d, int i, int j, int kk, StCell& cell)
 {
-    for (int n = 0; n < d->nchain; n++) {
-        float o = st_operand(d, d->chain[n].code, S, c);
-        tv = d->chain[n].tv_left ? st_arith(d->chain[n].op, tv, o) : st_arith(d->chain[n].op, o, tv);
+    // unconditional loads (an unused scalar re-reads scalar 0): no branch separates them, so they are
+    // issued together with the slot loads and waited for once
+#pragma unroll
+    for (int s = 0; s < ST_SCAL_MAX; s++) {
+        const StSlotT<decltype(d.scal[0].p)> sl = d.scal[s < d.nscal ? s : 0];
+        cell.S[s] = st_g(sl.p)[st_off(sl, i, j, kk)];
     }
-    return tv;
+    st_cell_program(d, cell);
+}
+// Runs the tv chain on N slot values at once: the loop over chain steps is a real loop (one table
+// read and one wave-uniform switch per step), each arm handles all N values, so the generated code
+// holds each operation once per arm instead of once per slot and step.
+template <int N, typename A>
+__device__ __forceinline__ void st_chain_apply(const A& d, const StCell& cell, float (&tv)[N])
+{
+    const int nchain = st_u(d.nchain);
+    for (int n = 0; n < nchain; n++) {
+        const StStep st = d.chain[n];
+        const float o = st_operand(st_u(st.code), st.cv, cell.S, cell.c);
+        switch (st_u(st.op * 2 + (st.tv_left ? 1 : 0))) {
+            case 0: case 1:
+#pragma unroll
+                for (int t = 0; t < N; t++) tv[t] = __fadd_rn(tv[t], o);
+                break;
+            case 2:
+#pragma unroll
+                for (int t = 0; t < N; t++) tv[t] = __fsub_rn(o, tv[t]);
+                break;
+            case 3:
+#pragma unroll
+                for (int t = 0; t < N; t++) tv[t] = __fsub_rn(tv[t], o);
+                break;
+            case 4: case 5:
+#pragma unroll
+                for (int t = 0; t < N; t++) tv[t] = __fmul_rn(tv[t], o);
+                break;
+            case 6:
+#pragma unroll
+                for (int t = 0; t < N; t++) tv[t] = __fdiv_rn(o, tv[t]);
+                break;
+            default:
+#pragma unroll
+                for (int t = 0; t < N; t++) tv[t] = __fdiv_rn(tv[t], o);
+                break;
+        }
+    }
+}
+
+// Host: lowered table + device array pointers -> kernel arguments.
+template <typename P>
+static inline void st_make_args(const StencilDev& low, const int* dcells, P const* arrays, StencilArgsT<P>* a)
+{
+    memset(a, 0, sizeof *a);
+    a->nrefs = low.nrefs; a->nscal = low.nscal; a->ncell = low.ncell; a->nchain = low.nchain;
+    for (int r = 0; r < low.nrefs + low.nscal; r++) {
+        const fortis_ref_t& f = r < low.nrefs ? low.refs[r] : low.scal[r - low.nrefs];
+        StSlotT<P>& s = r < low.nrefs ? a->refs[r] : a->scal[r - low.nrefs];
+        s.p = arrays[f.array] + f.base;
+        s.si = (int)f.si; s.sj = (int)f.sj;
+        s.plane = f.planar ? low.plane[f.array] : 0;
+    }
+    auto cval = [&](int code) { return (code >= 16 && code < 32) ? low.consts[code - 16] : 0.f; };
+    for (int n = 0; n < low.ncell; n++) {
+        StIns i = { low.cell[n].op, low.cell[n].a, low.cell[n].b, cval(low.cell[n].a), cval(low.cell[n].b) };
+        a->cell[n] = i;
+    }
+    for (int n = 0; n < low.nchain; n++) {
+        StStep s = { low.chain[n].op, low.chain[n].code, low.chain[n].tv_left, cval(low.chain[n].code) };
+        a->chain[n] = s;
+    }
+    if (low.nscal == 0) { a->scal[0].p = a->refs[0].p; a->scal[0].si = a->refs[0].si; a->scal[0].sj = a->refs[0].sj; a->scal[0].plane = a->refs[0].plane; }
+    a->count = (unsigned)low.count;
+    a->ilo = low.ilo; a->jlo = low.jlo; a->ni = low.ni; a->sx = low.sx;
+    a->cells = dcells;
 }
