@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # same command (see profiles/), or None where no counter run has been made for the workload.
-MEASURED_TRAFFIC = {"climsim": (122875 + 68525) * 1024, "zb": None, "zb_ref": None, "toy": None}
+MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": None, "zb_ref": None, "toy": None}
 
 
 def omp_threads():

@@ -35,16 +35,17 @@ __device__ __forceinline__ float gemm_act(float v, int act, float alpha)
     return v;
 }
 
-// Epilogue of a whole tile with nothing but bias and activation: per element one add, the activation
+// Epilogue of a tile with all its rows and nothing but bias and activation: per element one add, the activation
 // (MODE 0 none, 1 max(v, 0), 2 max(v, alpha v) for 0 <= alpha <= 1, 3 the general form) and a store to
 // uniform row base + one of TM*TN per-lane 32-bit offsets.
 template <int TM, int TN, int MODE>
 __device__ __forceinline__ void gemm_store_plain(const v16f (&acc)[TM][TN], float* cb, unsigned Nu, const float* bias,
-                                                 int wm, int wn, int lr, int lh, const GemmEpi& epi)
+                                                 int wm, int wn, int lr, int lh, int ncols, const GemmEpi& epi)
 {
     const float alpha = epi.alpha;
 #pragma unroll
     for (int j = 0; j < TN; j++) {
+        if (wn + j * 32 + lr >= ncols) continue;                         // column past the end of C
         const float bv = bias ? bias[wn + j * 32 + lr] : 0.f;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
@@ -76,8 +77,8 @@ __device__ __forceinline__ void lds_barrier()
 // Schedule of one k slab (NKG groups of 8 k, one group = TM*TN*4 MFMAs per wave):
 //   top      global loads of the next slab -> staging registers (ra, rw)
 //   group g  LDS reads of the fragments of group g+1, then the MFMAs of group g
-//   before the last group: staging registers -> other LDS buffer, barrier, LDS reads of the next
-//   slab's group 0, then the MFMAs of the last group
+//   before group NKG-2: staging registers -> other LDS buffer
+//   before the last group: barrier, LDS reads of the next slab's group 0
 // so every LDS read has a whole group of MFMAs to arrive, and the barrier is followed by MFMAs that
 // were already fed.  The staging registers belong to the caller: when `preloaded`, they already hold
 // this tile's slab 0, and when `has_next`, the last slab's "next slab" is slab 0 of tile (m0n, n0n),
@@ -212,25 +213,28 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
 #pragma unroll
         for (int kg = 0; kg + 1 < NKG; kg++) {
             read_frag((kg + 1) & 1, buf, kg + 1);
+            // the staged slab goes to LDS one group before the barrier, so the writes drain behind MFMAs
+            if (kg == NKG - 2 && NKG > 2 && more) store_slab(buf ^ 1);
             multiply(kg & 1);
         }
-        if (more) store_slab(buf ^ 1);
+        if (NKG == 2 && more) store_slab(buf ^ 1);
         lds_barrier();
         if (more) read_frag(0, buf ^ 1, 0);
         multiply((NKG - 1) & 1);
     }
 
     // epilogue: lane holds column n = lr of 16 rows per MFMA tile.
-    // Whole tiles with a plain bias + activation epilogue (every hidden layer) take a path with one
-    // add, the activation and one 32-bit offset add per element; everything else takes the guarded one.
-    const bool plain = !epi.out_scale && epi.mask_from >= N && m0 + BM <= B && n0 + BN <= N;
+    // Tiles with all their rows and a plain bias + activation epilogue (every hidden layer) take a path
+    // with one add and the activation per element; everything else takes the guarded one.
+    const bool plain = !epi.out_scale && epi.mask_from >= N && m0 + BM <= B;
+    const int ncols = (int)(N - n0 < BN ? N - n0 : BN);                 // columns of this tile that exist
     if (plain) {
         float* cb = C + m0 * N + n0;                                    // uniform
         const float* bias = epi.bias ? epi.bias + n0 : nullptr;
-        if (epi.act == FORTIS_ACT_RELU) gemm_store_plain<TM, TN, 1>(acc, cb, (unsigned)N, bias, wm, wn, lr, lh, epi);
-        else if (epi.act == FORTIS_ACT_LEAKY && epi.alpha >= 0.f && epi.alpha <= 1.f) gemm_store_plain<TM, TN, 2>(acc, cb, (unsigned)N, bias, wm, wn, lr, lh, epi);
-        else if (epi.act == FORTIS_ACT_NONE) gemm_store_plain<TM, TN, 0>(acc, cb, (unsigned)N, bias, wm, wn, lr, lh, epi);
-        else gemm_store_plain<TM, TN, 3>(acc, cb, (unsigned)N, bias, wm, wn, lr, lh, epi);
+        if (epi.act == FORTIS_ACT_RELU) gemm_store_plain<TM, TN, 1>(acc, cb, (unsigned)N, bias, wm, wn, lr, lh, ncols, epi);
+        else if (epi.act == FORTIS_ACT_LEAKY && epi.alpha >= 0.f && epi.alpha <= 1.f) gemm_store_plain<TM, TN, 2>(acc, cb, (unsigned)N, bias, wm, wn, lr, lh, ncols, epi);
+        else if (epi.act == FORTIS_ACT_NONE) gemm_store_plain<TM, TN, 0>(acc, cb, (unsigned)N, bias, wm, wn, lr, lh, ncols, epi);
+        else gemm_store_plain<TM, TN, 3>(acc, cb, (unsigned)N, bias, wm, wn, lr, lh, ncols, epi);
         return;
     }
 #pragma unroll
