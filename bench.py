@@ -224,9 +224,15 @@ def run_toy(L, args):
 def run_zb(L, args, reference_net=False):
     """gather -> MLP -> scatter for all 15 layers of the reference geometry in one kernel."""
     from fortis_amd import configs, plan as P, stencil as S
-    sx, sy, nz = 68, 78, 15
     g = os.path.join(ROOT, "tests", "golden")
-    gt, st, gd, sd, lp, kd = S.load_tables(f"{g}/zb_gather.json", f"{g}/zb_scatter.json", f"{g}/zb_loop.json", f"{g}/zb_kdist.json")
+    if args.grid:
+        # the same step on a larger synthetic grid (descriptors in the reference's schema)
+        sx, sy, nz = (int(v) for v in args.grid.lower().split("x"))
+        gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+        gt, st = S.build_table(gd, lp, kd, "gather"), S.build_table(sd, lp, kd, "scatter")
+    else:
+        sx, sy, nz = 68, 78, 15
+        gt, st, gd, sd, lp, kd = S.load_tables(f"{g}/zb_gather.json", f"{g}/zb_scatter.json", f"{g}/zb_loop.json", f"{g}/zb_kdist.json")
     A = configs.zb_arrays(sx, sy, nz)
     rows = gt.count * gt.nk
     if reference_net:
@@ -270,7 +276,7 @@ def run_zb(L, args, reference_net=False):
                 hbm_GBs=round(gbs, 2), mfma_TFLOPs=round(tf, 3), traffic=MEASURED_TRAFFIC["zb_ref" if reference_net else "zb"])
     # dt covers the validating launch too; whole-job throughput uses the clocked launches only
     out = dict(rows=rows, dt=ms * 1e-3, wall_dt=dt, dtype="f32",
-               config={"workload": "zb_gather_mlp_scatter_%s_68x78x15" % ("27_20_3" if reference_net else "27_64_64_3"),
+               config={"workload": "zb_gather_mlp_scatter_%s_%dx%dx%d" % ("27_20_3" if reference_net else "27_64_64_3", sx, sy, nz),
                        "columns": rows, "cells_per_layer": int(gt.count), "layers": int(gt.nk), "widths": widths,
                        "launches_per_step": 1},
                roofline=roof)
@@ -291,6 +297,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="climsim", choices=["climsim", "zb", "zb_ref", "toy", "copy", "unet", "tsrgan"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--grid", default=None, help="zb / zb_ref only: SXxSYxNZ grid instead of the reference's 68x78x15")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the fused step on ONE GPU; --gpus %d is not supported "

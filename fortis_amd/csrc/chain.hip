@@ -259,50 +259,174 @@ void chain_wave_kernel(ChainParams params)
     const int K0 = st_u(d.L[0].K), K0p = st_u(d.L[0].Kp);
     const int NO = st_u(d.L[nlayers - 1].N), mask_tail = st_u(d.mask_tail);
     const unsigned rows = P.rows;
-    const unsigned row0 = (blockIdx.x * 4 + wave) * 16;         // first row of this wave's tile
     const int lrow = lane & 15, lq = lane >> 4;
-    const unsigned row = row0 + lrow;
-    const bool valid = row < rows;
     const gfloat* wall = st_g(d.wall);
     const gfloat* in_div = st_g(d.in_div);
     const gfloat* out_mul = st_g(d.out_mul);
 
-    // ---- every global load of the tile is issued here -------------------------------------------------
-    float tv[QMAX], gS[ST_SCAL_MAX], sS[ST_SCAL_MAX], xr[XR];
-    int si = 0, sj = 0, skk = 0;
-    if (STENCIL) {
-        const unsigned rc = valid ? row : 0;
-        const int kk = (int)(rc / g.count);
-        int i, j;
-        st_cell(g, rc % g.count, i, j);
+    // Everything a tile reads from global memory, as registers: slot values, gather scalars, scatter
+    // scalars (stencil form) or the 16 x K0 input block (plain form).
+    struct TileIn {
+        float tv[QMAX], gS[ST_SCAL_MAX], sS[ST_SCAL_MAX], xr[XR];
+        int si, sj, skk;
+        unsigned row0;
+    };
+    // ---- issues every global load of the tile at row0 ---------------------------------------------------
+    auto issue = [&](TileIn& in, unsigned row0) __attribute__((always_inline)) {
+        in.row0 = row0;
+        in.si = in.sj = in.skk = 0;
+        if (STENCIL) {
+            const unsigned row = row0 + lrow;
+            const unsigned rc = row < rows ? row : 0;
+            const int kk = (int)(rc / g.count);
+            int i, j;
+            st_cell(g, rc % g.count, i, j);
 #pragma unroll
-        for (int t = 0; t < QMAX; t++) {
-            const int q = lq + 4 * t;
-            const StSlotT<const float*> sl = g.refs[q < K0 ? q : 0];
-            tv[t] = st_g(sl.p)[st_off(sl, i, j, kk)];
-        }
+            for (int t = 0; t < QMAX; t++) {
+                const int q = lq + 4 * t;
+                const StSlotT<const float*> sl = g.refs[q < K0 ? q : 0];
+                in.tv[t] = st_g(sl.p)[st_off(sl, i, j, kk)];
+            }
 #pragma unroll
-        for (int s = 0; s < ST_SCAL_MAX; s++) {
-            const StSlotT<const float*> sl = g.scal[s < g.nscal ? s : 0];
-            gS[s] = st_g(sl.p)[st_off(sl, i, j, kk)];
-        }
-        skk = (int)(rc / sc.count);
-        st_cell(sc, rc % sc.count, si, sj);
+            for (int s = 0; s < ST_SCAL_MAX; s++) {
+                const StSlotT<const float*> sl = g.scal[s < g.nscal ? s : 0];
+                in.gS[s] = st_g(sl.p)[st_off(sl, i, j, kk)];
+            }
+            in.skk = (int)(rc / sc.count);
+            st_cell(sc, rc % sc.count, in.si, in.sj);
 #pragma unroll
-        for (int s = 0; s < ST_SCAL_MAX; s++) {
-            const StSlotT<float*> sl = sc.scal[s < sc.nscal ? s : 0];
-            sS[s] = st_g(sl.p)[st_off(sl, si, sj, skk)];
-        }
-    } else {
-        const gfloat* X = st_g(P.X);
-        const long base = (long)row0 * K0;
-        const long lim = (long)rows * K0 - base;
+            for (int s = 0; s < ST_SCAL_MAX; s++) {
+                const StSlotT<float*> sl = sc.scal[s < sc.nscal ? s : 0];
+                in.sS[s] = st_g(sl.p)[st_off(sl, in.si, in.sj, in.skk)];
+            }
+        } else {
+            const gfloat* X = st_g(P.X);
+            const long base = (long)row0 * K0;
+            const long lim = (long)rows * K0 - base;
 #pragma unroll
-        for (int t = 0; t < XR; t++) {
-            const int idx = lane + t * 64;
-            xr[t] = (idx < 16 * K0 && idx < lim) ? X[base + idx] : 0.f;
+            for (int t = 0; t < XR; t++) {
+                const int idx = lane + t * 64;
+                in.xr[t] = (idx < 16 * K0 && idx < lim) ? X[base + idx] : 0.f;
+            }
         }
-    }
+    };
+    // ---- one tile: input into the wave's LDS tile, the layers in place, results out --------------------
+    auto process = [&](TileIn& in) __attribute__((always_inline)) {
+        const unsigned row0 = in.row0, row = row0 + lrow;
+        const bool valid = row < rows;
+        if (STENCIL) {
+            StCell cell;
+#pragma unroll
+            for (int s = 0; s < ST_SCAL_MAX; s++) cell.S[s] = in.gS[s];
+            st_cell_program(g, cell);
+            st_chain_apply(g, cell, in.tv);
+#pragma unroll
+            for (int t = 0; t < QMAX; t++) {
+                const int q = lq + 4 * t;
+                if (q < K0) {
+                    float v = valid ? in.tv[t] : 0.f;
+                    if (in_div) v = __fdiv_rn(v, in_div[q]);
+                    act[lrow * ld + q] = v;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < XR; t++) {
+                const int idx = lane + t * 64;
+                if (idx < 16 * K0) {
+                    const int r = idx / K0, c = idx - r * K0;
+                    float v = in.xr[t];
+                    if (in_div) v = __fdiv_rn(v, in_div[c]);
+                    act[r * ld + c] = v;
+                }
+            }
+        }
+        for (int idx = lane; idx < 16 * (K0p - K0); idx += 64) {
+            const int r = idx / (K0p - K0), c = idx - r * (K0p - K0);
+            act[r * ld + K0 + c] = 0.f;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const float* ap = act + lrow * ld + 4 * lq;
+        for (int l = 0; l < nlayers; l++) {
+            const LayerRegs R = layer_regs(d, l);
+            v4f acc[NTMAX];
+#pragma unroll
+            for (int u = 0; u < NTMAX; u++) acc[u] = (v4f){ 0.f, 0.f, 0.f, 0.f };
+            // n-tiles in groups of four; the size of the last group is dispatched once per layer so that
+            // the k loop itself is branch-free
+#pragma unroll
+            for (int gq = 0; gq < NTMAX / 4; gq++) {
+                const int rem = R.NT - gq * 4;
+                if (rem >= 4) mma_ntiles<4, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
+                else if (rem == 3) mma_ntiles<3, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
+                else if (rem == 2) mma_ntiles<2, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
+                else if (rem == 1) mma_ntiles<1, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
+            }
+            // every read of the tile is done (the accumulators depend on them): overwrite it
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int u = 0; u < NTMAX; u++)
+                if (u < R.NT) {
+                    const int col = u * 16 + lrow;
+                    const float bv = WLDS ? sWts[R.boff + col] : wall[R.boff + col];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) act[(4 * lq + r) * ld + col] = apply_act(acc[u][r] + bv, R.act, R.alpha);
+                }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (STENCIL) {
+            gfloat* Yraw = st_g(P.Yraw);
+            if (lq == 0 && valid) {
+                StCell cell;
+#pragma unroll
+                for (int s = 0; s < ST_SCAL_MAX; s++) cell.S[s] = in.sS[s];
+                st_cell_program(sc, cell);
+                for (int q0 = 0; q0 < NO; q0 += 4) {
+                    float ov[4];
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        ov[t] = q0 + t < NO ? act[lrow * ld + q0 + t] : 0.f;
+                        if (out_mul && q0 + t < NO) ov[t] = __fmul_rn(ov[t], out_mul[q0 + t]);
+                        if (Yraw && q0 + t < NO) Yraw[(size_t)row * NO + q0 + t] = ov[t];
+                    }
+                    st_chain_apply(sc, cell, ov);
+#pragma unroll
+                    for (int t = 0; t < 4; t++)
+                        if (q0 + t < NO) {
+                            const StSlotT<float*> sl = sc.refs[q0 + t];
+                            st_g(sl.p)[st_off(sl, in.si, in.sj, in.skk)] = ov[t];
+                        }
+                }
+            }
+        } else {
+            gfloat* Y = st_g(P.Y);
+            const long base = (long)row0 * NO;
+            const long lim = (long)rows * NO - base;
+            for (int idx = lane; idx < 16 * NO; idx += 64) {
+                if (idx >= lim) break;
+                const int r = idx / NO, c = idx - r * NO;
+                float v = act[r * ld + c];
+                if (out_mul) v = __fmul_rn(v, out_mul[c]);
+                if (c >= NO - mask_tail) v = v > 0.f ? v : 0.f;
+                Y[base + idx] = v;
+            }
+        }
+        // the next tile's input overwrites the LDS tile: every lane is done reading it
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    // The grid is persistent: this wave takes tiles first, first + stride, ...  The first tile's loads
+    // are in flight while the workgroup stages the weights; after that the loads of the next tile are
+    // issued before the current one is computed.
+    const unsigned long long ntile = ((unsigned long long)rows + 15) / 16;
+    const unsigned long long stride = (unsigned long long)gridDim.x * 4;
+    unsigned long long t = (unsigned long long)blockIdx.x * 4 + wave;
+    TileIn cur, nxt;
+    if (t < ntile) issue(cur, (unsigned)(t * 16));
     if (WLDS) {
         // weights into LDS: requests batched eight at a time so their latencies overlap
         const int n4 = wfloats / 4;
@@ -315,109 +439,11 @@ void chain_wave_kernel(ChainParams params)
         }
         __syncthreads();
     }
-    // ---- the tile's input into the wave's LDS tile ------------------------------------------------------
-    if (STENCIL) {
-        StCell cell;
-#pragma unroll
-        for (int s = 0; s < ST_SCAL_MAX; s++) cell.S[s] = gS[s];
-        st_cell_program(g, cell);
-        st_chain_apply(g, cell, tv);
-#pragma unroll
-        for (int t = 0; t < QMAX; t++) {
-            const int q = lq + 4 * t;
-            if (q < K0) {
-                float v = valid ? tv[t] : 0.f;
-                if (in_div) v = __fdiv_rn(v, in_div[q]);
-                act[lrow * ld + q] = v;
-            }
-        }
-    } else {
-#pragma unroll
-        for (int t = 0; t < XR; t++) {
-            const int idx = lane + t * 64;
-            if (idx < 16 * K0) {
-                const int r = idx / K0, c = idx - r * K0;
-                float v = xr[t];
-                if (in_div) v = __fdiv_rn(v, in_div[c]);
-                act[r * ld + c] = v;
-            }
-        }
-    }
-    for (int idx = lane; idx < 16 * (K0p - K0); idx += 64) {
-        const int r = idx / (K0p - K0), c = idx - r * (K0p - K0);
-        act[r * ld + K0 + c] = 0.f;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    // ---- the layers, in place ----------------------------------------------------------------------------
-    const float* ap = act + lrow * ld + 4 * lq;
-    for (int l = 0; l < nlayers; l++) {
-        const LayerRegs R = layer_regs(d, l);
-        v4f acc[NTMAX];
-#pragma unroll
-        for (int u = 0; u < NTMAX; u++) acc[u] = (v4f){ 0.f, 0.f, 0.f, 0.f };
-        // n-tiles in groups of four; the size of the last group is dispatched once per layer so that
-        // the k loop itself is branch-free
-#pragma unroll
-        for (int gq = 0; gq < NTMAX / 4; gq++) {
-            const int rem = R.NT - gq * 4;
-            if (rem >= 4) mma_ntiles<4, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
-            else if (rem == 3) mma_ntiles<3, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
-            else if (rem == 2) mma_ntiles<2, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
-            else if (rem == 1) mma_ntiles<1, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
-        }
-        // every read of the tile is done (the accumulators depend on them): overwrite it
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int u = 0; u < NTMAX; u++)
-            if (u < R.NT) {
-                const int col = u * 16 + lrow;
-                const float bv = WLDS ? sWts[R.boff + col] : wall[R.boff + col];
-#pragma unroll
-                for (int r = 0; r < 4; r++) act[(4 * lq + r) * ld + col] = apply_act(acc[u][r] + bv, R.act, R.alpha);
-            }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-    }
-
-    // ---- results out ---------------------------------------------------------------------------------------
-    if (STENCIL) {
-        gfloat* Yraw = st_g(P.Yraw);
-        if (lq == 0 && valid) {
-            StCell cell;
-#pragma unroll
-            for (int s = 0; s < ST_SCAL_MAX; s++) cell.S[s] = sS[s];
-            st_cell_program(sc, cell);
-            for (int q0 = 0; q0 < NO; q0 += 4) {
-                float ov[4];
-#pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    ov[t] = q0 + t < NO ? act[lrow * ld + q0 + t] : 0.f;
-                    if (out_mul && q0 + t < NO) ov[t] = __fmul_rn(ov[t], out_mul[q0 + t]);
-                    if (Yraw && q0 + t < NO) Yraw[(size_t)row * NO + q0 + t] = ov[t];
-                }
-                st_chain_apply(sc, cell, ov);
-#pragma unroll
-                for (int t = 0; t < 4; t++)
-                    if (q0 + t < NO) {
-                        const StSlotT<float*> sl = sc.refs[q0 + t];
-                        st_g(sl.p)[st_off(sl, si, sj, skk)] = ov[t];
-                    }
-            }
-        }
-    } else {
-        gfloat* Y = st_g(P.Y);
-        const long base = (long)row0 * NO;
-        const long lim = (long)rows * NO - base;
-        for (int idx = lane; idx < 16 * NO; idx += 64) {
-            if (idx >= lim) break;
-            const int r = idx / NO, c = idx - r * NO;
-            float v = act[r * ld + c];
-            if (out_mul) v = __fmul_rn(v, out_mul[c]);
-            if (c >= NO - mask_tail) v = v > 0.f ? v : 0.f;
-            Y[base + idx] = v;
-        }
+    for (; t < ntile; t += stride) {
+        const bool more = t + stride < ntile;
+        if (more) issue(nxt, (unsigned)((t + stride) * 16));
+        process(cur);
+        if (more) cur = nxt;
     }
 }
 
@@ -521,7 +547,7 @@ static void launch_variant(ChainParams& P, hipStream_t s)
 static bool chain_ok(const ChainDesc& d, long rows)
 {
     if (!chain_check(d)) { fprintf(stderr, "fortis: MLP chain descriptor rejected by the kernel launcher\n"); return false; }
-    if (rows >= 4294967295L / FORTIS_CHAIN_MAX_WIDTH) { fprintf(stderr, "fortis: too many rows for one MLP chain launch\n"); return false; }
+    if (rows >= 4294967295L - 1024) { fprintf(stderr, "fortis: too many rows for one MLP chain launch\n"); return false; }
     return rows > 0;
 }
 // weights live in LDS when they leave room for at least two workgroups per CU
@@ -533,11 +559,18 @@ static void launch_wave_variant(ChainParams& P, hipStream_t s)
     const ChainDesc& d = P.d;
     const size_t shmem = ((size_t)(WLDS ? d.wfloats : 0) + (size_t)4 * 16 * d.ld) * sizeof(float);
     static size_t attr = 0;
-    if (shmem > attr) {
+    static long slots = 0;
+    if (shmem > attr || !slots) {
         HIP_OK(hipFuncSetAttribute((const void*)chain_wave_kernel<ST, WLDS, NTMAX>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         attr = shmem;
+        int occ = 0;
+        HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void*)chain_wave_kernel<ST, WLDS, NTMAX>, CH_THREADS, shmem));
+        slots = (long)(occ < 1 ? 1 : occ) * num_cus();
     }
-    hipLaunchKernelGGL((chain_wave_kernel<ST, WLDS, NTMAX>), dim3((unsigned)cdiv(P.rows, 64)), dim3(CH_THREADS), shmem, s, P);
+    // persistent grid: as many workgroups as the chip holds at once, never more than 64-row groups
+    long grid = cdiv(P.rows, 64);
+    if (grid > slots) grid = slots;
+    hipLaunchKernelGGL((chain_wave_kernel<ST, WLDS, NTMAX>), dim3((unsigned)grid), dim3(CH_THREADS), shmem, s, P);
     HIP_OK(hipGetLastError());
 }
 static int chain_ntmax(const ChainDesc& d)
