@@ -264,6 +264,10 @@ void chain_wave_kernel(ChainParams params)
     const gfloat* in_div = st_g(d.in_div);
     const gfloat* out_mul = st_g(d.out_mul);
 
+    const bool g_uniform = STENCIL && st_u(g.uniform) != 0;
+    // gather and scatter usually visit the same cells in the same order: decode a row once
+    const bool same_cells = STENCIL && st_u((int)(g.count == sc.count && g.ni == sc.ni && g.ilo == sc.ilo && g.jlo == sc.jlo &&
+                                                  g.sx == sc.sx && g.cells == sc.cells)) != 0;
     // Everything a tile reads from global memory, as registers: slot values, gather scalars, scatter
     // scalars (stencil form) or the 16 x K0 input block (plain form).
     struct TileIn {
@@ -278,22 +282,33 @@ void chain_wave_kernel(ChainParams params)
         if (STENCIL) {
             const unsigned row = row0 + lrow;
             const unsigned rc = row < rows ? row : 0;
-            const int kk = (int)(rc / g.count);
-            int i, j;
-            st_cell(g, rc % g.count, i, j);
+            int i, j, kk;
+            st_row(g, rc, i, j, kk);
+            if (same_cells) { in.si = i; in.sj = j; in.skk = kk; }
+            else st_row(sc, rc, in.si, in.sj, in.skk);
+            if (g_uniform) {
+                // one element offset per cell; a slot is then its pointer plus that offset
+                const long off = st_off(g.refs[0], i, j, kk);
 #pragma unroll
-            for (int t = 0; t < QMAX; t++) {
-                const int q = lq + 4 * t;
-                const StSlotT<const float*> sl = g.refs[q < K0 ? q : 0];
-                in.tv[t] = st_g(sl.p)[st_off(sl, i, j, kk)];
-            }
+                for (int t = 0; t < QMAX; t++) {
+                    const int q = lq + 4 * t;
+                    in.tv[t] = st_g(g.refs[q < K0 ? q : 0].p)[off];
+                }
 #pragma unroll
-            for (int s = 0; s < ST_SCAL_MAX; s++) {
-                const StSlotT<const float*> sl = g.scal[s < g.nscal ? s : 0];
-                in.gS[s] = st_g(sl.p)[st_off(sl, i, j, kk)];
+                for (int s = 0; s < ST_SCAL_MAX; s++) in.gS[s] = st_g(g.scal[s < g.nscal ? s : 0].p)[off];
+            } else {
+#pragma unroll
+                for (int t = 0; t < QMAX; t++) {
+                    const int q = lq + 4 * t;
+                    const StSlotT<const float*> sl = g.refs[q < K0 ? q : 0];
+                    in.tv[t] = st_g(sl.p)[st_off(sl, i, j, kk)];
+                }
+#pragma unroll
+                for (int s = 0; s < ST_SCAL_MAX; s++) {
+                    const StSlotT<const float*> sl = g.scal[s < g.nscal ? s : 0];
+                    in.gS[s] = st_g(sl.p)[st_off(sl, i, j, kk)];
+                }
             }
-            in.skk = (int)(rc / sc.count);
-            st_cell(sc, rc % sc.count, in.si, in.sj);
 #pragma unroll
             for (int s = 0; s < ST_SCAL_MAX; s++) {
                 const StSlotT<float*> sl = sc.scal[s < sc.nscal ? s : 0];
@@ -366,14 +381,20 @@ void chain_wave_kernel(ChainParams params)
             // every read of the tile is done (the accumulators depend on them): overwrite it
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
             __builtin_amdgcn_wave_barrier();
+            auto write_back = [&](auto actf) __attribute__((always_inline)) {
 #pragma unroll
-            for (int u = 0; u < NTMAX; u++)
-                if (u < R.NT) {
-                    const int col = u * 16 + lrow;
-                    const float bv = WLDS ? sWts[R.boff + col] : wall[R.boff + col];
+                for (int u = 0; u < NTMAX; u++)
+                    if (u < R.NT) {
+                        const int col = u * 16 + lrow;
+                        const float bv = WLDS ? sWts[R.boff + col] : wall[R.boff + col];
 #pragma unroll
-                    for (int r = 0; r < 4; r++) act[(4 * lq + r) * ld + col] = apply_act(acc[u][r] + bv, R.act, R.alpha);
-                }
+                        for (int r = 0; r < 4; r++) act[(4 * lq + r) * ld + col] = actf(acc[u][r] + bv);
+                    }
+            };
+            // the activation is chosen once per layer, not per element
+            if (R.act == FORTIS_ACT_RELU) write_back([](float v) { return fmaxf(v, 0.f); });
+            else if (R.act == FORTIS_ACT_NONE) write_back([](float v) { return v; });
+            else write_back([&](float v) { return apply_act(v, R.act, R.alpha); });
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
             __builtin_amdgcn_wave_barrier();
         }

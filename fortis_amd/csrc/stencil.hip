@@ -25,10 +25,8 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
     const int tid = threadIdx.x;
     const unsigned row0 = blockIdx.x * ST_THREADS, row = row0 + tid;
     if (row < rows) {
-        const unsigned col = row % d.count;
-        const int kk = (int)(row / d.count);
-        int i, j;
-        st_cell(d, col, i, j);
+        int i, j, kk;
+        st_row(d, row, i, j, kk);
         // all slot loads are issued before any of them is consumed
         float tv[FORTIS_MAX_REFS];
 #pragma unroll

@@ -36,6 +36,26 @@ __device__ __forceinline__ int st_u(int v) { return __builtin_amdgcn_readfirstla
 struct StIns { int op, a, b; float ca, cb; };          // per-cell instruction, constants inlined
 struct StStep { int op, code, tv_left; float cv; };    // tv chain step, constant inlined
 
+// Exact unsigned division by a divisor fixed for the launch: q = (n * m) >> 64 with m = ceil(2^64 / d),
+// exact for every 32-bit n (n * (m d - 2^64) < 2^64).  d == 1 has no 64-bit m and is flagged.
+struct StMagic { unsigned mh, ml, d, one; };
+static inline StMagic st_magic(unsigned d)
+{
+    StMagic m = { 0u, 0u, d ? d : 1u, d <= 1u ? 1u : 0u };
+    if (!m.one) {
+        const unsigned __int128 v = (((unsigned __int128)1 << 64) + d - 1) / d;
+        m.mh = (unsigned)(v >> 32); m.ml = (unsigned)v;
+    }
+    return m;
+}
+__device__ __forceinline__ void st_divmod(unsigned n, const StMagic& m, unsigned& q, unsigned& r)
+{
+    if (st_u((int)m.one)) { q = n; r = 0; return; }
+    const unsigned long long t = (unsigned long long)n * m.mh + __umulhi(n, m.ml);
+    q = (unsigned)(t >> 32);
+    r = n - q * m.d;
+}
+
 template <typename P>
 struct alignas(16) StencilArgsT {
     int nrefs, nscal, ncell, nchain;
@@ -46,6 +66,9 @@ struct alignas(16) StencilArgsT {
     unsigned count;
     int ilo, jlo, ni, sx;
     const int* cells;
+    StMagic mcount, mni, msx;   // exact division by count, ni, sx
+    int uniform;                // every slot and scalar has the same (si, sj, plane): one offset per cell
+    int pad_[3];
 };
 typedef StencilArgsT<const float*> GatherArgs;
 typedef StencilArgsT<float*> ScatterArgs;
@@ -54,8 +77,18 @@ typedef StencilArgsT<float*> ScatterArgs;
 template <typename A>
 __device__ __forceinline__ void st_cell(const A& d, unsigned col, int& i, int& j)
 {
-    if (d.cells) { const unsigned c = (unsigned)((const __attribute__((address_space(1))) int*)d.cells)[col]; i = 1 + (int)(c % (unsigned)d.sx); j = 1 + (int)(c / (unsigned)d.sx); }
-    else { i = d.ilo + (int)(col % (unsigned)d.ni); j = d.jlo + (int)(col / (unsigned)d.ni); }
+    unsigned q, r;
+    if (d.cells) { const unsigned c = (unsigned)((const __attribute__((address_space(1))) int*)d.cells)[col]; st_divmod(c, d.msx, q, r); i = 1 + (int)r; j = 1 + (int)q; }
+    else { st_divmod(col, d.mni, q, r); i = d.ilo + (int)r; j = d.jlo + (int)q; }
+}
+// row of the flattened (cell, iteration) space -> iteration kk and 1-based (i, j)
+template <typename A>
+__device__ __forceinline__ void st_row(const A& d, unsigned row, int& i, int& j, int& kk)
+{
+    unsigned q, col;
+    st_divmod(row, d.mcount, q, col);
+    kk = (int)q;
+    st_cell(d, col, i, j);
 }
 template <typename S>
 __device__ __forceinline__ long st_off(const S& r, int i, int j, int kk)
@@ -177,4 +210,12 @@ static inline void st_make_args(const StencilDev& low, const int* dcells, P cons
     a->count = (unsigned)low.count;
     a->ilo = low.ilo; a->jlo = low.jlo; a->ni = low.ni; a->sx = low.sx;
     a->cells = dcells;
+    a->mcount = st_magic((unsigned)low.count);
+    a->mni = st_magic((unsigned)(low.ni > 0 ? low.ni : 1));
+    a->msx = st_magic((unsigned)(low.sx > 0 ? low.sx : 1));
+    a->uniform = 1;
+    for (int r = 0; r < low.nrefs; r++)
+        if (a->refs[r].si != a->refs[0].si || a->refs[r].sj != a->refs[0].sj || a->refs[r].plane != a->refs[0].plane) a->uniform = 0;
+    for (int r = 0; r < low.nscal; r++)
+        if (a->scal[r].si != a->refs[0].si || a->scal[r].sj != a->refs[0].sj || a->scal[r].plane != a->refs[0].plane) a->uniform = 0;
 }
