@@ -204,48 +204,59 @@ void chain_kernel(ChainParams params)
     }
 }
 
-// One m-tile (16 rows at ap) times NT n-tiles starting at nt0, NT known at compile time: no branch
-// inside the k loop, MFMAs interleaved over the NT independent accumulators.
-template <int NT, bool WLDS>
-__device__ __forceinline__ void mma_ntiles(const float* ap, const float* sWts, const gfloat* wall, int woff4, int nt0,
-                                           int KG, int lane, v4f* acc)
+// NTG n-tiles (starting at nt0) of one layer for the wave's 16 rows, in registers.
+// The product is formed transposed, D = W . X^T: the weights are the MFMA's A operand and the rows'
+// activations its B operand, so a lane ends up with features n = 16 nt + 4 (lane / 16) + r, r = 0..3, of
+// row lane % 16 -- exactly the four consecutive k a lane must supply for k group nt of the NEXT layer.
+// A layer's output registers are therefore the next layer's input registers: no LDS round trip, no
+// barrier between layers.  The accumulators start at the bias.
+template <int NTG, int KGMAX, bool WLDS>
+__device__ __forceinline__ void layer_group(const v4f (&a)[KGMAX], v4f* o, const float* sWts, const gfloat* wall,
+                                            int woff4, int boff, int nt0, int KG, int lane, int lq)
 {
+    v4f acc[NTG];
 #pragma unroll
-    for (int u = 0; u < NT; u++) acc[u] = (v4f){ 0.f, 0.f, 0.f, 0.f };
-#pragma unroll 2
-    for (int kg = 0; kg < KG; kg++) {
-        const v4f a = *(const v4f*)(ap + kg * 16);
-        v4f b[NT];
-#pragma unroll
-        for (int u = 0; u < NT; u++) {
-            const int off = woff4 + ((nt0 + u) * KG + kg) * 64 + lane;
-            if (WLDS) b[u] = ((const v4f*)sWts)[off]; else b[u] = ((const gv4f*)wall)[off];
-        }
-#pragma unroll
-        for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b[u].x, acc[u], 0, 0, 0);
-#pragma unroll
-        for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b[u].y, acc[u], 0, 0, 0);
-#pragma unroll
-        for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b[u].z, acc[u], 0, 0, 0);
-#pragma unroll
-        for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b[u].w, acc[u], 0, 0, 0);
+    for (int u = 0; u < NTG; u++) {
+        const int bo = (boff + (nt0 + u) * 16) / 4 + lq;
+        if (WLDS) acc[u] = ((const v4f*)sWts)[bo]; else acc[u] = ((const gv4f*)wall)[bo];
     }
+#pragma unroll
+    for (int kg = 0; kg < KGMAX; kg++) {
+        if (kg < KG) {
+            v4f w[NTG];
+#pragma unroll
+            for (int u = 0; u < NTG; u++) {
+                const int off = woff4 + ((nt0 + u) * KG + kg) * 64 + lane;
+                if (WLDS) w[u] = ((const v4f*)sWts)[off]; else w[u] = ((const gv4f*)wall)[off];
+            }
+#pragma unroll
+            for (int u = 0; u < NTG; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].x, a[kg].x, acc[u], 0, 0, 0);
+#pragma unroll
+            for (int u = 0; u < NTG; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].y, a[kg].y, acc[u], 0, 0, 0);
+#pragma unroll
+            for (int u = 0; u < NTG; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].z, a[kg].z, acc[u], 0, 0, 0);
+#pragma unroll
+            for (int u = 0; u < NTG; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].w, a[kg].w, acc[u], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < NTG; u++) o[u] = acc[u];
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Wave-independent variant: ONE WAVE owns 16 rows from the gather (or the X load) to the scatter (or
-// the Y store).  Every layer is computed in place in the wave's private 16 x ld LDS tile (all n-tiles
-// are accumulated in registers before anything is written back), so no workgroup barrier separates
-// the layers and the waves of a CU drift apart: while one waits for its slot loads another runs its
-// MFMAs.  The four waves of a workgroup only share the LDS copies of the parameter block and of the
-// weights.  All global loads a wave needs (slot values, gather scalars, scatter scalars) are issued
-// up front, before the weights are staged.
+// Wave-independent, register-resident variant: ONE WAVE owns 16 rows from the gather (or the X load)
+// to the scatter (or the Y store), and the activations never leave its registers (see layer_group).
+// Lane (row = lane % 16, q = lane / 16) holds, per 16-wide k group, the four features 4q..4q+3 of its
+// row: the gather loads exactly those slots, the last layer leaves exactly those outputs.  The four
+// waves of a workgroup only share the LDS copies of the parameter block and of the weights.  The grid
+// is persistent; the global loads of a wave's next tile are issued before the current one is computed.
 template <bool STENCIL, bool WLDS, int NTMAX>
-__global__ __launch_bounds__(CH_THREADS) __attribute__((amdgpu_waves_per_eu(1, 4)))
+__global__ __launch_bounds__(CH_THREADS) __attribute__((amdgpu_waves_per_eu(NTMAX <= 4 ? 4 : 2, NTMAX <= 4 ? 4 : 2)))
 void chain_wave_kernel(ChainParams params)
 {
-    constexpr int QMAX = FORTIS_MAX_REFS / 4;
-    constexpr int XR = 16;                                      // plain: 16 rows x K0 <= 64 floats = 16 per lane
+    constexpr int KG0 = STENCIL ? FORTIS_MAX_REFS / 16 : NTMAX;   // k groups the first layer can read
+    constexpr bool PREFETCH = KG0 <= 4;                           // wide inputs: no second register set
+    constexpr int NTO = STENCIL ? FORTIS_MAX_REFS / 16 : NTMAX;   // n-tiles the output stage can write
     __shared__ ChainParams P;
     extern __shared__ float4 smem4[];
     params_to_lds(&P, CH_THREADS);
@@ -253,25 +264,27 @@ void chain_wave_kernel(ChainParams params)
     const GatherArgs& g = P.g;
     const ScatterArgs& sc = P.sc;
     float* sWts = (float*)smem4;
-    const int wfloats = st_u(d.wfloats), ld = st_u(d.ld), nlayers = st_u(d.nlayers);
+    const int wfloats = st_u(d.wfloats), nlayers = st_u(d.nlayers);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    float* act = sWts + (WLDS ? wfloats : 0) + wave * 16 * ld;
-    const int K0 = st_u(d.L[0].K), K0p = st_u(d.L[0].Kp);
+    const int K0 = st_u(d.L[0].K);
     const int NO = st_u(d.L[nlayers - 1].N), mask_tail = st_u(d.mask_tail);
-    const unsigned rows = P.rows;
+    const unsigned rows = (unsigned)st_u((int)P.rows);
     const int lrow = lane & 15, lq = lane >> 4;
     const gfloat* wall = st_g(d.wall);
     const gfloat* in_div = st_g(d.in_div);
     const gfloat* out_mul = st_g(d.out_mul);
-
     const bool g_uniform = STENCIL && st_u(g.uniform) != 0;
     // gather and scatter usually visit the same cells in the same order: decode a row once
     const bool same_cells = STENCIL && st_u((int)(g.count == sc.count && g.ni == sc.ni && g.ilo == sc.ilo && g.jlo == sc.jlo &&
                                                   g.sx == sc.sx && g.cells == sc.cells)) != 0;
-    // Everything a tile reads from global memory, as registers: slot values, gather scalars, scatter
-    // scalars (stencil form) or the 16 x K0 input block (plain form).
+    const bool xvec = !STENCIL && st_u((int)((K0 & 3) == 0 && ((uintptr_t)P.X & 15) == 0)) != 0;   // 16-byte X loads
+    const bool yvec = !STENCIL && st_u((int)((NO & 3) == 0 && ((uintptr_t)P.Y & 15) == 0)) != 0;   // 16-byte Y stores
+
+    // Everything a tile reads from global memory, as registers: the first layer's operand (slot values
+    // or X), and for the stencil form the gather scalars and scatter scalars of the lane's cell.
     struct TileIn {
-        float tv[QMAX], gS[ST_SCAL_MAX], sS[ST_SCAL_MAX], xr[XR];
+        v4f x[KG0];
+        float gS[ST_SCAL_MAX], sS[ST_SCAL_MAX];
         int si, sj, skk;
         unsigned row0;
     };
@@ -279,8 +292,8 @@ void chain_wave_kernel(ChainParams params)
     auto issue = [&](TileIn& in, unsigned row0) __attribute__((always_inline)) {
         in.row0 = row0;
         in.si = in.sj = in.skk = 0;
+        const unsigned row = row0 + lrow;
         if (STENCIL) {
-            const unsigned row = row0 + lrow;
             const unsigned rc = row < rows ? row : 0;
             int i, j, kk;
             st_row(g, rc, i, j, kk);
@@ -290,19 +303,23 @@ void chain_wave_kernel(ChainParams params)
                 // one element offset per cell; a slot is then its pointer plus that offset
                 const long off = st_off(g.refs[0], i, j, kk);
 #pragma unroll
-                for (int t = 0; t < QMAX; t++) {
-                    const int q = lq + 4 * t;
-                    in.tv[t] = st_g(g.refs[q < K0 ? q : 0].p)[off];
-                }
+                for (int kg = 0; kg < KG0; kg++)
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; s4++) {
+                        const int q = 16 * kg + 4 * lq + s4;
+                        in.x[kg][s4] = st_g(g.refs[q < K0 ? q : 0].p)[off];
+                    }
 #pragma unroll
                 for (int s = 0; s < ST_SCAL_MAX; s++) in.gS[s] = st_g(g.scal[s < g.nscal ? s : 0].p)[off];
             } else {
 #pragma unroll
-                for (int t = 0; t < QMAX; t++) {
-                    const int q = lq + 4 * t;
-                    const StSlotT<const float*> sl = g.refs[q < K0 ? q : 0];
-                    in.tv[t] = st_g(sl.p)[st_off(sl, i, j, kk)];
-                }
+                for (int kg = 0; kg < KG0; kg++)
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; s4++) {
+                        const int q = 16 * kg + 4 * lq + s4;
+                        const StSlotT<const float*> sl = g.refs[q < K0 ? q : 0];
+                        in.x[kg][s4] = st_g(sl.p)[st_off(sl, i, j, kk)];
+                    }
 #pragma unroll
                 for (int s = 0; s < ST_SCAL_MAX; s++) {
                     const StSlotT<const float*> sl = g.scal[s < g.nscal ? s : 0];
@@ -315,139 +332,133 @@ void chain_wave_kernel(ChainParams params)
                 in.sS[s] = st_g(sl.p)[st_off(sl, in.si, in.sj, in.skk)];
             }
         } else {
-            const gfloat* X = st_g(P.X);
-            const long base = (long)row0 * K0;
-            const long lim = (long)rows * K0 - base;
+            const gfloat* xrow = st_g(P.X) + (size_t)(row < rows ? row : 0) * K0;
 #pragma unroll
-            for (int t = 0; t < XR; t++) {
-                const int idx = lane + t * 64;
-                in.xr[t] = (idx < 16 * K0 && idx < lim) ? X[base + idx] : 0.f;
+            for (int kg = 0; kg < KG0; kg++) {
+                const int c = 16 * kg + 4 * lq;
+                if (xvec) {
+                    in.x[kg] = c < K0 ? *(const gv4f*)(xrow + c) : (v4f)(0.f);
+                } else {
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; s4++) in.x[kg][s4] = c + s4 < K0 ? xrow[c + s4] : 0.f;
+                }
             }
         }
     };
-    // ---- one tile: input into the wave's LDS tile, the layers in place, results out --------------------
+    // ---- one tile: first operand from the loaded values, the layers in registers, results out ----------
     auto process = [&](TileIn& in) __attribute__((always_inline)) {
-        const unsigned row0 = in.row0, row = row0 + lrow;
+        const unsigned row = in.row0 + lrow;
         const bool valid = row < rows;
+        v4f a[NTMAX], o[NTMAX];
+#pragma unroll
+        for (int kg = 0; kg < NTMAX; kg++) a[kg] = (v4f)(0.f);
         if (STENCIL) {
             StCell cell;
 #pragma unroll
             for (int s = 0; s < ST_SCAL_MAX; s++) cell.S[s] = in.gS[s];
             st_cell_program(g, cell);
-            st_chain_apply(g, cell, in.tv);
+            float tv[KG0 * 4];
 #pragma unroll
-            for (int t = 0; t < QMAX; t++) {
-                const int q = lq + 4 * t;
-                if (q < K0) {
-                    float v = valid ? in.tv[t] : 0.f;
-                    if (in_div) v = __fdiv_rn(v, in_div[q]);
-                    act[lrow * ld + q] = v;
-                }
+            for (int t = 0; t < KG0 * 4; t++) tv[t] = in.x[t >> 2][t & 3];
+            st_chain_apply(g, cell, tv);
+#pragma unroll
+            for (int t = 0; t < KG0 * 4; t++) {
+                const int q = 16 * (t >> 2) + 4 * lq + (t & 3);
+                float v = (valid && q < K0) ? tv[t] : 0.f;
+                if (in_div && q < K0) v = __fdiv_rn(v, in_div[q]);
+                if ((t >> 2) < NTMAX) a[(t >> 2) < NTMAX ? (t >> 2) : 0][t & 3] = v;
             }
         } else {
 #pragma unroll
-            for (int t = 0; t < XR; t++) {
-                const int idx = lane + t * 64;
-                if (idx < 16 * K0) {
-                    const int r = idx / K0, c = idx - r * K0;
-                    float v = in.xr[t];
-                    if (in_div) v = __fdiv_rn(v, in_div[c]);
-                    act[r * ld + c] = v;
-                }
-            }
-        }
-        for (int idx = lane; idx < 16 * (K0p - K0); idx += 64) {
-            const int r = idx / (K0p - K0), c = idx - r * (K0p - K0);
-            act[r * ld + K0 + c] = 0.f;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        const float* ap = act + lrow * ld + 4 * lq;
-        for (int l = 0; l < nlayers; l++) {
-            const LayerRegs R = layer_regs(d, l);
-            v4f acc[NTMAX];
+            for (int kg = 0; kg < KG0; kg++)
 #pragma unroll
-            for (int u = 0; u < NTMAX; u++) acc[u] = (v4f){ 0.f, 0.f, 0.f, 0.f };
-            // n-tiles in groups of four; the size of the last group is dispatched once per layer so that
-            // the k loop itself is branch-free
+                for (int s4 = 0; s4 < 4; s4++) {
+                    const int c = 16 * kg + 4 * lq + s4;
+                    float v = (valid && c < K0) ? in.x[kg][s4] : 0.f;
+                    if (in_div && c < K0) v = __fdiv_rn(v, in_div[c]);
+                    a[kg][s4] = v;
+                }
+        }
+        for (int l = 0; l < nlayers; l++) {
+            asm volatile("" ::: "memory");
+            const LayerRegs R = layer_regs(d, l);
+            // n-tiles in groups of four independent accumulators; the size of the last group is
+            // dispatched once per layer
 #pragma unroll
             for (int gq = 0; gq < NTMAX / 4; gq++) {
                 const int rem = R.NT - gq * 4;
-                if (rem >= 4) mma_ntiles<4, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
-                else if (rem == 3) mma_ntiles<3, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
-                else if (rem == 2) mma_ntiles<2, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
-                else if (rem == 1) mma_ntiles<1, WLDS>(ap, sWts, wall, R.woff / 4, gq * 4, R.KG, lane, acc + gq * 4);
+                if (rem >= 4) layer_group<4, NTMAX, WLDS>(a, o + gq * 4, sWts, wall, R.woff / 4, R.boff, gq * 4, R.KG, lane, lq);
+                else if (rem == 3) layer_group<3, NTMAX, WLDS>(a, o + gq * 4, sWts, wall, R.woff / 4, R.boff, gq * 4, R.KG, lane, lq);
+                else if (rem == 2) layer_group<2, NTMAX, WLDS>(a, o + gq * 4, sWts, wall, R.woff / 4, R.boff, gq * 4, R.KG, lane, lq);
+                else if (rem == 1) layer_group<1, NTMAX, WLDS>(a, o + gq * 4, sWts, wall, R.woff / 4, R.boff, gq * 4, R.KG, lane, lq);
             }
-            // every read of the tile is done (the accumulators depend on them): overwrite it
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            auto write_back = [&](auto actf) __attribute__((always_inline)) {
+            // activation, chosen once per layer; the outputs become the next layer's operand
+            auto next_in = [&](auto actf) __attribute__((always_inline)) {
 #pragma unroll
                 for (int u = 0; u < NTMAX; u++)
-                    if (u < R.NT) {
-                        const int col = u * 16 + lrow;
-                        const float bv = WLDS ? sWts[R.boff + col] : wall[R.boff + col];
 #pragma unroll
-                        for (int r = 0; r < 4; r++) act[(4 * lq + r) * ld + col] = actf(acc[u][r] + bv);
-                    }
+                    for (int r = 0; r < 4; r++) a[u][r] = u < R.NT ? actf(o[u][r]) : 0.f;
             };
-            // the activation is chosen once per layer, not per element
-            if (R.act == FORTIS_ACT_RELU) write_back([](float v) { return fmaxf(v, 0.f); });
-            else if (R.act == FORTIS_ACT_NONE) write_back([](float v) { return v; });
-            else write_back([&](float v) { return apply_act(v, R.act, R.alpha); });
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();
+            if (R.act == FORTIS_ACT_RELU) next_in([](float v) { return fmaxf(v, 0.f); });
+            else if (R.act == FORTIS_ACT_NONE) next_in([](float v) { return v; });
+            else next_in([&](float v) { return apply_act(v, R.act, R.alpha); });
         }
+        // ---- results out: the lane holds outputs n = 16 nt + 4 lq + r of its row ----------------------
+        asm volatile("" ::: "memory");
         if (STENCIL) {
             gfloat* Yraw = st_g(P.Yraw);
-            if (lq == 0 && valid) {
-                StCell cell;
+            StCell cell;
 #pragma unroll
-                for (int s = 0; s < ST_SCAL_MAX; s++) cell.S[s] = in.sS[s];
-                st_cell_program(sc, cell);
-                for (int q0 = 0; q0 < NO; q0 += 4) {
-                    float ov[4];
+            for (int s = 0; s < ST_SCAL_MAX; s++) cell.S[s] = in.sS[s];
+            st_cell_program(sc, cell);
 #pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        ov[t] = q0 + t < NO ? act[lrow * ld + q0 + t] : 0.f;
-                        if (out_mul && q0 + t < NO) ov[t] = __fmul_rn(ov[t], out_mul[q0 + t]);
-                        if (Yraw && q0 + t < NO) Yraw[(size_t)row * NO + q0 + t] = ov[t];
+            for (int nt = 0; nt < (NTO < NTMAX ? NTO : NTMAX); nt++) {
+                if (nt * 16 >= NO) break;
+                float ov[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int n = nt * 16 + 4 * lq + r;
+                    ov[r] = a[nt][r];
+                    if (out_mul && n < NO) ov[r] = __fmul_rn(ov[r], out_mul[n]);
+                    if (Yraw && valid && n < NO) Yraw[(size_t)row * NO + n] = ov[r];
+                }
+                st_chain_apply(sc, cell, ov);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int n = nt * 16 + 4 * lq + r;
+                    if (valid && n < NO) {
+                        const StSlotT<float*> sl = sc.refs[n];
+                        st_g(sl.p)[st_off(sl, in.si, in.sj, in.skk)] = ov[r];
                     }
-                    st_chain_apply(sc, cell, ov);
-#pragma unroll
-                    for (int t = 0; t < 4; t++)
-                        if (q0 + t < NO) {
-                            const StSlotT<float*> sl = sc.refs[q0 + t];
-                            st_g(sl.p)[st_off(sl, in.si, in.sj, in.skk)] = ov[t];
-                        }
                 }
             }
         } else {
-            gfloat* Y = st_g(P.Y);
-            const long base = (long)row0 * NO;
-            const long lim = (long)rows * NO - base;
-            for (int idx = lane; idx < 16 * NO; idx += 64) {
-                if (idx >= lim) break;
-                const int r = idx / NO, c = idx - r * NO;
-                float v = act[r * ld + c];
-                if (out_mul) v = __fmul_rn(v, out_mul[c]);
-                if (c >= NO - mask_tail) v = v > 0.f ? v : 0.f;
-                Y[base + idx] = v;
+            gfloat* yrow = st_g(P.Y) + (size_t)row * NO;
+#pragma unroll
+            for (int nt = 0; nt < NTMAX; nt++) {
+                if (nt * 16 >= NO) break;
+                const int n0 = nt * 16 + 4 * lq;
+                v4f v = a[nt];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (out_mul && n0 + r < NO) v[r] = __fmul_rn(v[r], out_mul[n0 + r]);
+                    if (n0 + r >= NO - mask_tail) v[r] = v[r] > 0.f ? v[r] : 0.f;
+                }
+                if (!valid) continue;
+                if (yvec) { if (n0 < NO) *(gv4f*)(yrow + n0) = v; }
+                else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) if (n0 + r < NO) yrow[n0 + r] = v[r];
+                }
             }
         }
-        // the next tile's input overwrites the LDS tile: every lane is done reading it
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
     };
 
-    // The grid is persistent: this wave takes tiles first, first + stride, ...  The first tile's loads
-    // are in flight while the workgroup stages the weights; after that the loads of the next tile are
-    // issued before the current one is computed.
     const unsigned long long ntile = ((unsigned long long)rows + 15) / 16;
     const unsigned long long stride = (unsigned long long)gridDim.x * 4;
     unsigned long long t = (unsigned long long)blockIdx.x * 4 + wave;
     TileIn cur, nxt;
-    if (t < ntile) issue(cur, (unsigned)(t * 16));
+    if (t < ntile) issue(cur, (unsigned)(t * 16));      // in flight while the weights are staged
     if (WLDS) {
         // weights into LDS: requests batched eight at a time so their latencies overlap
         const int n4 = wfloats / 4;
@@ -461,10 +472,18 @@ void chain_wave_kernel(ChainParams params)
         __syncthreads();
     }
     for (; t < ntile; t += stride) {
+        // Table values (slot pointers, strides, layer shapes) are re-read from LDS per tile: hoisted out of
+        // this loop they would occupy more registers than the tile itself.
+        asm volatile("" ::: "memory");
         const bool more = t + stride < ntile;
-        if (more) issue(nxt, (unsigned)((t + stride) * 16));
-        process(cur);
-        if (more) cur = nxt;
+        if (PREFETCH) {
+            if (more) issue(nxt, (unsigned)((t + stride) * 16));
+            process(cur);
+            if (more) cur = nxt;
+        } else {
+            process(cur);
+            if (more) issue(cur, (unsigned)((t + stride) * 16));
+        }
     }
 }
 
@@ -578,7 +597,7 @@ template <bool ST, bool WLDS, int NTMAX>
 static void launch_wave_variant(ChainParams& P, hipStream_t s)
 {
     const ChainDesc& d = P.d;
-    const size_t shmem = ((size_t)(WLDS ? d.wfloats : 0) + (size_t)4 * 16 * d.ld) * sizeof(float);
+    const size_t shmem = (size_t)(WLDS ? d.wfloats : 0) * sizeof(float);
     static size_t attr = 0;
     static long slots = 0;
     if (shmem > attr || !slots) {
@@ -596,7 +615,7 @@ static void launch_wave_variant(ChainParams& P, hipStream_t s)
 }
 static int chain_ntmax(const ChainDesc& d)
 {
-    int nt = 0;
+    int nt = d.L[0].Kp / 16;
     for (int l = 0; l < d.nlayers; l++) if (d.L[l].Np / 16 > nt) nt = d.L[l].Np / 16;
     return nt;
 }
@@ -606,7 +625,7 @@ static bool chain_wave_wlds(const ChainDesc& d)
     static int force = -2;
     if (force == -2) { const char* e = getenv("FORTIS_CHAIN_WLDS"); force = e ? atoi(e) : -1; }
     if (force >= 0) return force != 0;
-    return ((size_t)d.wfloats + 4 * 16 * d.ld) * sizeof(float) + sizeof(ChainParams) <= 52 * 1024;
+    return (size_t)d.wfloats * sizeof(float) + sizeof(ChainParams) <= 52 * 1024;
 }
 
 template <bool ST>
@@ -628,7 +647,7 @@ void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows
     ChainParams P;
     fill_params(&P, d, X, Y, rows, nullptr);
     // many rows of a narrow input: the wave-independent kernel
-    if (rows >= 64L * num_cus() && d.L[0].K <= 64) { launch_wave<false>(P, s); return; }
+    if (rows >= 64L * num_cus()) { launch_wave<false>(P, s); return; }
     const bool wlds = chain_wlds(d);
     // few rows: 16-row tiles spread the work over more CUs (the four waves then split the n-tiles)
     if (rows < 64L * num_cus()) {
