@@ -274,6 +274,7 @@ void chain_wave_kernel(ChainParams params)
     const gfloat* in_div = st_g(d.in_div);
     const gfloat* out_mul = st_g(d.out_mul);
     const bool g_uniform = STENCIL && st_u(g.uniform) != 0;
+    const bool s_uniform = STENCIL && st_u(sc.uniform) != 0;
     // gather and scatter usually visit the same cells in the same order: decode a row once
     const bool same_cells = STENCIL && st_u((int)(g.count == sc.count && g.ni == sc.ni && g.ilo == sc.ilo && g.jlo == sc.jlo &&
                                                   g.sx == sc.sx && g.cells == sc.cells)) != 0;
@@ -307,10 +308,10 @@ void chain_wave_kernel(ChainParams params)
 #pragma unroll
                     for (int s4 = 0; s4 < 4; s4++) {
                         const int q = 16 * kg + 4 * lq + s4;
-                        in.x[kg][s4] = st_g(g.refs[q < K0 ? q : 0].p)[off];
+                        in.x[kg][s4] = st_g(g.refs[q].p)[off];      // entries past nrefs repeat slot 0
                     }
 #pragma unroll
-                for (int s = 0; s < ST_SCAL_MAX; s++) in.gS[s] = st_g(g.scal[s < g.nscal ? s : 0].p)[off];
+                for (int s = 0; s < ST_SCAL_MAX; s++) in.gS[s] = st_g(g.scal[s].p)[off];
             } else {
 #pragma unroll
                 for (int kg = 0; kg < KG0; kg++)
@@ -326,10 +327,16 @@ void chain_wave_kernel(ChainParams params)
                     in.gS[s] = st_g(sl.p)[st_off(sl, i, j, kk)];
                 }
             }
+            if (s_uniform) {
+                const long off = st_off(sc.refs[0], in.si, in.sj, in.skk);
 #pragma unroll
-            for (int s = 0; s < ST_SCAL_MAX; s++) {
-                const StSlotT<float*> sl = sc.scal[s < sc.nscal ? s : 0];
-                in.sS[s] = st_g(sl.p)[st_off(sl, in.si, in.sj, in.skk)];
+                for (int s = 0; s < ST_SCAL_MAX; s++) in.sS[s] = st_g(sc.scal[s].p)[off];
+            } else {
+#pragma unroll
+                for (int s = 0; s < ST_SCAL_MAX; s++) {
+                    const StSlotT<float*> sl = sc.scal[s];
+                    in.sS[s] = st_g(sl.p)[st_off(sl, in.si, in.sj, in.skk)];
+                }
             }
         } else {
             const gfloat* xrow = st_g(P.X) + (size_t)(row < rows ? row : 0) * K0;
@@ -395,9 +402,9 @@ void chain_wave_kernel(ChainParams params)
             // activation, chosen once per layer; the outputs become the next layer's operand
             auto next_in = [&](auto actf) __attribute__((always_inline)) {
 #pragma unroll
-                for (int u = 0; u < NTMAX; u++)
+                for (int u = 0; u < NTMAX; u++)      // tiles past R.NT hold stale values no later stage reads
 #pragma unroll
-                    for (int r = 0; r < 4; r++) a[u][r] = u < R.NT ? actf(o[u][r]) : 0.f;
+                    for (int r = 0; r < 4; r++) a[u][r] = actf(o[u][r]);
             };
             if (R.act == FORTIS_ACT_RELU) next_in([](float v) { return fmaxf(v, 0.f); });
             else if (R.act == FORTIS_ACT_NONE) next_in([](float v) { return v; });
@@ -423,12 +430,13 @@ void chain_wave_kernel(ChainParams params)
                     if (Yraw && valid && n < NO) Yraw[(size_t)row * NO + n] = ov[r];
                 }
                 st_chain_apply(sc, cell, ov);
+                const long soff = st_off(sc.refs[0], in.si, in.sj, in.skk);
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int n = nt * 16 + 4 * lq + r;
                     if (valid && n < NO) {
                         const StSlotT<float*> sl = sc.refs[n];
-                        st_g(sl.p)[st_off(sl, in.si, in.sj, in.skk)] = ov[r];
+                        st_g(sl.p)[s_uniform ? soff : st_off(sl, in.si, in.sj, in.skk)] = ov[r];
                     }
                 }
             }

@@ -206,7 +206,9 @@ static inline void st_make_args(const StencilDev& low, const int* dcells, P cons
         StStep s = { low.chain[n].op, low.chain[n].code, low.chain[n].tv_left, cval(low.chain[n].code) };
         a->chain[n] = s;
     }
-    if (low.nscal == 0) { a->scal[0].p = a->refs[0].p; a->scal[0].si = a->refs[0].si; a->scal[0].sj = a->refs[0].sj; a->scal[0].plane = a->refs[0].plane; }
+    // unused table entries repeat slot 0, so that a kernel may load through any of them without a clamp
+    for (int r = low.nrefs; r < FORTIS_MAX_REFS; r++) a->refs[r] = a->refs[0];
+    for (int r = low.nscal; r < ST_SCAL_MAX; r++) a->scal[r] = a->refs[0];
     a->count = (unsigned)low.count;
     a->ilo = low.ilo; a->jlo = low.jlo; a->ni = low.ni; a->sx = low.sx;
     a->cells = dcells;
