@@ -148,6 +148,9 @@ class Plan:
     def num_kernels(self):
         return self._L.fortis_plan_num_kernels(self._p)
 
+    def kernel_names(self):
+        return [self._L.fortis_plan_kernel_name(self._p, k).decode() for k in range(self.num_kernels)]
+
     def profile(self, enable=True):
         self._L.fortis_plan_profile(self._p, 1 if enable else 0)
 

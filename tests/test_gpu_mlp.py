@@ -150,3 +150,51 @@ def test_boundary_pre_post_bit_exact(L, gpu, dtype, NI, NK):
     assert np.array_equal(X.view(np.uint32), Xref.view(np.uint32))
     assert np.array_equal(Bm, O.boundary_post(Xref, scale, dtype))
     p.close()
+
+
+@pytest.mark.parametrize("B,N,K,act", [
+    (8300, 1100, 40, "leaky"),     # 585 tiles: whole rounds + a partial round of quarters; ragged B and N; K tail slab
+    (12000, 1100, 36, "relu"),     # 846 tiles: whole rounds + a round of halves + quarters
+    (16384, 512, 64, None),        # 512 tiles: whole rounds only, no activation
+    (257, 385, 4, "leaky"),        # one row / one column past a tile edge, a single 4-wide k slab
+])
+def test_gemm_schedule_phases(L, gpu, B, N, K, act):
+    """The persistent GEMM hands out whole 128 x 128 tiles round by round and cuts the remainder into
+    halves and quarters; every phase, ragged edges and the slab that runs past K against numpy float64
+    (fortis_gemm + epilogue: runtime/fortis_rt.c:45-75, compiler/FortisFuse.cpp:685-760)."""
+    rng = np.random.default_rng(7)
+    W = (rng.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    X = rng.standard_normal((B, K)).astype(np.float32)
+    p = P.Plan()
+    t0, t1 = p.tensor(B * K), p.tensor(B * N)
+    p.linear(t0, t1, W, b, B, act, 0.15)
+    plan = p.finalize(t0, t1)
+    assert plan.kernel_names() == ["gemm_bias_act"]
+    Y = plan.forward(X, (B, N))
+    ref = O.mlp_f64([W], [b], [act or "none"], X, alphas=[0.15])
+    assert maxrel(Y, ref) < TOL
+    plan.close()
+
+
+@pytest.mark.parametrize("rows,widths", [
+    (20000, [200, 256, 17]),       # 13 k groups in, 16 n-tiles: the wide register-resident variant, ragged tail tile
+    (16400, [61, 128, 128, 148]),  # SAM-shaped widths, input not a multiple of 4 (scalar loads), 148 outputs
+    (16385, [64, 64, 8]),          # 16-byte input loads and output stores, one row past a tile
+])
+def test_chain_wave_kernel_plain_shapes(L, gpu, rows, widths):
+    """Many rows take the wave-per-16-rows chain kernel; widths up to 256, vector and scalar row access."""
+    rng = np.random.default_rng(11)
+    n = len(widths) - 1
+    Ws = [(rng.standard_normal((widths[i + 1], widths[i])) / np.sqrt(widths[i])).astype(np.float32) for i in range(n)]
+    bs = [rng.standard_normal(widths[i + 1]).astype(np.float32) * 0.1 for i in range(n)]
+    acts = ["relu"] * (n - 1) + [None]
+    X = rng.standard_normal((rows, widths[0])).astype(np.float32)
+    plan = P.mlp_plan(Ws, bs, acts, rows)
+    assert plan.num_kernels == 1
+    Y = plan.forward(X, (rows, widths[-1]))
+    idx = np.r_[0:64, rows - 64:rows, np.random.default_rng(3).choice(rows, 256, replace=False)]
+    ref = O.mlp_f64(Ws, bs, ["relu"] * (n - 1) + ["none"], X[idx])
+    assert maxrel(Y[idx], ref) < TOL
+    assert np.isfinite(Y).all()
+    plan.close()
