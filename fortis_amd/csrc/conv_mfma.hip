@@ -22,23 +22,36 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 #define CM_THREADS 256
 #define CM_CC 4        // input channels per staged chunk (two MFMA channel pairs)
-#define CM_FT 64       // output channels per workgroup
 #define CM_NXMAX 16    // staged input elements per thread per chunk, at most
 
 struct ConvMShape {
     int C, D, H, W, F;         // F = output channels of the GEMM (4x the real ones in transposed mode)
     int P, plane, tiles, nchunks, R;
     int mode;                  // 0: convolution, 1: 2x2 stride-2 transposed conv scatter
+    int ksplit, chunks_per;    // channel chunks are split over blockIdx.z; > 1: raw partial sums go to `part`
+    float* part;               // [ksplit][output elements]
+    long osize;                // output elements
 };
 
-template <int KD, int KS, int MT>
+// FT output channels per workgroup: 64 (waves 2 x 2 over channels x positions) or 32 (4 waves over positions).
+// Workgroup barrier that orders LDS traffic only: global loads already issued stay in flight across it.
+__device__ __forceinline__ void cm_lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+template <int KD, int KS, int MT, int FT>
 __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
 {
     constexpr int T = KD * KS * KS;
-    constexpr int WCH = 2 * T * 2 * CM_FT;                       // floats of packed weights per chunk
+    constexpr int WCH = 2 * T * 2 * FT;                          // floats of packed weights per chunk
     constexpr int NW = (WCH / 4 + CM_THREADS - 1) / CM_THREADS;  // float4 per thread
-    constexpr int NMT = MT / 64;                                 // m-tiles per wave
+    constexpr int FW = FT / 32;                                  // waves along the channels
+    constexpr int NMT = MT / 32 / (4 / FW);                      // m-tiles per wave
+    static_assert(NMT >= 1, "tile too small for the wave layout");
     constexpr int PADK = KS / 2;
     extern __shared__ float4 smem4[];
     float* sW = (float*)smem4;                                    // [2][WCH]
@@ -81,7 +94,13 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         const float* xsrc = x + (long)ch * CM_CC * chan;
 #pragma unroll
         for (int i = 0; i < CM_NXMAX; i++)
-            rx[i] = (goff[i] >= 0 && ch * CM_CC + gch[i] < s.C) ? xsrc[goff[i]] : 0.f;
+        {
+            // always load from a valid address (the element itself, or element 0 of a valid channel) and
+            // select afterwards: no branch around the load
+            const bool ok = goff[i] >= 0 && ch * CM_CC + gch[i] < s.C;
+            const float v = xsrc[ok ? goff[i] : 0];
+            rx[i] = ok ? v : 0.f;
+        }
     };
     auto store_chunk = [&](int buf) {
         float4* wdst = (float4*)(sW + buf * WCH);
@@ -98,8 +117,8 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         }
     };
 
-    const int ft = wave & 1, mt0 = (wave >> 1) * NMT;
-    const int wbase = (lane >> 5) * CM_FT + ft * 32 + (lane & 31);
+    const int ft = wave % FW, mt0 = (wave / FW) * NMT;
+    const int wbase = (lane >> 5) * FT + ft * 32 + (lane & 31);
     const int xbase = (lane >> 5) * KD * s.R + mt0 * 32 + (lane & 31);
     v16f acc[NMT];
 #pragma unroll
@@ -107,12 +126,14 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
-    load_chunk(0);
+    const int ch0 = blockIdx.z * s.chunks_per;
+    const int ch1 = ch0 + s.chunks_per < s.nchunks ? ch0 + s.chunks_per : s.nchunks;
+    load_chunk(ch0);
     store_chunk(0);
-    __syncthreads();
-    for (int ch = 0; ch < s.nchunks; ch++) {
-        const int buf = ch & 1;
-        if (ch + 1 < s.nchunks) load_chunk(ch + 1);
+    cm_lds_barrier();
+    for (int ch = ch0; ch < ch1; ch++) {
+        const int buf = (ch - ch0) & 1;
+        if (ch + 1 < ch1) load_chunk(ch + 1);
         const float* w = sW + buf * WCH + wbase;
         const float* xs = sX + buf * XCH + xbase;
 #pragma unroll
@@ -124,14 +145,14 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
 #pragma unroll
                     for (int kw = 0; kw < KS; kw++) {
                         const int tap = (kd * KS + kh) * KS + kw;
-                        const float a = w[(cp * T + tap) * 2 * CM_FT];
+                        const float a = w[(cp * T + tap) * 2 * FT];
                         const int xoff = (2 * cp * KD + kd) * s.R + kh * s.P + kw;
 #pragma unroll
                         for (int j = 0; j < NMT; j++)
                             acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, xs[j * 32 + xoff], acc[j], 0, 0, 0);
                     }
-        if (ch + 1 < s.nchunks) store_chunk(buf ^ 1);
-        __syncthreads();
+        if (ch + 1 < ch1) store_chunk(buf ^ 1);
+        cm_lds_barrier();
     }
 
     // epilogue: a lane holds one position and 16 output channels per m-tile
@@ -144,7 +165,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         if (xx >= s.W) continue;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const int f = fg * CM_FT + ft * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int f = fg * FT + ft * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             if (f >= s.F) continue;
             int fo = f;
             long opos = ((long)z * s.H + yy) * s.W + xx;
@@ -153,6 +174,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
                 opos = (long)(2 * yy + ((f >> 1) & 1)) * (2 * s.W) + 2 * xx + (f & 1);
             }
             float v = acc[j][r];
+            if (s.ksplit > 1) { s.part[blockIdx.z * s.osize + fo * ospatial + opos] = v; continue; }
             if (e.scale) v = v * e.scale[fo];
             if (e.shift) v = v + e.shift[fo];
             if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
@@ -163,15 +185,46 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     }
 }
 
+// Sums the partial results of a channel-split launch in split order (deterministic) and applies the
+// epilogue.  ospatial = elements per output channel.
+__global__ void conv_split_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, long osize, long ospatial,
+                                         int ksplit, ConvEpi e)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= osize) return;
+    float v = part[idx];
+    for (int k = 1; k < ksplit; k++) v += part[k * osize + idx];
+    const long fo = idx / ospatial;
+    if (e.scale) v = v * e.scale[fo];
+    if (e.shift) v = v + e.shift[fo];
+    if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
+    else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
+    if (e.res) v = v + e.res[idx];
+    y[idx] = v;
+}
+
 // ---- host side ---------------------------------------------------------------------------------------
+static inline long conv_ft(long Fg) { return Fg <= 32 ? 32 : 64; }
+static int conv_cus()
+{
+    static int n = 0;
+    if (!n) {
+        hipDeviceProp_t prop;
+        n = hipGetDeviceProperties(&prop, 0) == hipSuccess ? prop.multiProcessorCount : 256;
+    }
+    return n;
+}
+
 // Packs conv weights W[F][C][T] (T taps, row-major) into the kernel's order
-//   [F/64][ceil(C/4)][channel pair 2][tap T][half 2][64 channels], zero padded.
+//   [F/FT][ceil(C/4)][channel pair 2][tap T][half 2][FT channels], zero padded; FT = 32 when the GEMM
+//   has at most 32 output channels, else 64 (the launcher applies the same rule).
 // Transposed 2x2 conv: W is [C][F][2][2]; GEMM channel f' = f*4 + a*2 + b.
 float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats)
 {
     const long Fg = transposed ? 4 * F : F;
-    const long nfg = cdiv(Fg, CM_FT), nch = cdiv(C, CM_CC);
-    const long wch = 2L * T * 2 * CM_FT;
+    const long FT = conv_ft(Fg);
+    const long nfg = cdiv(Fg, FT), nch = cdiv(C, CM_CC);
+    const long wch = 2L * T * 2 * FT;
     const long n = nfg * nch * wch;
     float* h = (float*)calloc(n, sizeof(float));
     for (long fgi = 0; fgi < nfg; fgi++)
@@ -179,11 +232,11 @@ float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transpos
             for (int cp = 0; cp < 2; cp++)
                 for (int t = 0; t < T; t++)
                     for (int hh = 0; hh < 2; hh++)
-                        for (int fl = 0; fl < CM_FT; fl++) {
-                            const long f = fgi * CM_FT + fl, c = ch * CM_CC + cp * 2 + hh;
+                        for (int fl = 0; fl < FT; fl++) {
+                            const long f = fgi * FT + fl, c = ch * CM_CC + cp * 2 + hh;
                             if (f >= Fg || c >= C) continue;
                             const float v = transposed ? W[(c * F + (f >> 2)) * 4 + (f & 3)] : W[(f * C + c) * T + t];
-                            h[((fgi * nch + ch) * 2 + cp) * T * 2 * CM_FT + ((long)t * 2 + hh) * CM_FT + fl] = v;
+                            h[((fgi * nch + ch) * 2 + cp) * T * 2 * FT + ((long)t * 2 + hh) * FT + fl] = v;
                         }
     float* d = nullptr;
     HIP_OK(hipMalloc((void**)&d, n * sizeof(float)));
@@ -193,27 +246,70 @@ float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transpos
     return d;
 }
 
-template <int KD, int KS, int MT>
+template <int KD, int KS, int MT, int FT>
 static int launch(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {
     constexpr int T = KD * KS * KS;
-    s.P = KS == 3 ? s.W + 1 : s.W;
-    s.plane = s.H * s.P;
     s.tiles = (int)cdiv(s.plane, MT);
-    s.nchunks = (int)cdiv(s.C, CM_CC);
     s.R = MT + (KS == 3 ? 2 * s.P + 2 : 0);
     if ((long)CM_CC * KD * s.R > (long)CM_THREADS * CM_NXMAX) return -1;     // run too long to stage
-    const size_t shmem = (size_t)2 * (2 * T * 2 * CM_FT + CM_CC * KD * s.R) * sizeof(float);
+    const size_t shmem = (size_t)2 * (2 * T * 2 * FT + CM_CC * KD * s.R) * sizeof(float);
     if (shmem > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
-        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         attr = shmem;
     }
-    dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, CM_FT));
-    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+    // A launch that leaves most CUs idle (deep, small images) is split over the input channels: each
+    // split writes raw partial sums, a second kernel adds them in order and applies the epilogue.
+    const long wgs = (long)s.D * s.tiles * cdiv(s.F, FT);
+    s.ksplit = 1;
+    s.chunks_per = s.nchunks;
+    if (wgs < conv_cus() && s.nchunks >= 8) {
+        long k = cdiv(2L * conv_cus(), wgs);
+        if (k > s.nchunks / 4) k = s.nchunks / 4;
+        if (k > 16) k = 16;
+        s.chunks_per = (int)cdiv(s.nchunks, k);
+        s.ksplit = (int)cdiv(s.nchunks, s.chunks_per);
+    }
+    const long ospatial = (long)s.D * s.H * s.W * (s.mode ? 4 : 1);
+    s.osize = (long)(s.mode ? s.F / 4 : s.F) * ospatial;
+    if (s.ksplit > 1) {
+        // scratch grows on the first (eager) run of a plan; replays and captured runs find it in place
+        static float* scratch = nullptr;
+        static size_t cap = 0;
+        const size_t need = (size_t)s.ksplit * s.osize * sizeof(float);
+        if (need > cap) {
+            // an outgrown buffer stays allocated: a graph captured earlier may still name it
+            HIP_OK(hipMalloc((void**)&scratch, need));
+            cap = need;
+        }
+        s.part = scratch;
+    }
+    dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);
+    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
     HIP_OK(hipGetLastError());
+    if (s.ksplit > 1) {
+        hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)cdiv(s.osize, 256)), dim3(256), 0, st, s.part, y, s.osize,
+                           ospatial, s.ksplit, e);
+        HIP_OK(hipGetLastError());
+    }
     return 0;
+}
+
+// Positions per workgroup: the largest tile that still gives every CU about two workgroups; small images
+// (deep UNet levels) take the smallest tile so that the launch spreads over the chip at all.
+template <int KD, int KS, int FT>
+static int launch_mt(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
+{
+    s.P = KS == 3 ? s.W + 1 : s.W;
+    s.plane = s.H * s.P;
+    s.nchunks = (int)cdiv(s.C, CM_CC);
+    const long want = 2L * conv_cus(), groups = (long)s.D * cdiv(s.F, FT);
+    constexpr int MTMIN = FT == 64 ? 64 : 128;
+    if (KD == 1 && groups * cdiv(s.plane, 256) >= want && launch<KD, KS, 256, FT>(x, wp, y, s, e, st) == 0) return 0;
+    if (2 * groups * cdiv(s.plane, 128) >= want || MTMIN == 128) return launch<KD, KS, 128, FT>(x, wp, y, s, e, st);
+    return launch<KD, KS, MTMIN, FT>(x, wp, y, s, e, st);
 }
 
 // kind: 0 conv (KD x KS x KS, pad KS/2), 1 transposed 2x2 stride 2.  Returns -1 if the shape is not
@@ -222,10 +318,14 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
                             int KS, int kind, const ConvEpi& e, hipStream_t st)
 {
     if (C * D * H * Wd >= 2147483647L || F * D * H * Wd * (kind ? 4 : 1) >= 2147483647L) return -1;
-    ConvMShape s = { (int)C, (int)D, (int)H, (int)Wd, (int)(kind ? 4 * F : F), 0, 0, 0, 0, 0, kind };
-    if (kind == 1) return D == 1 ? launch<1, 1, 256>(x, wp, y, s, e, st) : -1;
-    if (KD == 3 && KS == 3) return launch<3, 3, 128>(x, wp, y, s, e, st);
-    if (KD == 1 && KS == 3) return launch<1, 3, 256>(x, wp, y, s, e, st);
-    if (KD == 1 && KS == 1) return launch<1, 1, 256>(x, wp, y, s, e, st);
+    ConvMShape s = { (int)C, (int)D, (int)H, (int)Wd, (int)(kind ? 4 * F : F), 0, 0, 0, 0, 0, kind, 1, 0, nullptr, 0 };
+    const bool thin = conv_ft(s.F) == 32;
+    if (kind == 1) {
+        if (D != 1) return -1;
+        return thin ? launch_mt<1, 1, 32>(x, wp, y, s, e, st) : launch_mt<1, 1, 64>(x, wp, y, s, e, st);
+    }
+    if (KD == 3 && KS == 3) return thin ? launch_mt<3, 3, 32>(x, wp, y, s, e, st) : launch_mt<3, 3, 64>(x, wp, y, s, e, st);
+    if (KD == 1 && KS == 3) return thin ? launch_mt<1, 3, 32>(x, wp, y, s, e, st) : launch_mt<1, 3, 64>(x, wp, y, s, e, st);
+    if (KD == 1 && KS == 1) return thin ? launch_mt<1, 1, 32>(x, wp, y, s, e, st) : launch_mt<1, 1, 64>(x, wp, y, s, e, st);
     return -1;
 }
