@@ -67,6 +67,129 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_direct_kernel(const float* 
         if (f0 + f < s.F) y[(long)(f0 + f) * ospatial + opos] = conv_epilogue(acc[f], f0 + f, opos, ospatial, e);
 }
 
+// 3x3x3, stride 1, pad 1 convolution with at most CT_F output channels (image-space heads such as
+// 64 -> 3): the matrix cores would multiply 32-row tiles that are nine tenths padding, so this one runs on
+// the vector ALUs, which have the same fp32 peak on this part.
+// Positions of one z-plane are linearised with pitch P = W + 1 (tap (kh, kw) of position m is element
+// m + kh*P + kw of the zero-padded plane, a lane-independent offset).  A workgroup takes CT_MT positions,
+// a thread CT_PT consecutive ones times all output channels in registers; per chunk of CT_CC input
+// channels the three z-planes' runs are staged in LDS (double buffered through registers), and the
+// chunk's weights [channel][tap][output channel] next to them; a weight read has the same address in
+// every lane (LDS broadcast) and fetches one tap for all output channels.
+#define CT_F 4
+#define CT_PT 2
+#define CT_MT (CONV_THREADS * CT_PT)
+#define CT_CC 2
+#define CT_NX 16     // staged elements per thread per chunk, at most
+
+template <int NF>      // output channels computed: 3 (F <= 3) or 4
+__global__ __launch_bounds__(CONV_THREADS) void conv3d_thin_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                   float* __restrict__ y, int C, int D, int H, int W, int F,
+                                                                   int P, int plane, int tiles, int R, ConvEpi e)
+{
+    extern __shared__ float ct_lds[];                       // [2][CT_CC][3][R] inputs, then [2][CT_CC][27][CT_F] weights
+    const int tid = threadIdx.x;
+    const int z = blockIdx.x / tiles, tile = blockIdx.x - z * tiles;
+    const int m0 = tile * CT_MT;
+    const long HW = (long)H * W, chan = (long)D * HW;
+    const int XCH = CT_CC * 3 * R;
+
+    // staging map (the same for every chunk): offset of the element inside a CT_CC-channel group, or -1
+    int goff[CT_NX];
+#pragma unroll
+    for (int i = 0; i < CT_NX; i++) {
+        const int el = tid + i * CONV_THREADS;
+        goff[i] = -1;
+        if (el < XCH) {
+            const int c = el / (3 * R), rem = el - c * (3 * R), kd = rem / R, r = rem - kd * R;
+            const int v = m0 + r, yp = v / P, xp = v - yp * P;
+            const int zz = z + kd - 1, yy = yp - 1, xx = xp - 1;
+            if (zz >= 0 && zz < D && yy >= 0 && yy < H && xx >= 0 && xx < W)
+                goff[i] = (int)(c * chan + zz * HW + (long)yy * W + xx);
+        }
+    }
+    float rx[CT_NX];
+    float rwt = 0.f;
+    float* wl = ct_lds + 2 * XCH;
+    // weight element this thread stages: (cc, tap, f) -> w[f][c][tap]
+    const int wcc = tid / (27 * CT_F), wtap = (tid / CT_F) % 27, wf = tid % CT_F;
+    auto load_chunk = [&](int ch) __attribute__((always_inline)) {
+        if (tid < CT_CC * 27 * CT_F) {
+            const int c = ch * CT_CC + wcc;
+            rwt = (wf < F && c < C) ? w[((long)wf * C + c) * 27 + wtap] : 0.f;
+        }
+        const float* xsrc = x + (long)ch * CT_CC * chan;
+#pragma unroll
+        for (int i = 0; i < CT_NX; i++) {
+            const int el = tid + i * CONV_THREADS;
+            const bool ok = goff[i] >= 0 && ch * CT_CC + el / (3 * R) < C;
+            const float v = xsrc[ok ? goff[i] : 0];
+            rx[i] = ok ? v : 0.f;
+        }
+    };
+    auto store_chunk = [&](int buf) __attribute__((always_inline)) {
+        if (tid < CT_CC * 27 * CT_F) wl[buf * CT_CC * 27 * CT_F + tid] = rwt;
+        float* dst = ct_lds + buf * XCH;
+#pragma unroll
+        for (int i = 0; i < CT_NX; i++) {
+            const int el = tid + i * CONV_THREADS;
+            if (el < XCH) dst[el] = rx[i];
+        }
+    };
+
+    float acc[NF][CT_PT];
+#pragma unroll
+    for (int f = 0; f < NF; f++)
+#pragma unroll
+        for (int p = 0; p < CT_PT; p++) acc[f][p] = 0.f;
+
+    const int nchunks = (C + CT_CC - 1) / CT_CC;
+    load_chunk(0);
+    store_chunk(0);
+    __syncthreads();
+    for (int ch = 0; ch < nchunks; ch++) {
+        const int buf = ch & 1;
+        if (ch + 1 < nchunks) load_chunk(ch + 1);
+        const float* xs = ct_lds + buf * XCH + tid * CT_PT;
+#pragma unroll
+        for (int cc = 0; cc < CT_CC; cc++) {
+            const int c = ch * CT_CC + cc;
+            if (c >= C) break;
+#pragma unroll
+            for (int kd = 0; kd < 3; kd++)
+#pragma unroll
+                for (int kh = 0; kh < 3; kh++) {
+                    float in[CT_PT + 2];
+                    const float* row = xs + (cc * 3 + kd) * R + kh * P;
+#pragma unroll
+                    for (int t = 0; t < CT_PT + 2; t++) in[t] = row[t];
+                    // the three taps' weights for all output channels: same address in every lane (LDS broadcast)
+                    const float4* wt = (const float4*)(wl + ((buf * CT_CC + cc) * 27 + (kd * 3 + kh) * 3) * CT_F);
+                    const float4 w0 = wt[0], w1 = wt[1], w2 = wt[2];
+                    const float wa[3][CT_F] = { { w0.x, w0.y, w0.z, w0.w }, { w1.x, w1.y, w1.z, w1.w }, { w2.x, w2.y, w2.z, w2.w } };
+#pragma unroll
+                    for (int f = 0; f < NF; f++)
+#pragma unroll
+                        for (int p = 0; p < CT_PT; p++)
+                            acc[f][p] = fmaf(in[p + 2], wa[2][f], fmaf(in[p + 1], wa[1][f], fmaf(in[p], wa[0][f], acc[f][p])));
+                }
+        }
+        if (ch + 1 < nchunks) store_chunk(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int p = 0; p < CT_PT; p++) {
+        const int m = m0 + tid * CT_PT + p;
+        if (m >= plane) continue;
+        const int yy = m / P, xx = m - yy * P;
+        if (xx >= W) continue;
+        const long opos = ((long)z * H + yy) * W + xx;
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+            if (f < F) y[f * chan + opos] = conv_epilogue(acc[f][p], f, opos, chan, e);
+    }
+}
+
 // Transposed conv2d in gather form: y[f][oy][ox] = sum_c sum_{kh,kw : (oy+p-kh) % s == 0, ...}
 //     x[c][(oy+p-kh)/s][(ox+p-kw)/s] * w[c][f][kh][kw]
 __global__ __launch_bounds__(CONV_THREADS) void convt2d_kernel(const float* __restrict__ x, const float* __restrict__ w,
@@ -143,6 +266,26 @@ int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long 
 {
     if (!fits_int(C * D * H * Wd) || !fits_int(F * Do * Ho * Wo) || KD <= 0 || KH <= 0 || KW <= 0) return -1;
     if (Do != D + 2 * pd - KD + 1 || Ho != H + 2 * ph - KH + 1 || Wo != Wd + 2 * pw - KW + 1) return -1;
+    if (KD == 3 && KH == 3 && KW == 3 && pd == 1 && ph == 1 && pw == 1 && F <= CT_F) {
+        const int P = (int)Wd + 1, plane = (int)H * P, tiles = (int)cdiv(plane, CT_MT), R = CT_MT + 2 * P + 2;
+        const size_t shmem = (size_t)2 * (CT_CC * 3 * R + CT_CC * 27 * CT_F) * sizeof(float);
+        if ((long)CT_CC * 3 * R <= (long)CONV_THREADS * CT_NX && shmem <= 160 * 1024) {
+            static size_t attr = 0;
+            if (shmem > attr) {
+                HIP_OK(hipFuncSetAttribute((const void*)conv3d_thin_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+                HIP_OK(hipFuncSetAttribute((const void*)conv3d_thin_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+                attr = shmem;
+            }
+            if (F <= 3)
+                hipLaunchKernelGGL(conv3d_thin_kernel<3>, dim3((unsigned)(D * tiles)), dim3(CONV_THREADS), shmem, s, x, w, y, (int)C,
+                                   (int)D, (int)H, (int)Wd, (int)F, P, plane, tiles, R, e);
+            else
+                hipLaunchKernelGGL(conv3d_thin_kernel<4>, dim3((unsigned)(D * tiles)), dim3(CONV_THREADS), shmem, s, x, w, y, (int)C,
+                                   (int)D, (int)H, (int)Wd, (int)F, P, plane, tiles, R, e);
+            HIP_OK(hipGetLastError());
+            return 0;
+        }
+    }
     ConvShape sh = { (int)C, (int)D, (int)H, (int)Wd, (int)F, (int)KD, (int)KH, (int)KW, (int)Do, (int)Ho, (int)Wo, 1, 1, 1,
                      (int)pd, (int)ph, (int)pw };
     hipLaunchKernelGGL(conv_direct_kernel, dim3((unsigned)cdiv(Do * Ho * Wo, CONV_THREADS), (unsigned)cdiv(F, CONV_FB)),

@@ -30,6 +30,7 @@ struct ConvMShape {
     int mode;                  // 0: convolution, 1: 2x2 stride-2 transposed conv scatter
     int ksplit, chunks_per;    // channel chunks are split over blockIdx.z; > 1: raw partial sums go to `part`
     float* part;               // [ksplit][output elements]
+    int ups;                   // 1: the input tensor is (D/2, H/2, W/2) and is read through a nearest x2 upsample
     long osize;                // output elements
 };
 
@@ -63,6 +64,9 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     const int fg = blockIdx.y;
     const int m0 = tile * MT;
     const long HW = (long)s.H * s.W, chan = (long)s.D * HW;
+    // source geometry: the tensor itself, or the half-resolution tensor a fused nearest upsample reads
+    const int sh = s.ups ? 1 : 0;
+    const long srcW = s.W >> sh, sHW = (long)(s.H >> sh) * srcW, schan = (long)(s.D >> sh) * sHW;
 
     // per-thread staging map of the input run (same for every chunk): global offset inside a 4-channel group
     int goff[CM_NXMAX];
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
             const int zz = z + kd - (KD / 2), yy = yp - PADK, xx = xp - PADK;
             gch[i] = c;
             if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W)
-                goff[i] = (int)(c * chan + zz * HW + (long)yy * s.W + xx);
+                goff[i] = (int)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh));
         }
     }
 
@@ -91,7 +95,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
             const int f4 = tid + i * CM_THREADS;
             if (f4 < WCH / 4) rw[i] = wsrc[f4];
         }
-        const float* xsrc = x + (long)ch * CM_CC * chan;
+        const float* xsrc = x + (long)ch * CM_CC * schan;
 #pragma unroll
         for (int i = 0; i < CM_NXMAX; i++)
         {
@@ -312,13 +316,16 @@ static int launch_mt(const float* x, const float* wp, float* y, ConvMShape s, co
     return launch<KD, KS, MTMIN, FT>(x, wp, y, s, e, st);
 }
 
-// kind: 0 conv (KD x KS x KS, pad KS/2), 1 transposed 2x2 stride 2.  Returns -1 if the shape is not
+// kind: 0 conv (KD x KS x KS, pad KS/2), 1 transposed 2x2 stride 2, 2 conv whose input (given at half
+// resolution) is read through a nearest x2 upsample; D, H, Wd are always the conv's own input extents.  Returns -1 if the shape is not
 // one the MFMA kernel takes (the caller then uses the direct kernel).
 int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, long D, long H, long Wd, long F, int KD,
                             int KS, int kind, const ConvEpi& e, hipStream_t st)
 {
-    if (C * D * H * Wd >= 2147483647L || F * D * H * Wd * (kind ? 4 : 1) >= 2147483647L) return -1;
-    ConvMShape s = { (int)C, (int)D, (int)H, (int)Wd, (int)(kind ? 4 * F : F), 0, 0, 0, 0, 0, kind, 1, 0, nullptr, 0 };
+    if (C * D * H * Wd >= 2147483647L || F * D * H * Wd * (kind == 1 ? 4 : 1) >= 2147483647L) return -1;
+    ConvMShape s = { (int)C, (int)D, (int)H, (int)Wd, (int)(kind == 1 ? 4 * F : F), 0, 0, 0, 0, 0, kind == 1 ? 1 : 0, 1, 0, nullptr, 0, 0 };
+    s.ups = kind == 2 ? 1 : 0;
+    if (kind == 2 && ((D | H | Wd) & 1)) return -1;
     const bool thin = conv_ft(s.F) == 32;
     if (kind == 1) {
         if (D != 1) return -1;

@@ -52,6 +52,7 @@ struct fortis_plan {
     bool finalized = false;
     int in_t = -1, out_t = -1;
     long rows0 = 0;             // rows at finalize (row-wise plans), for run-time extents
+    int exec_skip = 0;          // ops folded into a neighbour at finalize
     bool prof = false;          // per-kernel event timing (fortis_plan_profile)
     std::vector<hipEvent_t> ev; // events of the recorded passes: (nexec + 1) per pass
     size_t ev_used = 0;
@@ -335,6 +336,7 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
         p->tptr.push_back(d);
     }
     const std::vector<Op>& ops = p->ops;
+    int fuse_ups_src = -1;      // source tensor of an upsample folded into the convolution that follows
     for (size_t i = 0; i < ops.size();) {
         Exec ex;
         size_t took = try_chain(p, i, &ex);
@@ -381,6 +383,8 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
             case OP_CONVT2D:
             case OP_CONV3D: {
                 ex.kind = o.kind == OP_CONV2D ? EX_CONV2D : o.kind == OP_CONVT2D ? EX_CONVT2D : EX_CONV3D;
+                if (o.kind == OP_CONV3D && fuse_ups_src >= 0) { ex.src = fuse_ups_src; ex.flag = 1; }
+                fuse_ups_src = -1;
                 ex.W = (const float*)upload(p, o.w.data(), o.w.size() * 4);
                 // y = act(scale * conv + shift): bias and BatchNorm-eval folded into two vectors.
                 // scale = gamma / sqrt(var + eps); shift = beta + (bias - mean) * scale.
@@ -413,7 +417,22 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                 break;
             }
             case OP_MAXPOOL: ex.kind = EX_MAXPOOL; break;
-            case OP_UPSAMPLE: ex.kind = EX_UPSAMPLE; break;
+            case OP_UPSAMPLE: {
+                ex.kind = EX_UPSAMPLE;
+                // A 3-D nearest x2 upsample whose only reader is the next 3x3x3 convolution is not run:
+                // the convolution reads the half-resolution tensor through the upsample's index map.
+                static int direct_only = -1;
+                if (direct_only < 0) direct_only = getenv("FORTIS_CONV_DIRECT") != 0;
+                if (!direct_only && o.nd == 3 && o.sfac == 2 && i + 1 < ops.size() && ops[i + 1].kind == OP_CONV3D &&
+                    ops[i + 1].src == o.dst && ops[i + 1].KD == 3 && ops[i + 1].pad == 1 && ops[i + 1].F >= 16 && out_t != o.dst) {
+                    bool other = false;
+                    for (size_t j = 0; j < ops.size(); j++)
+                        if (j != i + 1 && (ops[j].src == o.dst || ops[j].res == o.dst)) other = true;
+                    if (ops[i + 1].res == o.dst) other = true;
+                    if (!other) { fuse_ups_src = o.src; p->exec_skip++; i += 1; continue; }
+                }
+                break;
+            }
             case OP_CONCAT: ex.kind = EX_CONCAT; break;
             case OP_PERMUTE: ex.kind = EX_PERMUTE; break;
         }
@@ -474,7 +493,8 @@ void fortis_plan_run(fortis_plan* p)
                 ConvEpi epi = e.epi;
                 epi.res = e.res >= 0 ? (const float*)p->tptr[e.res] : nullptr;
                 const long Do = o->D + 2 * o->pad - o->KD + 1, Ho = o->H + 2 * o->pad - o->KH + 1, Wo = o->W + 2 * o->pad - o->KW + 1;
-                rc = e.Wmfma ? fortis_launch_conv_mfma(src, e.Wmfma, dst, o->C, o->D, o->H, o->W, o->F, 3, 3, 0, epi, s) : -1;
+                rc = e.Wmfma ? fortis_launch_conv_mfma(src, e.Wmfma, dst, o->C, o->D, o->H, o->W, o->F, 3, 3, e.flag ? 2 : 0, epi, s) : -1;
+                if (rc != 0 && e.flag) { fprintf(stderr, "fortis_plan_run: fused upsample + conv3d shape not taken by the kernel\n"); break; }
                 if (rc != 0)
                     rc = fortis_launch_conv3d(src, e.W, dst, o->C, o->D, o->H, o->W, o->F, o->KD, o->KH, o->KW, Do, Ho, Wo, o->pad,
                                               o->pad, o->pad, epi, s);
