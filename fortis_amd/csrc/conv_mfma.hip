@@ -269,7 +269,7 @@ static int launch(const float* x, const float* wp, float* y, ConvMShape s, const
     const long wgs = (long)s.D * s.tiles * cdiv(s.F, FT);
     s.ksplit = 1;
     s.chunks_per = s.nchunks;
-    if (wgs < conv_cus() && s.nchunks >= 8) {
+    if (2 * wgs < 3 * conv_cus() && s.nchunks >= 8) {
         long k = cdiv(2L * conv_cus(), wgs);
         if (k > s.nchunks / 4) k = s.nchunks / 4;
         if (k > 16) k = 16;
