@@ -19,6 +19,7 @@
 #include "common.h"
 
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float cm_v4f __attribute__((ext_vector_type(4)));   // native vector: conditional copies stay in registers
 
 #define CM_THREADS 256
 #define CM_CC 4        // input channels per staged chunk (two MFMA channel pairs)
@@ -86,14 +87,14 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         }
     }
 
-    float4 rw[NW];
+    cm_v4f rw[NW];
     float rx[CM_NXMAX];
     auto load_chunk = [&](int ch) {
-        const float4* wsrc = (const float4*)(wp + ((long)fg * s.nchunks + ch) * WCH);
+        const cm_v4f* wsrc = (const cm_v4f*)(wp + ((long)fg * s.nchunks + ch) * WCH);
 #pragma unroll
         for (int i = 0; i < NW; i++) {
             const int f4 = tid + i * CM_THREADS;
-            if (f4 < WCH / 4) rw[i] = wsrc[f4];
+            rw[i] = wsrc[f4 < WCH / 4 ? f4 : 0];
         }
         const float* xsrc = x + (long)ch * CM_CC * schan;
 #pragma unroll
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         }
     };
     auto store_chunk = [&](int buf) {
-        float4* wdst = (float4*)(sW + buf * WCH);
+        cm_v4f* wdst = (cm_v4f*)(sW + buf * WCH);
 #pragma unroll
         for (int i = 0; i < NW; i++) {
             const int f4 = tid + i * CM_THREADS;
