@@ -332,6 +332,34 @@ __global__ void gemm_naive_kernel(const float* __restrict__ A, const float* __re
     C[idx] = v;
 }
 
+// Work list for C[B][N] on `slots` resident workgroups (a multiple of 8): whole rounds of 128 x 128 tiles,
+// then one round of halves if at least half a round is left, one round of quarters if at least a quarter
+// round is left, and the rest as quarters.
+static void gemm_make_sched(long B, long N, long slots, GemmSched* out)
+{
+    GemmSched sc = {};
+    sc.tiles_n = (int)cdiv(N, 128);
+    sc.slots = slots;
+    const long total = cdiv(B, 128) * sc.tiles_n;
+    long base = total / slots * slots, rem = total - base;
+    auto phase = [&](int level, long b, long count) { GemmPhase ph = { level, 0, b, count }; sc.ph[sc.nphase++] = ph; };
+    if (base) phase(0, 0, base);
+    if (2 * rem >= slots) { phase(1, base, slots); base += slots / 2; rem -= slots / 2; }
+    if (4 * rem >= slots) { phase(2, base, slots); base += slots / 4; rem -= slots / 4; }
+    if (rem) phase(2, base, 4 * rem);
+    *out = sc;
+}
+
+// Test hook: the schedule as (level, first tile, items) triples; returns the number of phases.
+extern "C" int fortis_gemm_schedule(long B, long N, long slots, long* triples)
+{
+    if (B <= 0 || N <= 0 || slots < 8 || slots % 8) return -1;
+    GemmSched sc;
+    gemm_make_sched(B, N, slots, &sc);
+    for (int p = 0; p < sc.nphase; p++) { triples[3 * p] = sc.ph[p].level; triples[3 * p + 1] = sc.ph[p].base; triples[3 * p + 2] = sc.ph[p].count; }
+    return sc.nphase;
+}
+
 // slots = workgroups resident at once (occupancy x CUs), a multiple of 8
 template <int BK>
 static void launch_tiled(const float* A, const float* W, float* C, long B, long N, long K, const GemmEpi& epi, hipStream_t s)
@@ -349,16 +377,8 @@ static void launch_tiled(const float* A, const float* W, float* C, long B, long 
         slots = (long)occ * prop.multiProcessorCount / 8 * 8;
         if (slots < 8) slots = 8;
     }
-    GemmSched sc = {};
-    sc.tiles_n = (int)cdiv(N, 128);
-    sc.slots = slots;
-    const long total = cdiv(B, 128) * sc.tiles_n;
-    long base = total / slots * slots, rem = total - base;
-    auto phase = [&](int level, long b, long count) { GemmPhase ph = { level, 0, b, count }; sc.ph[sc.nphase++] = ph; };
-    if (base) phase(0, 0, base);
-    if (2 * rem >= slots) { phase(1, base, slots); base += slots / 2; rem -= slots / 2; }
-    if (4 * rem >= slots) { phase(2, base, slots); base += slots / 4; rem -= slots / 4; }
-    if (rem) phase(2, base, 4 * rem);
+    GemmSched sc;
+    gemm_make_sched(B, N, slots, &sc);
     long items = 0;
     for (int p = 0; p < sc.nphase; p++) items = sc.ph[p].count > items ? sc.ph[p].count : items;
     const long grid = items < slots ? cdiv(items, 8) * 8 : slots;

@@ -383,3 +383,14 @@ float fortis_stencil_step_fused_time_ms(const fortis_stencil_t* g, const fortis_
     return fortis_time_ms(fused_cb, &a, iters);
 }
 }  // extern "C"
+
+// Test hook: quotient and remainder of n / d through the multiply-shift the kernels use (host evaluation of
+// the same arithmetic as st_divmod).
+extern "C" void fortis_magic_divmod(unsigned n, unsigned d, unsigned* q, unsigned* r)
+{
+    const StMagic m = st_magic(d);
+    if (m.one) { *q = n; *r = 0; return; }
+    const unsigned long long t = (unsigned long long)n * m.mh + (unsigned)(((unsigned long long)n * m.ml) >> 32);
+    *q = (unsigned)(t >> 32);
+    *r = n - *q * m.d;
+}

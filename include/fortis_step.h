@@ -226,6 +226,15 @@ void  fortis_plan_profile(fortis_plan* p, int enable);
 int   fortis_plan_profile_read(fortis_plan* p, float* ms_per_kernel);
 const char* fortis_plan_kernel_name(fortis_plan* p, int idx);
 
+/* ================================ test hooks ============================================ */
+/* No reference counterpart; host-only, usable without a GPU.
+ * fortis_gemm_schedule: the persistent GEMM's work list for C[B][N] on `slots` resident workgroups, as
+ *   (level, first 128 x 128 tile, items) triples, level 0 whole tiles, 1 halves (128 x 64), 2 quarters
+ *   (64 x 64); returns the number of phases (at most 4), -1 on bad arguments.
+ * fortis_magic_divmod: n / d and n % d by the exact multiply-shift the stencil kernels decode cells with. */
+int  fortis_gemm_schedule(long B, long N, long slots, long* triples);
+void fortis_magic_divmod(unsigned n, unsigned d, unsigned* q, unsigned* r);
+
 #ifdef __cplusplus
 }
 #endif

@@ -164,3 +164,57 @@ def test_lowering_accepts_chains_and_rejects_the_rest(L, capfd):
     for ins in bad:
         assert L.fortis_stencil_check(C.byref(_table_with(ins))) == -1
     capfd.readouterr()
+
+
+# ---- persistent GEMM work list --------------------------------------------------------------------
+@pytest.mark.parametrize("B,N,slots", [(24576, 768, 512), (24576, 368, 512), (24576, 768, 768), (8300, 1100, 512),
+                                       (12000, 1100, 512), (1, 1, 512), (128, 128, 8), (100000, 4000, 512), (257, 385, 512)])
+def test_gemm_schedule_covers_every_tile_once(L, B, N, slots):
+    """Whole rounds of 128 x 128 tiles, then halves, then quarters: every 64 x 64 quarter of every tile
+    is produced exactly once, no phase but the first exceeds one round, and full tiles come in whole rounds."""
+    tri = (C.c_long * 12)()
+    n = L.fortis_gemm_schedule(B, N, slots, tri)
+    assert 1 <= n <= 4
+    tiles = -(-B // 128) * -(-N // 128)
+    cover = np.zeros((tiles, 4), np.int32)
+    for p in range(n):
+        level, base, count = tri[3 * p], tri[3 * p + 1], tri[3 * p + 2]
+        if level == 0:
+            assert p == 0 and base == 0 and count % slots == 0
+            cover[:count] += 1
+        elif level == 1:
+            assert count <= slots and count % 2 == 0
+            cover[base:base + count // 2] += 1
+        else:
+            assert level == 2 and count <= slots and count % 4 == 0
+            cover[base:base + count // 4] += 1
+    assert (cover == 1).all()
+    # balance: the items of the tail phases are at most one round each, so no workgroup gets more than
+    # (whole rounds) + 1/2 + 1/4 + 1/4 of a tile beyond the ideal share
+    work = sum({0: 1.0, 1: 0.5, 2: 0.25}[tri[3 * p]] * -(-tri[3 * p + 2] // slots) for p in range(n))
+    assert work <= tiles / slots + 1.0
+
+
+def test_gemm_schedule_rejects_bad_arguments(L):
+    tri = (C.c_long * 12)()
+    assert L.fortis_gemm_schedule(0, 5, 512, tri) == -1
+    assert L.fortis_gemm_schedule(5, 5, 7, tri) == -1
+
+
+# ---- exact division by a launch constant (cell decode of the stencil kernels) ---------------------------
+def test_magic_divmod_is_exact():
+    """q = (n * ceil(2^64 / d)) >> 64 must equal n // d for every 32-bit n: checked on the edges of the
+    range, around multiples of d, and on random pairs, against Python integers."""
+    import fortis_amd
+    L = fortis_amd.load()
+    rng = np.random.default_rng(0)
+    ds = [1, 2, 3, 5, 7, 64, 65, 4736, 2376, 1048576, 65535, 65537, 2**31 - 1, 2**31, 2**31 + 1, 2**32 - 1] + \
+        [int(v) for v in rng.integers(1, 2**32, 40)]
+    q, r = C.c_uint(), C.c_uint()
+    for d in ds:
+        ns = {0, 1, d - 1, d, d + 1, 2**32 - 1, 2**32 - 2, 2**31, (2**32 - 1) // d * d, max((2**32 - 1) // d * d - 1, 0)}
+        ns |= {int(v) for v in rng.integers(0, 2**32, 200)}
+        ns |= {min(int(k) * d + off, 2**32 - 1) for k in rng.integers(0, max(2**32 // d, 1), 50) for off in (-1, 0, 1) if int(k) * d + off >= 0}
+        for n_ in (v for v in ns if 0 <= v < 2**32):
+            L.fortis_magic_divmod(n_, d, C.byref(q), C.byref(r))
+            assert (q.value, r.value) == (n_ // d, n_ % d), (n_, d)
