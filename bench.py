@@ -26,7 +26,8 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # same command (see profiles/), or None where no counter run has been made for the workload.
-MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": None, "zb_ref": None, "toy": None}
+MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((2482.4 * 2 + 936.6) * 1024),
+                    "zb_ref": int((2396.6 * 2 + 936.6) * 1024), "zb_1028x1028x15": int((331322.2 * 2 + 207387.3) * 1024), "toy": None}
 
 
 def omp_threads():
@@ -273,7 +274,7 @@ def run_zb(L, args, reference_net=False):
                 unit="TFLOP/s" if bound == "mfma" else "GB/s",
                 frac=round((tf / PEAK_F32_MFMA_TFLOPS) if bound == "mfma" else (gbs / PEAK_HBM_GBS), 5),
                 avg_launch_ms=round(avg, 5), flop_per_launch=flops, bytes_per_launch=nbytes,
-                hbm_GBs=round(gbs, 2), mfma_TFLOPs=round(tf, 3), traffic=MEASURED_TRAFFIC["zb_ref" if reference_net else "zb"])
+                hbm_GBs=round(gbs, 2), mfma_TFLOPs=round(tf, 3), traffic=MEASURED_TRAFFIC.get(("zb_ref" if reference_net else "zb") + ("_%dx%dx%d" % (sx, sy, nz) if args.grid else "")))
     # dt covers the validating launch too; whole-job throughput uses the clocked launches only
     out = dict(rows=rows, dt=ms * 1e-3, wall_dt=dt, dtype="f32",
                config={"workload": "zb_gather_mlp_scatter_%s_%dx%dx%d" % ("27_20_3" if reference_net else "27_64_64_3", sx, sy, nz),
