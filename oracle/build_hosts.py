@@ -1,0 +1,66 @@
+"""Builds the reference's own Fortran host programs, from their sources where they lie under
+/root/reference, against this library: the drop-in check of the entry tier.  Outputs go to oracle/_ref/
+only (git-ignored).  Test infrastructure: run by tests/test_gpu_hosts.py, built by __graft_entry__.build().
+
+  toy_dev_hip     benchmarks/toy/bench_dev.f90  (mlp_upload / mlp_forward_dev x1000 / mlp_download; the
+                  model is frontend/export_mlp.py's: seed 42, Linear(1024,256) ReLU Linear(256,1024))
+  zb_expert_hip   mom6_zb/zb_host_expert.f90    (per-layer hand-batched mlp_forward(xb(27,4736), yb(3,4736));
+                  the model is mom6_zb/zb_nn.npz with its input and output norms)
+
+Each links: host.o + step file emitted by fortis_amd/emit.py + libfortis_rt.so."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+REF = os.environ.get("FORTIS_REFERENCE", "/root/reference")
+FLANG = os.environ.get("FLANG", "/opt/rocm/lib/llvm/bin/flang")
+OUT = os.path.join(HERE, "_ref")
+
+
+def run(cmd):
+    r = subprocess.run(cmd, cwd=OUT, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("build_hosts: %s\n%s\n%s" % (" ".join(cmd), r.stdout, r.stderr))
+
+
+def link(host_f90, step_c, exe):
+    obj = os.path.join(OUT, exe + "_host.o")
+    run([FLANG, "-O2", "-c", host_f90, "-o", obj])
+    sobj = os.path.join(OUT, exe + "_step.o")
+    run(["gcc", "-O2", "-c", "-I", os.path.join(ROOT, "include"), step_c, "-o", sobj])
+    run([FLANG, obj, sobj, "-L", os.path.join(ROOT, "fortis_amd"), "-lfortis_rt", "-Wl,-rpath,$ORIGIN/../../fortis_amd",
+         "-o", os.path.join(OUT, exe)])
+    for f in (obj, sobj, step_c[:-2] + ".bin"):      # the weights are inside the object now
+        os.remove(f)
+
+
+def main():
+    if not os.path.isdir(os.path.join(REF, "mom6_zb")) or not os.access(FLANG, os.X_OK):
+        print("build_hosts: reference sources or flang not present, skipping")
+        return 0
+    sys.path.insert(0, ROOT)
+    from fortis_amd import emit
+    os.makedirs(OUT, exist_ok=True)
+    # toy: the exporter's model, reproduced from its seed (frontend/export_mlp.py:3-15)
+    import torch
+    torch.manual_seed(42)
+    net = torch.nn.Sequential(torch.nn.Linear(1024, 256), torch.nn.ReLU(), torch.nn.Linear(256, 1024)).eval()
+    Ws = [net[0].weight.detach().numpy(), net[2].weight.detach().numpy()]
+    bs = [net[0].bias.detach().numpy(), net[2].bias.detach().numpy()]
+    c, _ = emit.emit_mlp_step(os.path.join(OUT, "toy_dev_step"), Ws, bs, ["relu", None], rows=1, graph=True)
+    link(os.path.join(REF, "benchmarks/toy/bench_dev.f90"), c, "toy_dev_hip")
+    # ZB expert host: one call per layer on 4736 cells
+    W = np.load(os.path.join(ROOT, "tests", "golden", "zb_nn.npz"))
+    c, _ = emit.emit_mlp_step(os.path.join(OUT, "zb_expert_step"), [W["A0"], W["A1"]], [W["b0"], W["b1"]], ["relu", None],
+                              rows=4736, in_norms=W["in_norms"], out_norms=W["out_norms"])
+    link(os.path.join(REF, "mom6_zb/zb_host_expert.f90"), c, "zb_expert_hip")
+    print("build_hosts: built toy_dev_hip, zb_expert_hip in", OUT)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,52 @@
+"""The reference's own Fortran host programs, compiled from its sources and linked against this library
+(oracle/build_hosts.py): they call the entry points by bind(c) name exactly as they do in a FORTIS
+build, and their printed checksums and written fields are compared with the reference-held numbers."""
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+REFBIN = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref")
+
+
+def run_host(name, cwd, env=None):
+    exe = os.path.join(REFBIN, name)
+    if not os.path.exists(exe):
+        pytest.skip(f"{exe} not built (needs the reference sources and flang at build time)")
+    e = dict(os.environ)
+    e.update(env or {})
+    r = subprocess.run([exe], cwd=cwd, capture_output=True, text=True, timeout=120, env=e)
+    assert r.returncode == 0, r.stdout + r.stderr
+    return r.stdout
+
+
+def test_toy_host_upload_forward_dev_download(gpu, tmp_path):
+    """benchmarks/toy/bench_dev.f90: upload once, 1000 x mlp_forward_dev (captured as a graph on the
+    second call and replayed), download; README.md:25 stamps the checksum 7.775037."""
+    out = run_host("toy_dev_hip", tmp_path)
+    chk = float(re.search(r"checksum:\s*([-0-9.Ee+]+)", out).group(1))
+    assert abs(chk - 7.775037) / 7.775037 < 1e-5, out
+    per_call = float(re.search(r"per-call us:\s*([-0-9.Ee+]+)", out).group(1))
+    print("toy host per-call us:", per_call)
+    assert 0 < per_call < 1000
+
+
+def test_zb_expert_host_matches_native_golden(gpu, tmp_path, golden):
+    """mom6_zb/zb_host_expert.f90: the host packs 4736 stencils per layer itself and calls
+    mlp_forward(xb, yb) 15 x 11 times; its Txx/Tyy/Txy must agree with the reference's native CPU build
+    (golden checksums and layers 1, 8, 15) within the reference's own difftest tolerance of 5e-6 of the
+    field maximum (mom6_zb/README.md:16)."""
+    out = run_host("zb_expert_hip", tmp_path)
+    m = re.search(r"checksum Txx:\s*([-0-9.Ee+]+)\s+Tyy:\s*([-0-9.Ee+]+)\s+Txy:\s*([-0-9.Ee+]+)", out)
+    chk = np.array([float(m.group(i)) for i in (1, 2, 3)])
+    G = np.load(os.path.join(golden, "zb_native_golden.npz"))
+    assert np.all(np.abs(chk - G["checksum"]) < 1e-5 * np.abs(G["checksum"])), (chk, G["checksum"])
+    raw = np.fromfile(os.path.join(tmp_path, "zb_out.bin"), dtype=np.float64).reshape(3, 15, 78, 68)
+    for f, name in enumerate(("Txx", "Tyy", "Txy")):
+        for n, layer in enumerate(G["layers"]):
+            ref = G[name][n].astype(np.float64)
+            got = raw[f, layer - 1]
+            assert np.abs(got - ref).max() <= 5e-6 * np.abs(ref).max(), (name, layer)
