@@ -54,6 +54,26 @@ def cpu_baseline_mlp(case, sample_rows, X, min_seconds=8.0, **kw):
                        f"(native Fortran loop order, fp32, OpenMP over columns), {dt:.1f} s")
 
 
+def timed_steps(L, plan, steps):
+    """Two passes of `steps` steps each: the first, with nothing but the step's own launches on the stream,
+    is the clocked one (-> value, ms_per_step); the second records a HIP event on the library's stream
+    before and after every kernel (-> per-kernel durations for the roofline figure).  Events between
+    kernels cost a few microseconds of idle stream each, which is why the clocked pass carries none."""
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        plan.run()
+    L.fortis_sync()
+    dt = time.perf_counter() - t0
+    plan.profile(True)
+    for _ in range(steps):
+        plan.run()
+    L.fortis_sync()
+    passes, per = plan.profile_read()
+    plan.profile(False)
+    assert passes == steps
+    return dt, passes, per
+
+
 def run_climsim(L, args):
     from fortis_amd import configs
     case = configs.climsim()
@@ -62,15 +82,7 @@ def run_climsim(L, args):
     for _ in range(args.warmup):
         plan.run()
     L.fortis_sync()
-    plan.profile(True)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        plan.run()
-    L.fortis_sync()
-    dt = time.perf_counter() - t0
-    passes, per = plan.profile_read()
-    plan.profile(False)
-    assert passes == args.steps
+    dt, passes, per = timed_steps(L, plan, args.steps)
     gemm_ms = sum(ms for name, ms in per if name == "gemm_bias_act")
     ngemm = sum(1 for name, _ in per if name == "gemm_bias_act")
     avg_launch_ms = gemm_ms / (ngemm * passes)
@@ -134,14 +146,7 @@ def run_conv(L, args, which):
     for _ in range(args.warmup):
         plan.run()
     L.fortis_sync()
-    plan.profile(True)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        plan.run()
-    L.fortis_sync()
-    dt = time.perf_counter() - t0
-    passes, per = plan.profile_read()
-    plan.profile(False)
+    dt, passes, per = timed_steps(L, plan, args.steps)
     kern, count = {}, {}
     for n, ms in per:
         kern[n] = kern.get(n, 0.0) + ms / passes

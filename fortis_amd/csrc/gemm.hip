@@ -316,6 +316,47 @@ __global__ __launch_bounds__(GM_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
     }
 }
 
+// Small batches (B <= 16; the reference's generated warp-per-output kernel for batch < 32,
+// compiler/FortisFuse.cpp:667-719): one wave per output column n.  The lanes stride over k with 16-byte
+// loads of W[n][:] (1 KiB per wave per step, fully coalesced) and of the few A rows (the same for every
+// wave: served by the caches), then the 64 partial sums are folded with a shuffle tree.  Memory-bound on
+// reading W once; a 128 x 128 MFMA tile would be 1 % useful.
+template <int BR>
+__global__ __launch_bounds__(256) void gemm_small_kernel(const float* __restrict__ A, const float* __restrict__ W,
+                                                         float* __restrict__ C, int B, long N, long K, GemmEpi epi)
+{
+    const int lane = threadIdx.x & 63;
+    const long n = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    float acc[BR];
+#pragma unroll
+    for (int r = 0; r < BR; r++) acc[r] = 0.f;
+    const float* wrow = W + n * K;
+    for (long k0 = lane * 4; k0 < K; k0 += 256) {
+        const v4f w = *(const v4f*)(wrow + k0);
+#pragma unroll
+        for (int r = 0; r < BR; r++) {
+            const v4f a = *(const v4f*)(A + (long)(r < B ? r : 0) * K + k0);
+            acc[r] = fmaf(w.w, a.w, fmaf(w.z, a.z, fmaf(w.y, a.y, fmaf(w.x, a.x, acc[r]))));
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < BR; r++)
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) acc[r] += __shfl_xor(acc[r], off, 64);
+    if (lane == 0) {
+        const float bv = epi.bias ? epi.bias[n] : 0.f;
+#pragma unroll
+        for (int r = 0; r < BR; r++) {
+            if (r >= B) break;
+            float v = gemm_act(acc[r] + bv, epi.act, epi.alpha);
+            if (epi.out_scale) v = v * epi.out_scale[n];
+            if (n >= epi.mask_from) v = v > 0.f ? v : 0.f;
+            C[(long)r * N + n] = v;
+        }
+    }
+}
+
 // Generic guarded fallback for K not a multiple of 4 (16-byte row loads impossible): one thread
 // per output element, fp32 FMA chain.  Correct for any shape; not a fast path.
 __global__ void gemm_naive_kernel(const float* __restrict__ A, const float* __restrict__ W, float* __restrict__ C,
@@ -394,6 +435,14 @@ int fortis_launch_gemm(const float* A, const float* W, const float* bias, float*
     const bool vec_ok = (K % 4 == 0) && K < (1L << 22) && N < (1L << 24) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
     if (!vec_ok) {
         hipLaunchKernelGGL(gemm_naive_kernel, dim3((unsigned)cdiv(B * N, 256)), dim3(256), 0, s, A, W, C, B, N, K, epi);
+        HIP_OK(hipGetLastError());
+        return 0;
+    }
+    if (B <= 16) {
+        const dim3 grid((unsigned)cdiv(N, 4)), block(256);
+        if (B == 1) hipLaunchKernelGGL(gemm_small_kernel<1>, grid, block, 0, s, A, W, C, (int)B, N, K, epi);
+        else if (B <= 4) hipLaunchKernelGGL(gemm_small_kernel<4>, grid, block, 0, s, A, W, C, (int)B, N, K, epi);
+        else hipLaunchKernelGGL(gemm_small_kernel<16>, grid, block, 0, s, A, W, C, (int)B, N, K, epi);
         HIP_OK(hipGetLastError());
         return 0;
     }
