@@ -648,6 +648,26 @@ void mlp_forward_dev(void)
         fortis_capturing = 0;
         if (hipStreamEndCapture(s, &g) == hipSuccess && g && hipGraphInstantiate(&g_step.gexec, g, nullptr, nullptr, 0) == hipSuccess) {
             HIP_OK(hipGraphLaunch(g_step.gexec, s));
+            // Replay is kept only if it is measured to be no slower than launching the kernels one by one:
+            // on this runtime a graph launch costs more than a few plain launches, so short steps are
+            // faster eager.  The step is a pure function of the resident input, so the trial passes change
+            // nothing.  FORTIS_GRAPH_KEEP in the environment keeps the replay unconditionally.
+            if (!getenv("FORTIS_GRAPH_KEEP")) {
+                const int trials = 3;
+                hipEvent_t e0, e1, e2;
+                HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1)); HIP_OK(hipEventCreate(&e2));
+                HIP_OK(hipEventRecord(e0, s));
+                for (int i = 0; i < trials; i++) HIP_OK(hipGraphLaunch(g_step.gexec, s));
+                HIP_OK(hipEventRecord(e1, s));
+                for (int i = 0; i < trials; i++) fortis_plan_run(g_step.plan);
+                HIP_OK(hipEventRecord(e2, s));
+                HIP_OK(hipEventSynchronize(e2));
+                float replay_ms = 0.f, eager_ms = 0.f;
+                HIP_OK(hipEventElapsedTime(&replay_ms, e0, e1));
+                HIP_OK(hipEventElapsedTime(&eager_ms, e1, e2));
+                HIP_OK(hipEventDestroy(e0)); HIP_OK(hipEventDestroy(e1)); HIP_OK(hipEventDestroy(e2));
+                if (replay_ms > eager_ms) { HIP_OK(hipGraphExecDestroy(g_step.gexec)); g_step.gexec = nullptr; }
+            }
         } else {
             fprintf(stderr, "fortis: graph capture failed, running eagerly\n");
             g_step.gexec = nullptr;

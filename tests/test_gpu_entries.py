@@ -40,10 +40,12 @@ def test_whole_array_call_and_resident_entries(L, gpu):
     assert bits_equal(y, y2)
 
 
-def test_graph_capture_on_second_call_and_replay(L, gpu):
+def test_graph_capture_on_second_call_and_replay(L, gpu, monkeypatch):
     """fortis.graph set: call 1 eager, call 2 captures and launches, later calls replay
     (driver/fortis_shim.py:82-90).  Every replay must equal the eager result, with eager work and
-    synchronisations in between."""
+    synchronisations in between.  FORTIS_GRAPH_KEEP pins the replay (without it the library keeps the
+    graph only where it measures faster than plain launches)."""
+    monkeypatch.setenv("FORTIS_GRAPH_KEEP", "1")
     case, plan, ref = _toy()
     ST.bind(plan, case["X"].size, ref.size, graph=True)
     outs = []
@@ -69,10 +71,27 @@ def test_graph_env_switch(L, gpu, monkeypatch):
     assert not ST.graph_active()
     ST.reset()
     monkeypatch.setenv("FORTIS_GRAPH", "1")
+    monkeypatch.setenv("FORTIS_GRAPH_KEEP", "1")
     ST.bind(plan, case["X"].size, ref.size, graph=False)
     ST.mlp_forward(case["X"], y)
     ST.mlp_forward(case["X"], y)
     assert ST.graph_active() and maxrel(y, ref) < TOL
+
+
+def test_graph_kept_only_when_measured_faster(L, gpu):
+    """Without FORTIS_GRAPH_KEEP the second call captures, times replay against plain launches and keeps the
+    faster; either way every later call must give the eager result."""
+    case, plan, ref = _toy()
+    ST.bind(plan, case["X"].size, ref.size, graph=True)
+    y = np.empty_like(ref)
+    first = None
+    for n in range(5):
+        ST.mlp_forward(case["X"], y)
+        assert maxrel(y, ref) < TOL
+        first = y.copy() if first is None else first
+        assert bits_equal(y, first)
+    assert ST.graph_active() in (True, False)
+    ST.reset()
 
 
 def test_pack_batched_unpack(L, gpu):
@@ -164,10 +183,11 @@ def _corner_interp(Txy_h, maskBu, sx=68, sy=78):
     return out
 
 
-def test_zb_host_step_through_gather_batched_scatter(L, gpu, golden):
+def test_zb_host_step_through_gather_batched_scatter(L, gpu, golden, monkeypatch):
     """The fissioned ZB host's step (mom6_zb/host_fissioned.fir:732-740): fortis_gather(4 arrays) ->
     mlp_forward_batched() -> do k: fortis_scatter(k, 5 arrays) + host corner interpolation; results
     against the fixture written by the reference's own CPU build."""
+    monkeypatch.setenv("FORTIS_GRAPH_KEEP", "1")                   # exercise the replay path whatever the timing says
     gt, st, gd, sd, lp, kd = S.load_tables(*[os.path.join(golden, f"zb_{n}.json") for n in ("gather", "scatter", "loop", "kdist")])
     W = np.load(os.path.join(golden, "zb_nn.npz"))
     G = np.load(os.path.join(golden, "zb_native_golden.npz"))
