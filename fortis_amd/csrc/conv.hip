@@ -12,7 +12,7 @@
 #include "common.h"
 
 #define CONV_THREADS 256
-#define CONV_FB 8
+#define CONV_FB 8      // output channels per thread of the transposed-conv kernel and the wide direct kernel
 
 __device__ __forceinline__ float conv_epilogue(float acc, long f, long opos, long ospatial, const ConvEpi& e)
 {
@@ -29,41 +29,87 @@ struct ConvShape {
     int C, D, H, W, F, KD, KH, KW, Do, Ho, Wo, sd, sh, sw, pd, ph, pw;
 };
 
+// FB output channels per thread: 8 keeps an input value in a register for eight products; 1 gives a small
+// problem (the 3 -> 8 channel probe on 16^3) eight times as many threads to spread over the chip.
+#define CONV_WLDS 4096   // weights of a block's output channels staged in LDS when they fit (floats)
+// K3: the kernel is 3 x 3 x 3 (or 1 x 3 x 3) with stride 1: the tap loops are unrolled and every load is
+// issued unconditionally from a clamped coordinate (its weight is replaced by zero outside the image), so
+// a thread's loads overlap instead of each waiting behind a bounds branch.
+template <int FB, bool K3>
 __global__ __launch_bounds__(CONV_THREADS) void conv_direct_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                                    float* __restrict__ y, ConvShape s, ConvEpi e)
 {
+    __shared__ float sw[CONV_WLDS];
     const long ospatial = (long)s.Do * s.Ho * s.Wo;
     const long opos = (long)blockIdx.x * CONV_THREADS + threadIdx.x;
-    const int f0 = blockIdx.y * CONV_FB;
+    const int f0 = blockIdx.y * FB;
+    const int kvol = s.KD * s.KH * s.KW, ckv = s.C * kvol;
+    // the block's weights [FB][C][taps]: one cooperative copy instead of a scalar load (and its wait) per product
+    const bool wl = FB * ckv <= CONV_WLDS;
+    if (wl) {
+        for (int i = threadIdx.x; i < FB * ckv; i += CONV_THREADS) {
+            const int f = i / ckv;
+            sw[i] = f0 + f < s.F ? w[(long)f0 * ckv + i] : 0.f;
+        }
+        __syncthreads();
+    }
     if (opos >= ospatial) return;
     const int ox = (int)(opos % s.Wo), oy = (int)((opos / s.Wo) % s.Ho), oz = (int)(opos / ((long)s.Wo * s.Ho));
-    const int kvol = s.KD * s.KH * s.KW;
-    float acc[CONV_FB];
+    const long chan = (long)s.D * s.H * s.W;
+    float acc[FB];
 #pragma unroll
-    for (int f = 0; f < CONV_FB; f++) acc[f] = 0.f;
-    for (int c = 0; c < s.C; c++) {
-        const float* xc = x + (long)c * s.D * s.H * s.W;
-        const float* wc = w + ((long)f0 * s.C + c) * kvol;
-        for (int kd = 0; kd < s.KD; kd++) {
-            const int iz = oz * s.sd + kd - s.pd;
-            if (iz < 0 || iz >= s.D) continue;
-            for (int kh = 0; kh < s.KH; kh++) {
-                const int iy = oy * s.sh + kh - s.ph;
-                if (iy < 0 || iy >= s.H) continue;
-                for (int kw = 0; kw < s.KW; kw++) {
-                    const int ix = ox * s.sw + kw - s.pw;
-                    if (ix < 0 || ix >= s.W) continue;
-                    const float xv = xc[((long)iz * s.H + iy) * s.W + ix];
-                    const int k = (kd * s.KH + kh) * s.KW + kw;
+    for (int f = 0; f < FB; f++) acc[f] = 0.f;
+    if (K3 && wl) {
+        const int nkd = s.KD;                        // 3, or 1 for a 2-D convolution
+        for (int c = 0; c < s.C; c++) {
+            const float* xc = x + c * chan;
+            for (int kd = 0; kd < nkd; kd++) {
+                const int iz = oz + kd - s.pd;
+                const bool vz = iz >= 0 && iz < s.D;
+                const int cz = vz ? iz : 0;
+                float xv[9];
+                bool ok[9];
 #pragma unroll
-                    for (int f = 0; f < CONV_FB; f++)
-                        if (f0 + f < s.F) acc[f] = fmaf(xv, wc[(long)f * s.C * kvol + k], acc[f]);
+                for (int t = 0; t < 9; t++) {
+                    const int iy = oy + t / 3 - s.ph, ix = ox + t % 3 - s.pw;
+                    ok[t] = vz && iy >= 0 && iy < s.H && ix >= 0 && ix < s.W;
+                    const int cy = iy < 0 ? 0 : iy >= s.H ? s.H - 1 : iy, cx = ix < 0 ? 0 : ix >= s.W ? s.W - 1 : ix;
+                    xv[t] = xc[((long)cz * s.H + cy) * s.W + cx];
+                }
+#pragma unroll
+                for (int t = 0; t < 9; t++)
+#pragma unroll
+                    for (int f = 0; f < FB; f++)
+                        acc[f] = fmaf(ok[t] ? xv[t] : 0.f, sw[f * ckv + c * kvol + kd * 9 + t], acc[f]);
+            }
+        }
+    } else {
+    // taps outermost (bounds are checked once per tap), input channels innermost
+    for (int kd = 0; kd < s.KD; kd++) {
+        const int iz = oz * s.sd + kd - s.pd;
+        if (iz < 0 || iz >= s.D) continue;
+        for (int kh = 0; kh < s.KH; kh++) {
+            const int iy = oy * s.sh + kh - s.ph;
+            if (iy < 0 || iy >= s.H) continue;
+            for (int kw = 0; kw < s.KW; kw++) {
+                const int ix = ox * s.sw + kw - s.pw;
+                if (ix < 0 || ix >= s.W) continue;
+                const float* xp = x + ((long)iz * s.H + iy) * s.W + ix;
+                const int k = (kd * s.KH + kh) * s.KW + kw;
+                for (int c = 0; c < s.C; c++) {
+                    const float xv = xp[c * chan];
+#pragma unroll
+                    for (int f = 0; f < FB; f++) {
+                        const float wv = wl ? sw[f * ckv + c * kvol + k] : (f0 + f < s.F ? w[((long)(f0 + f) * s.C + c) * kvol + k] : 0.f);
+                        acc[f] = fmaf(xv, wv, acc[f]);
+                    }
                 }
             }
         }
     }
+    }
 #pragma unroll
-    for (int f = 0; f < CONV_FB; f++)
+    for (int f = 0; f < FB; f++)
         if (f0 + f < s.F) y[(long)(f0 + f) * ospatial + opos] = conv_epilogue(acc[f], f0 + f, opos, ospatial, e);
 }
 
@@ -260,6 +306,26 @@ __global__ void copy_kernel(const float* __restrict__ x, float* __restrict__ y, 
 
 static bool fits_int(long v) { return v > 0 && v < 2147483647L; }
 
+static void launch_direct(const float* x, const float* w, float* y, const ConvShape& sh, const ConvEpi& e, long ospatial, long F,
+                          hipStream_t s)
+{
+    static int cus = 0;
+    if (!cus) {
+        hipDeviceProp_t prop;
+        cus = hipGetDeviceProperties(&prop, 0) == hipSuccess ? prop.multiProcessorCount : 256;
+    }
+    const long blocks = cdiv(ospatial, CONV_THREADS);
+    const bool k3 = sh.KH == 3 && sh.KW == 3 && (sh.KD == 3 || sh.KD == 1) && sh.sd == 1 && sh.sh == 1 && sh.sw == 1;
+    const dim3 g1((unsigned)blocks, (unsigned)F), g8((unsigned)blocks, (unsigned)cdiv(F, 8)), b(CONV_THREADS);
+    if (blocks * cdiv(F, 8) < cus) {
+        if (k3) hipLaunchKernelGGL((conv_direct_kernel<1, true>), g1, b, 0, s, x, w, y, sh, e);
+        else hipLaunchKernelGGL((conv_direct_kernel<1, false>), g1, b, 0, s, x, w, y, sh, e);
+    } else {
+        if (k3) hipLaunchKernelGGL((conv_direct_kernel<8, true>), g8, b, 0, s, x, w, y, sh, e);
+        else hipLaunchKernelGGL((conv_direct_kernel<8, false>), g8, b, 0, s, x, w, y, sh, e);
+    }
+}
+
 int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long D, long H, long Wd, long F, long KD,
                          long KH, long KW, long Do, long Ho, long Wo, long pd, long ph, long pw, const ConvEpi& e,
                          hipStream_t s)
@@ -288,8 +354,7 @@ int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long 
     }
     ConvShape sh = { (int)C, (int)D, (int)H, (int)Wd, (int)F, (int)KD, (int)KH, (int)KW, (int)Do, (int)Ho, (int)Wo, 1, 1, 1,
                      (int)pd, (int)ph, (int)pw };
-    hipLaunchKernelGGL(conv_direct_kernel, dim3((unsigned)cdiv(Do * Ho * Wo, CONV_THREADS), (unsigned)cdiv(F, CONV_FB)),
-                       dim3(CONV_THREADS), 0, s, x, w, y, sh, e);
+    launch_direct(x, w, y, sh, e, Do * Ho * Wo, F, s);
     HIP_OK(hipGetLastError());
     return 0;
 }
@@ -302,8 +367,7 @@ int fortis_launch_conv2d(const float* x, const float* w, float* y, long C, long 
     if (Ho != (H + 2 * ph - KH) / sh_ + 1 || Wo != (Wd + 2 * pw - KW) / sw_ + 1 || coff < 0 || coff + F > ctot) return -1;
     ConvShape sh = { (int)C, 1, (int)H, (int)Wd, (int)F, 1, (int)KH, (int)KW, 1, (int)Ho, (int)Wo, 1, (int)sh_, (int)sw_,
                      0, (int)ph, (int)pw };
-    hipLaunchKernelGGL(conv_direct_kernel, dim3((unsigned)cdiv(Ho * Wo, CONV_THREADS), (unsigned)cdiv(F, CONV_FB)),
-                       dim3(CONV_THREADS), 0, s, x, w, y + coff * Ho * Wo, sh, e);
+    launch_direct(x, w, y + coff * Ho * Wo, sh, e, Ho * Wo, F, s);
     HIP_OK(hipGetLastError());
     return 0;
 }

@@ -4,6 +4,10 @@ only (git-ignored).  Test infrastructure: run by tests/test_gpu_hosts.py, built 
 
   toy_dev_hip     benchmarks/toy/bench_dev.f90  (mlp_upload / mlp_forward_dev x1000 / mlp_download; the
                   model is frontend/export_mlp.py's: seed 42, Linear(1024,256) ReLU Linear(256,1024))
+  toy_call_hip    benchmarks/toy/bench_fortis.f90  (mlp_forward(x, y) x1000: upload, step, download per call)
+  conv_dev_hip    benchmarks/toy/bench_dev_conv.f90, conv_call_hip  benchmarks/toy/bench_fortis_conv.f90
+                  (the same two call patterns on frontend/export_conv.py's model: seed 3, Conv3d(3,8,3,pad 1)
+                  LeakyReLU(0.1) on 1x3x16^3)
   zb_expert_hip   mom6_zb/zb_host_expert.f90    (per-layer hand-batched mlp_forward(xb(27,4736), yb(3,4736));
                   the model is mom6_zb/zb_nn.npz with its input and output norms)
 
@@ -53,12 +57,22 @@ def main():
     bs = [net[0].bias.detach().numpy(), net[2].bias.detach().numpy()]
     c, _ = emit.emit_mlp_step(os.path.join(OUT, "toy_dev_step"), Ws, bs, ["relu", None], rows=1, graph=True)
     link(os.path.join(REF, "benchmarks/toy/bench_dev.f90"), c, "toy_dev_hip")
+    c, _ = emit.emit_mlp_step(os.path.join(OUT, "toy_call_step"), Ws, bs, ["relu", None], rows=1)
+    link(os.path.join(REF, "benchmarks/toy/bench_fortis.f90"), c, "toy_call_hip")
+    # conv probe: the exporter's model from its seed (frontend/export_conv.py:3-4)
+    torch.manual_seed(3)
+    conv = torch.nn.Conv3d(3, 8, 3, padding=1)
+    cw, cb = conv.weight.detach().numpy(), conv.bias.detach().numpy()
+    c, _ = emit.emit_conv3d_step(os.path.join(OUT, "conv_dev_step"), cw, cb, (3, 16, 16, 16), act="leaky", alpha=0.1, graph=True)
+    link(os.path.join(REF, "benchmarks/toy/bench_dev_conv.f90"), c, "conv_dev_hip")
+    c, _ = emit.emit_conv3d_step(os.path.join(OUT, "conv_call_step"), cw, cb, (3, 16, 16, 16), act="leaky", alpha=0.1)
+    link(os.path.join(REF, "benchmarks/toy/bench_fortis_conv.f90"), c, "conv_call_hip")
     # ZB expert host: one call per layer on 4736 cells
     W = np.load(os.path.join(ROOT, "tests", "golden", "zb_nn.npz"))
     c, _ = emit.emit_mlp_step(os.path.join(OUT, "zb_expert_step"), [W["A0"], W["A1"]], [W["b0"], W["b1"]], ["relu", None],
                               rows=4736, in_norms=W["in_norms"], out_norms=W["out_norms"])
     link(os.path.join(REF, "mom6_zb/zb_host_expert.f90"), c, "zb_expert_hip")
-    print("build_hosts: built toy_dev_hip, zb_expert_hip in", OUT)
+    print("build_hosts: built toy_dev_hip, toy_call_hip, conv_dev_hip, conv_call_hip, zb_expert_hip in", OUT)
     return 0
 
 

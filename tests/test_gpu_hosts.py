@@ -34,6 +34,24 @@ def test_toy_host_upload_forward_dev_download(gpu, tmp_path):
     assert 0 < per_call < 1000
 
 
+def test_toy_host_per_call(gpu, tmp_path):
+    """benchmarks/toy/bench_fortis.f90: mlp_forward(x, y) with upload and download inside every call."""
+    out = run_host("toy_call_hip", tmp_path)
+    chk = float(re.search(r"checksum:\s*([-0-9.Ee+]+)", out).group(1))
+    assert abs(chk - 7.775037) / 7.775037 < 1e-5, out
+    print("toy host per-call (upload + step + download) us:", float(re.search(r"per-call us:\s*([-0-9.Ee+]+)", out).group(1)))
+
+
+@pytest.mark.parametrize("exe", ["conv_dev_hip", "conv_call_hip"])
+def test_conv_probe_hosts(gpu, tmp_path, exe):
+    """benchmarks/toy/bench_dev_conv.f90 / bench_fortis_conv.f90 on the conv probe; README.md:25 stamps the
+    checksum 9617.28 (an fp32 sum of 32768 terms: agreement to 3e-5)."""
+    out = run_host(exe, tmp_path)
+    chk = float(re.search(r"checksum:\s*([-0-9.Ee+]+)", out).group(1))
+    assert abs(chk - 9617.28) / 9617.28 < 3e-5, out
+    print(exe, "per-call us:", float(re.search(r"per-call us:\s*([-0-9.Ee+]+)", out).group(1)))
+
+
 def test_zb_expert_host_matches_native_golden(gpu, tmp_path, golden):
     """mom6_zb/zb_host_expert.f90: the host packs 4736 stencils per layer itself and calls
     mlp_forward(xb, yb) 15 x 11 times; its Txx/Tyy/Txy must agree with the reference's native CPU build
