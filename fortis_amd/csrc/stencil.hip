@@ -145,7 +145,8 @@ struct BoundStencil {
     fortis_stencil_t host;       // as configured (cells pointer not owned)
     StencilDev low;              // lowered table
     int* dcells = nullptr;       // device copy of the cell list
-    void* darr[FORTIS_MAX_ARRAYS] = {};       // device planes of the host arrays
+    void* darr[FORTIS_MAX_ARRAYS] = {};       // planes of the host arrays: device memory (gather) or page-locked host memory (scatter)
+    bool host_planes = false;
     const void* reg[FORTIS_MAX_ARRAYS] = {};  // last host address seen per array
     bool written[FORTIS_MAX_ARRAYS] = {};
     bool init = false;
@@ -166,7 +167,8 @@ static int upload_table(const fortis_stencil_t* t, StencilDev* low, int** dcells
 static void release(BoundStencil& b)
 {
     if (b.dcells) HIP_OK(hipFree(b.dcells));
-    for (int a = 0; a < FORTIS_MAX_ARRAYS; a++) if (b.darr[a]) HIP_OK(hipFree(b.darr[a]));
+    for (int a = 0; a < FORTIS_MAX_ARRAYS; a++)
+        if (b.darr[a]) { if (b.host_planes) HIP_OK(hipHostFree(b.darr[a])); else HIP_OK(hipFree(b.darr[a])); }
     b = BoundStencil();
 }
 
@@ -283,40 +285,50 @@ void fortis_scatter_v(const int* a, void* const* H)
     if (!b.ok) { fprintf(stderr, "fortis_scatter: no scatter table configured\n"); return; }
     hipStream_t s = fortis_stream_get();
     const fortis_stencil_t& t = b.host;
+    // One page-locked host plane per array, which the kernel reads and writes directly over the bus: the
+    // scalars' planes are copied in by the CPU, the visited cells of the written planes are copied out by
+    // the CPU after the one synchronisation.  The reference issues two uploads and three pitched downloads
+    // per call (gather.cu:84-90); as copy commands from and to pageable memory those cost far more than the
+    // kernel here (a pitched download is handled row by row).
     if (!b.init) {
-        for (int ai = 0; ai < t.narrays; ai++) HIP_OK(hipMalloc(&b.darr[ai], (size_t)t.plane[ai] * sizeof(float)));   // gather.cu:60-64
+        for (int ai = 0; ai < t.narrays; ai++) HIP_OK(hipHostMalloc(&b.darr[ai], (size_t)t.plane[ai] * sizeof(float), hipHostMallocDefault));
+        b.host_planes = true;
         b.init = true;
     }
     const int k1 = a ? a[0] : 1;   // 1-based enclosing-loop index
+    bool whole_plane[FORTIS_MAX_ARRAYS] = {};
+    for (int r = 0; r < t.nrefs; r++)
+        if (t.cells || t.refs[r].si != 1) whole_plane[t.refs[r].array] = true;
     float* dptr[FORTIS_MAX_ARRAYS];
     for (int ai = 0; ai < t.narrays; ai++) {
         note_host(b, ai, H[ai]);
         dptr[ai] = (float*)b.darr[ai];
-        if (!b.written[ai]) {
+        // inputs always; a written array only when its whole plane goes back (unvisited cells must survive)
+        if (!b.written[ai] || whole_plane[ai]) {
             const long off = t.total[ai] > t.plane[ai] ? (long)(k1 - 1) * t.plane[ai] : 0;
-            HIP_OK(hipMemcpyAsync(b.darr[ai], (const float*)H[ai] + off, t.plane[ai] * sizeof(float), hipMemcpyHostToDevice, s));
+            memcpy(b.darr[ai], (const float*)H[ai] + off, t.plane[ai] * sizeof(float));
         }
     }
-    // the device holds ONE plane per array here, so the kernel runs with plane index 0
+    // the staging holds ONE plane per array, so the kernel runs with plane index 0
     const long yoff = t.nk > 1 ? (long)(k1 - t.klo) * t.count * t.nrefs : 0;   // gather.cu:86
     launch_scatter(b.low, dptr, (const float*)fortis_model_output() + yoff, 0, s);
+    HIP_OK(hipStreamSynchronize(s));
     for (int r = 0; r < t.nrefs; r++) {
         const int ai = t.refs[r].array;
         const long off = t.total[ai] > t.plane[ai] ? (long)(k1 - 1) * t.plane[ai] : 0;
         float* hbase = (float*)H[ai] + off;
-        if (t.cells || t.refs[r].si != 1) {
+        const float* stage = (const float*)b.darr[ai];
+        if (whole_plane[ai]) {
             // cell list or non-unit inner stride: no rectangle to copy, return the whole plane
-            HIP_OK(hipMemcpyAsync(hbase, b.darr[ai], t.plane[ai] * sizeof(float), hipMemcpyDeviceToHost, s));
+            memcpy(hbase, stage, t.plane[ai] * sizeof(float));
         } else {
             // visited rectangle, pitch = stride of the j index (gather.cu:87-89; gather_emit.py:88-95)
             const long rect = t.refs[r].base + (long)t.ilo * t.refs[r].si + (long)t.jlo * t.refs[r].sj;
             const long pitch = t.refs[r].sj > 0 ? t.refs[r].sj : t.ni;
-            HIP_OK(hipMemcpy2DAsync(hbase + rect, pitch * sizeof(float), (float*)b.darr[ai] + rect, pitch * sizeof(float),
-                                    (size_t)t.ni * sizeof(float), (size_t)(t.nj > 0 ? t.nj : t.count / t.ni),
-                                    hipMemcpyDeviceToHost, s));
+            const long nrow = t.nj > 0 ? t.nj : t.count / t.ni;
+            for (long j = 0; j < nrow; j++) memcpy(hbase + rect + j * pitch, stage + rect + j * pitch, (size_t)t.ni * sizeof(float));
         }
     }
-    HIP_OK(hipStreamSynchronize(s));
 }
 
 void fortis_gather(const float* H0, const float* H1, const float* H2, const float* H3)
