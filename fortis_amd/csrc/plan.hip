@@ -736,14 +736,19 @@ void mlp_forward_batched(void* in, void* out)
         HIP_OK(hipStreamSynchronize(s));
         return;
     }
-    // strided / offset loop: rows minc, minc+|step|, ... of the host arrays (driver/fortis_shim.py:119-121)
+    // strided / offset loop: rows minc, minc+|step|, ... of the host arrays (driver/fortis_shim.py:119-121, a
+    // cudaMemcpy2D there).  Pitched copies from and to pageable memory are executed row by row by the runtime,
+    // so the rows are packed by the CPU into page-locked staging and cross the bus as one copy each way.
     const long st = h.step < 0 ? -h.step : h.step;
-    HIP_OK(hipMemcpy2DAsync(g_step.din, NIN, (const char*)in + (size_t)(h.minc - 1) * NIN, (size_t)st * NIN, NIN, (size_t)h.count,
-                            hipMemcpyHostToDevice, s));
+    if (!g_step.X) setup_xy();
+    for (long r = 0; r < h.count; r++)
+        memcpy((char*)g_step.X + (size_t)r * NIN, (const char*)in + (size_t)(h.minc - 1 + r * st) * NIN, NIN);
+    HIP_OK(hipMemcpyAsync(g_step.din, g_step.X, NIN * h.count, hipMemcpyHostToDevice, s));
     mlp_forward_dev();
-    HIP_OK(hipMemcpy2DAsync((char*)out + (size_t)(h.minc - 1) * NOUT, (size_t)st * NOUT, g_step.dout, NOUT, NOUT, (size_t)h.count,
-                            hipMemcpyDeviceToHost, s));
+    HIP_OK(hipMemcpyAsync(g_step.Y, g_step.dout, NOUT * h.count, hipMemcpyDeviceToHost, s));
     HIP_OK(hipStreamSynchronize(s));
+    for (long r = 0; r < h.count; r++)
+        memcpy((char*)out + (size_t)(h.minc - 1 + r * st) * NOUT, (const char*)g_step.Y + (size_t)r * NOUT, NOUT);
 }
 
 void mlp_forward(void* in, void* out)
