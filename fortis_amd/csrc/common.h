@@ -14,6 +14,7 @@
             fprintf(stderr, "fortis: %s failed: %s (%s:%d)\n", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
     } while (0)
 
+extern "C" long fortis_step_generation(void);   // plan.hip: count of forward passes of the bound step
 static inline hipStream_t fortis_stream_get() { return (hipStream_t)mgpuStreamCreate(); }
 static inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 

@@ -623,12 +623,15 @@ static bool bound(const char* who)
     return true;
 }
 
+static long g_forward_gen = 0;   // bumped by every forward pass of the bound step
 void* fortis_model_input(void) { return g_step.din; }
 void* fortis_model_output(void) { return g_step.dout; }
+long fortis_step_generation(void) { return g_forward_gen; }   // internal: lets the scatter entry notice a new forward pass
 
 void mlp_forward_dev(void)
 {
     if (!bound("mlp_forward_dev")) return;
+    g_forward_gen++;
     hipStream_t s = fortis_stream_get();
     if (g_step.gexec) { HIP_OK(hipGraphLaunch(g_step.gexec, s)); return; }
     const int cap = (++g_step.ncalls == 2) && (g_step.h.graph || getenv("FORTIS_GRAPH") != 0);
@@ -782,6 +785,7 @@ void mlp_forward(void* in, void* out)
         void* dout = p->tptr[p->out_t];
         p->tptr[p->in_t] = g_step.X;
         p->tptr[p->out_t] = g_step.Y;
+        g_forward_gen++;
         fortis_plan_run(p);
         p->tptr[p->in_t] = din;
         p->tptr[p->out_t] = dout;

@@ -218,3 +218,46 @@ def test_zb_host_step_through_gather_batched_scatter(L, gpu, golden, monkeypatch
     X = np.empty((71040, 27), np.float32)
     L.fortis_d2h(X.ctypes.data, L.fortis_model_input(), X.nbytes)
     assert bits_equal(X, O.stencil_gather(gd, [Pp["sh_xy_h"], F["sh_xx"], Pp["vort_xy_h"], Pp["norm_h"]], 4736, 15, 3, 3, 64))
+
+
+def test_scatter_reuse_is_verified_against_the_host_arrays(L, gpu, golden):
+    """Under loop distribution the first fortis_scatter of a step computes every iteration and later calls
+    only copy rows out -- but only while the scalars' planes the host passes are still the bytes read at the
+    first call.  A host that changes norm_h(:,:,k) between two scatter calls must get the result for the
+    changed values (the one-iteration path), bit for bit what the per-call path gives."""
+    gt, st, gd, sd, lp, kd = S.load_tables(*[os.path.join(golden, f"zb_{n}.json") for n in ("gather", "scatter", "loop", "kdist")])
+    W = np.load(os.path.join(golden, "zb_nn.npz"))
+    F = O.zb_fields()
+    Pp = O.zb_prep(F)
+    n3 = 68 * 78 * 15
+    results = {}
+    for mode in ("reuse", "per_call"):
+        if mode == "per_call":
+            os.environ["FORTIS_SCATTER_PER_CALL"] = "1"
+        try:
+            ST.reset()
+            plan = P.mlp_plan([W["A0"], W["A1"]], [W["b0"], W["b1"]], ["relu", None], 71040, in_norms=W["in_norms"], out_norms=W["out_norms"])
+            ST.bind(plan, 71040 * 27, 71040 * 3, verdict="batched", expanded=True, count=71040, gather=True, scatter=True)
+            ST.gather_config(gt)
+            ST.scatter_config(st)
+            norm = Pp["norm_h"].copy()
+            Txy_h, Txx, Tyy = np.zeros(68 * 78, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)
+            L.fortis_gather(*[a.ctypes.data for a in (Pp["sh_xy_h"], F["sh_xx"], Pp["vort_xy_h"], norm)])
+            ST.mlp_forward_batched()
+            planes = []
+            for k in range(1, 16):
+                if k == 7:
+                    norm.reshape(15, 78, 68)[6] *= np.float32(1.5)          # the host changes layer 7's scalars
+                L.fortis_scatter(k, *[a.ctypes.data for a in (norm, F["kappa_h"], Txy_h, Txx, Tyy)])
+                planes.append(Txy_h.copy())
+            results[mode] = (Txx.copy(), Tyy.copy(), np.stack(planes))
+            plan.close()
+        finally:
+            os.environ.pop("FORTIS_SCATTER_PER_CALL", None)
+    for a, b in zip(results["reuse"], results["per_call"]):
+        assert bits_equal(a, b)
+    # and layer 7 really was computed from the changed scalars: (y * S0 * S0) * S1 grows by 1.5^2 there
+    G = np.load(os.path.join(golden, "zb_native_golden.npz"))
+    Txx = results["reuse"][0].reshape(15, 78, 68)
+    assert maxrel(Txx[7], G["Txx"][1]) < TOL                       # layer 8 untouched
+    assert np.abs(Txx[6]).max() > 0
