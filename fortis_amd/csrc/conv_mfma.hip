@@ -16,7 +16,7 @@
 // (zero-filled outside the image), and every B operand is a single ds_read at lane base + constant.
 // Weights are re-packed once at plan time in exactly the order the kernel consumes them, so their
 // staging is a straight 16-byte copy.  Both are double buffered through registers.
-#include "common.h"
+#include "stencil_dev.h"      // StMagic / st_divmod: exact division by a launch constant
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float cm_v4f __attribute__((ext_vector_type(4)));   // native vector: conditional copies stay in registers
@@ -33,6 +33,7 @@ struct ConvMShape {
     float* part;               // [ksplit][output elements]
     int ups;                   // 1: the input tensor is (D/2, H/2, W/2) and is read through a nearest x2 upsample
     long osize;                // output elements
+    StMagic mP, mR, mKR;       // exact division by P, R and KD * R (the staging map would otherwise spend its time dividing)
 };
 
 // FT output channels per workgroup: 64 (waves 2 x 2 over channels x positions) or 32 (4 waves over positions).
@@ -78,10 +79,12 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         goff[i] = -1;
         gch[i] = 0;
         if (el < XCH) {
-            const int c = el / (KD * s.R), rem = el - c * (KD * s.R), kd = rem / s.R, r = rem - kd * s.R;
-            const int v = m0 + r, yp = v / s.P, xp = v - yp * s.P;
-            const int zz = z + kd - (KD / 2), yy = yp - PADK, xx = xp - PADK;
-            gch[i] = c;
+            unsigned c, rem, kd, r, yp, xp;
+            st_divmod((unsigned)el, s.mKR, c, rem);
+            st_divmod(rem, s.mR, kd, r);
+            st_divmod((unsigned)(m0 + r), s.mP, yp, xp);
+            const int zz = z + (int)kd - (KD / 2), yy = (int)yp - PADK, xx = (int)xp - PADK;
+            gch[i] = (int)c;
             if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W)
                 goff[i] = (int)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh));
         }
@@ -166,8 +169,9 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     for (int j = 0; j < NMT; j++) {
         const int m = m0 + (mt0 + j) * 32 + (lane & 31);
         if (m >= s.plane) continue;
-        const int yy = m / s.P, xx = m - yy * s.P;
-        if (xx >= s.W) continue;
+        unsigned yy, xx;
+        st_divmod((unsigned)m, s.mP, yy, xx);
+        if ((int)xx >= s.W) continue;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int f = fg * FT + ft * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
@@ -257,6 +261,7 @@ static int launch(const float* x, const float* wp, float* y, ConvMShape s, const
     constexpr int T = KD * KS * KS;
     s.tiles = (int)cdiv(s.plane, MT);
     s.R = MT + (KS == 3 ? 2 * s.P + 2 : 0);
+    s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
     if ((long)CM_CC * KD * s.R > (long)CM_THREADS * CM_NXMAX) return -1;     // run too long to stage
     const size_t shmem = (size_t)2 * (2 * T * 2 * FT + CM_CC * KD * s.R) * sizeof(float);
     if (shmem > 160 * 1024) return -1;
