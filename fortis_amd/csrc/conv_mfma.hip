@@ -22,8 +22,12 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float cm_v4f __attribute__((ext_vector_type(4)));   // native vector: conditional copies stay in registers
 
 #define CM_THREADS 256
-#define CM_CC 4        // input channels per staged chunk (two MFMA channel pairs)
-#define CM_NXMAX 16    // staged input elements per thread per chunk, at most
+// Input channels per staged chunk.  A chunk's multiply phase has to outlast the latency of the next
+// chunk's global loads: with 9 or 27 taps 4 channels do, a single tap takes 16.  (8 channels at 9 taps
+// gain 10% on 32 x 32 images and lose 30% on 256 x 256 ones, whose halo then no longer fits the larger tile.)
+static constexpr int cm_cc(int T) { return T >= 9 ? 4 : 16; }
+// staged input elements per thread per chunk, at most
+static constexpr int cm_nx(int T) { return cm_cc(T) == 8 ? 24 : 16; }
 
 struct ConvMShape {
     int C, D, H, W, F;         // F = output channels of the GEMM (4x the real ones in transposed mode)
@@ -50,7 +54,8 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
 {
     constexpr int T = KD * KS * KS;
-    constexpr int WCH = 2 * T * 2 * FT;                          // floats of packed weights per chunk
+    constexpr int CC = cm_cc(T), NCP = CC / 2, NX = cm_nx(T);
+    constexpr int WCH = NCP * T * 2 * FT;                        // floats of packed weights per chunk
     constexpr int NW = (WCH / 4 + CM_THREADS - 1) / CM_THREADS;  // float4 per thread
     constexpr int FW = FT / 32;                                  // waves along the channels
     constexpr int NMT = MT / 32 / (4 / FW);                      // m-tiles per wave
@@ -58,8 +63,8 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     constexpr int PADK = KS / 2;
     extern __shared__ float4 smem4[];
     float* sW = (float*)smem4;                                    // [2][WCH]
-    float* sX = sW + 2 * WCH;                                     // [2][CM_CC * KD * R]
-    const int XCH = CM_CC * KD * s.R;
+    float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R]
+    const int XCH = CC * KD * s.R;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int z = blockIdx.x / s.tiles, tile = blockIdx.x - z * s.tiles;
@@ -70,28 +75,26 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     const int sh = s.ups ? 1 : 0;
     const long srcW = s.W >> sh, sHW = (long)(s.H >> sh) * srcW, schan = (long)(s.D >> sh) * sHW;
 
-    // per-thread staging map of the input run (same for every chunk): global offset inside a 4-channel group
-    int goff[CM_NXMAX];
-    int gch[CM_NXMAX];
+    // per-thread staging map of the input run (same for every chunk): global offset inside a chunk's
+    // channel group, c * schan + offset in the channel; -1: zero padding
+    int goff[NX];
 #pragma unroll
-    for (int i = 0; i < CM_NXMAX; i++) {
+    for (int i = 0; i < NX; i++) {
         const int el = tid + i * CM_THREADS;
         goff[i] = -1;
-        gch[i] = 0;
         if (el < XCH) {
             unsigned c, rem, kd, r, yp, xp;
             st_divmod((unsigned)el, s.mKR, c, rem);
             st_divmod(rem, s.mR, kd, r);
             st_divmod((unsigned)(m0 + r), s.mP, yp, xp);
             const int zz = z + (int)kd - (KD / 2), yy = (int)yp - PADK, xx = (int)xp - PADK;
-            gch[i] = (int)c;
             if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W)
                 goff[i] = (int)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh));
         }
     }
 
     cm_v4f rw[NW];
-    float rx[CM_NXMAX];
+    float rx[NX];
     auto load_chunk = [&](int ch) {
         const cm_v4f* wsrc = (const cm_v4f*)(wp + ((long)fg * s.nchunks + ch) * WCH);
 #pragma unroll
@@ -99,13 +102,17 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
             const int f4 = tid + i * CM_THREADS;
             rw[i] = wsrc[f4 < WCH / 4 ? f4 : 0];
         }
-        const float* xsrc = x + (long)ch * CM_CC * schan;
+        const float* xsrc = x + (long)ch * CC * schan;
+        // offsets at or beyond lim belong to channels past the last one (partial last chunk); as
+        // unsigned, the padding mark -1 is beyond it too
+        const int cleft = s.C - ch * CC;
+        const unsigned lim = (unsigned)((cleft < CC ? cleft : CC) * schan);
 #pragma unroll
-        for (int i = 0; i < CM_NXMAX; i++)
+        for (int i = 0; i < NX; i++)
         {
             // always load from a valid address (the element itself, or element 0 of a valid channel) and
             // select afterwards: no branch around the load
-            const bool ok = goff[i] >= 0 && ch * CM_CC + gch[i] < s.C;
+            const bool ok = (unsigned)goff[i] < lim;
             const float v = xsrc[ok ? goff[i] : 0];
             rx[i] = ok ? v : 0.f;
         }
@@ -119,7 +126,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         }
         float* xdst = sX + buf * XCH;
 #pragma unroll
-        for (int i = 0; i < CM_NXMAX; i++) {
+        for (int i = 0; i < NX; i++) {
             const int el = tid + i * CM_THREADS;
             if (el < XCH) xdst[el] = rx[i];
         }
@@ -145,7 +152,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         const float* w = sW + buf * WCH + wbase;
         const float* xs = sX + buf * XCH + xbase;
 #pragma unroll
-        for (int cp = 0; cp < 2; cp++)
+        for (int cp = 0; cp < NCP; cp++)
 #pragma unroll
             for (int kd = 0; kd < KD; kd++)
 #pragma unroll
@@ -225,27 +232,29 @@ static int conv_cus()
 }
 
 // Packs conv weights W[F][C][T] (T taps, row-major) into the kernel's order
-//   [F/FT][ceil(C/4)][channel pair 2][tap T][half 2][FT channels], zero padded; FT = 32 when the GEMM
-//   has at most 32 output channels, else 64 (the launcher applies the same rule).
+//   [F/FT][ceil(C/CC)][channel pair CC/2][tap T][half 2][FT channels], zero padded; CC = cm_cc(T)
+//   channels per chunk; FT = 32 when the GEMM has at most 32 output channels, else 64 (the launcher
+//   applies the same rules).
 // Transposed 2x2 conv: W is [C][F][2][2]; GEMM channel f' = f*4 + a*2 + b.
 float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats)
 {
     const long Fg = transposed ? 4 * F : F;
     const long FT = conv_ft(Fg);
-    const long nfg = cdiv(Fg, FT), nch = cdiv(C, CM_CC);
-    const long wch = 2L * T * 2 * FT;
+    const long CC = cm_cc(T), NCP = CC / 2;
+    const long nfg = cdiv(Fg, FT), nch = cdiv(C, CC);
+    const long wch = NCP * T * 2 * FT;
     const long n = nfg * nch * wch;
     float* h = (float*)calloc(n, sizeof(float));
     for (long fgi = 0; fgi < nfg; fgi++)
         for (long ch = 0; ch < nch; ch++)
-            for (int cp = 0; cp < 2; cp++)
+            for (int cp = 0; cp < NCP; cp++)
                 for (int t = 0; t < T; t++)
                     for (int hh = 0; hh < 2; hh++)
                         for (int fl = 0; fl < FT; fl++) {
-                            const long f = fgi * FT + fl, c = ch * CM_CC + cp * 2 + hh;
+                            const long f = fgi * FT + fl, c = ch * CC + cp * 2 + hh;
                             if (f >= Fg || c >= C) continue;
                             const float v = transposed ? W[(c * F + (f >> 2)) * 4 + (f & 3)] : W[(f * C + c) * T + t];
-                            h[((fgi * nch + ch) * 2 + cp) * T * 2 * FT + ((long)t * 2 + hh) * FT + fl] = v;
+                            h[((fgi * nch + ch) * NCP + cp) * T * 2 * FT + ((long)t * 2 + hh) * FT + fl] = v;
                         }
     float* d = nullptr;
     HIP_OK(hipMalloc((void**)&d, n * sizeof(float)));
@@ -259,11 +268,12 @@ template <int KD, int KS, int MT, int FT>
 static int launch(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {
     constexpr int T = KD * KS * KS;
+    constexpr int CC = cm_cc(T);
     s.tiles = (int)cdiv(s.plane, MT);
     s.R = MT + (KS == 3 ? 2 * s.P + 2 : 0);
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
-    if ((long)CM_CC * KD * s.R > (long)CM_THREADS * CM_NXMAX) return -1;     // run too long to stage
-    const size_t shmem = (size_t)2 * (2 * T * 2 * FT + CM_CC * KD * s.R) * sizeof(float);
+    if ((long)CC * KD * s.R > (long)CM_THREADS * cm_nx(T)) return -1;     // run too long to stage
+    const size_t shmem = (size_t)2 * (CC * T * FT + CC * KD * s.R) * sizeof(float);
     if (shmem > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
@@ -275,9 +285,9 @@ static int launch(const float* x, const float* wp, float* y, ConvMShape s, const
     const long wgs = (long)s.D * s.tiles * cdiv(s.F, FT);
     s.ksplit = 1;
     s.chunks_per = s.nchunks;
-    if (2 * wgs < 3 * conv_cus() && s.nchunks >= 8) {
+    if (2 * wgs < 3 * conv_cus() && s.C >= 32) {
         long k = cdiv(2L * conv_cus(), wgs);
-        if (k > s.nchunks / 4) k = s.nchunks / 4;
+        if (k > s.C / 16) k = s.C / 16;               // at least 16 input channels per split
         if (k > 16) k = 16;
         s.chunks_per = (int)cdiv(s.nchunks, k);
         s.ksplit = (int)cdiv(s.nchunks, s.chunks_per);
@@ -314,7 +324,7 @@ static int launch_mt(const float* x, const float* wp, float* y, ConvMShape s, co
 {
     s.P = KS == 3 ? s.W + 1 : s.W;
     s.plane = s.H * s.P;
-    s.nchunks = (int)cdiv(s.C, CM_CC);
+    s.nchunks = (int)cdiv(s.C, cm_cc(KD * KS * KS));
     const long want = 2L * conv_cus(), groups = (long)s.D * cdiv(s.F, FT);
     constexpr int MTMIN = FT == 64 ? 64 : 128;
     if (KD == 1 && groups * cdiv(s.plane, 256) >= want && launch<KD, KS, 256, FT>(x, wp, y, s, e, st) == 0) return 0;
