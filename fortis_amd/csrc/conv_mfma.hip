@@ -25,9 +25,8 @@ typedef float cm_v4f __attribute__((ext_vector_type(4)));   // native vector: co
 // Input channels per staged chunk.  A chunk's multiply phase has to outlast the latency of the next
 // chunk's global loads: with 9 or 27 taps 4 channels do, a single tap takes 16.  (8 channels at 9 taps
 // gain 10% on 32 x 32 images and lose 30% on 256 x 256 ones, whose halo then no longer fits the larger tile.)
-static constexpr int cm_cc(int T) { return T >= 9 ? 4 : 16; }
-// staged input elements per thread per chunk, at most
-static constexpr int cm_nx(int T) { return cm_cc(T) == 8 ? 24 : 16; }
+static constexpr int cm_cc(int T) { return T >= 27 ? 2 : T >= 9 ? 4 : 16; }
+#define CM_NXMAX 16   // staging rounds of the input run, at most (the kernel is built for 8 and for 16)
 
 struct ConvMShape {
     int C, D, H, W, F;         // F = output channels of the GEMM (4x the real ones in transposed mode)
@@ -49,12 +48,12 @@ __device__ __forceinline__ void cm_lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <int KD, int KS, int MT, int FT>
+template <int KD, int KS, int MT, int FT, int NX>
 __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
 {
     constexpr int T = KD * KS * KS;
-    constexpr int CC = cm_cc(T), NCP = CC / 2, NX = cm_nx(T);
+    constexpr int CC = cm_cc(T), NCP = CC / 2;       // NX: staging rounds of the input run (8 or 16)
     constexpr int WCH = NCP * T * 2 * FT;                        // floats of packed weights per chunk
     constexpr int NW = (WCH / 4 + CM_THREADS - 1) / CM_THREADS;  // float4 per thread
     constexpr int FW = FT / 32;                                  // waves along the channels
@@ -63,8 +62,9 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     constexpr int PADK = KS / 2;
     extern __shared__ float4 smem4[];
     float* sW = (float*)smem4;                                    // [2][WCH]
-    float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R]
+    float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R rounded up to the workgroup size]
     const int XCH = CC * KD * s.R;
+    const int XCHP = (XCH + CM_THREADS - 1) / CM_THREADS * CM_THREADS;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int z = blockIdx.x / s.tiles, tile = blockIdx.x - z * s.tiles;
@@ -93,6 +93,12 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         }
     }
 
+    // offsets at or beyond chunk_lim belong to channels past the last one (partial last chunk); as
+    // unsigned, the padding mark -1 is beyond it too
+    auto chunk_lim = [&](int ch) {
+        const int cleft = s.C - ch * CC;
+        return (unsigned)((cleft < CC ? cleft : CC) * schan);
+    };
     cm_v4f rw[NW];
     float rx[NX];
     auto load_chunk = [&](int ch) {
@@ -103,33 +109,25 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
             rw[i] = wsrc[f4 < WCH / 4 ? f4 : 0];
         }
         const float* xsrc = x + (long)ch * CC * schan;
-        // offsets at or beyond lim belong to channels past the last one (partial last chunk); as
-        // unsigned, the padding mark -1 is beyond it too
-        const int cleft = s.C - ch * CC;
-        const unsigned lim = (unsigned)((cleft < CC ? cleft : CC) * schan);
+        const unsigned lim = chunk_lim(ch);
 #pragma unroll
         for (int i = 0; i < NX; i++)
-        {
-            // always load from a valid address (the element itself, or element 0 of a valid channel) and
-            // select afterwards: no branch around the load
-            const bool ok = (unsigned)goff[i] < lim;
-            const float v = xsrc[ok ? goff[i] : 0];
-            rx[i] = ok ? v : 0.f;
-        }
+            // always load from a valid address (the element itself, or element 0 of a valid channel); the
+            // value is replaced by zero only when it is stored, so that nothing waits for the load here
+            rx[i] = xsrc[(unsigned)goff[i] < lim ? goff[i] : 0];
     };
-    auto store_chunk = [&](int buf) {
+    auto store_chunk = [&](int buf, int ch) {
         cm_v4f* wdst = (cm_v4f*)(sW + buf * WCH);
 #pragma unroll
         for (int i = 0; i < NW; i++) {
             const int f4 = tid + i * CM_THREADS;
             if (f4 < WCH / 4) wdst[f4] = rw[i];
         }
-        float* xdst = sX + buf * XCH;
+        float* xdst = sX + buf * XCHP + tid;
+        const unsigned lim = chunk_lim(ch);
 #pragma unroll
-        for (int i = 0; i < NX; i++) {
-            const int el = tid + i * CM_THREADS;
-            if (el < XCH) xdst[el] = rx[i];
-        }
+        for (int i = 0; i < NX; i++)
+            if (i * CM_THREADS < XCHP) xdst[i * CM_THREADS] = (unsigned)goff[i] < lim ? rx[i] : 0.f;
     };
 
     const int ft = wave % FW, mt0 = (wave / FW) * NMT;
@@ -144,13 +142,13 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     const int ch0 = blockIdx.z * s.chunks_per;
     const int ch1 = ch0 + s.chunks_per < s.nchunks ? ch0 + s.chunks_per : s.nchunks;
     load_chunk(ch0);
-    store_chunk(0);
+    store_chunk(0, ch0);
     cm_lds_barrier();
     for (int ch = ch0; ch < ch1; ch++) {
         const int buf = (ch - ch0) & 1;
         if (ch + 1 < ch1) load_chunk(ch + 1);
         const float* w = sW + buf * WCH + wbase;
-        const float* xs = sX + buf * XCH + xbase;
+        const float* xs = sX + buf * XCHP + xbase;
 #pragma unroll
         for (int cp = 0; cp < NCP; cp++)
 #pragma unroll
@@ -166,7 +164,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
                         for (int j = 0; j < NMT; j++)
                             acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, xs[j * 32 + xoff], acc[j], 0, 0, 0);
                     }
-        if (ch + 1 < ch1) store_chunk(buf ^ 1);
+        if (ch + 1 < ch1) store_chunk(buf ^ 1, ch + 1);
         cm_lds_barrier();
     }
 
@@ -264,20 +262,19 @@ float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transpos
     return d;
 }
 
-template <int KD, int KS, int MT, int FT>
-static int launch(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
+template <int KD, int KS, int MT, int FT, int NX>
+static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {
     constexpr int T = KD * KS * KS;
     constexpr int CC = cm_cc(T);
     s.tiles = (int)cdiv(s.plane, MT);
     s.R = MT + (KS == 3 ? 2 * s.P + 2 : 0);
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
-    if ((long)CC * KD * s.R > (long)CM_THREADS * cm_nx(T)) return -1;     // run too long to stage
-    const size_t shmem = (size_t)2 * (CC * T * FT + CC * KD * s.R) * sizeof(float);
+    const size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, CM_THREADS) * CM_THREADS) * sizeof(float);
     if (shmem > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
-        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         attr = shmem;
     }
     // A launch that leaves most CUs idle (deep, small images) is split over the input channels: each
@@ -307,7 +304,7 @@ static int launch(const float* x, const float* wp, float* y, ConvMShape s, const
         s.part = scratch;
     }
     dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);
-    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
     HIP_OK(hipGetLastError());
     if (s.ksplit > 1) {
         hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)cdiv(s.osize, 256)), dim3(256), 0, st, s.part, y, s.osize,
@@ -315,6 +312,14 @@ static int launch(const float* x, const float* wp, float* y, ConvMShape s, const
         HIP_OK(hipGetLastError());
     }
     return 0;
+}
+
+template <int KD, int KS, int MT, int FT>
+static int launch(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
+{
+    const long R = MT + (KS == 3 ? 2 * s.P + 2 : 0), xch = (long)cm_cc(KD * KS * KS) * KD * R;
+    if (xch > (long)CM_THREADS * CM_NXMAX) return -1;     // run too long to stage
+    return xch <= CM_THREADS * 8 ? launch_nx<KD, KS, MT, FT, 8>(x, wp, y, s, e, st) : launch_nx<KD, KS, MT, FT, 16>(x, wp, y, s, e, st);
 }
 
 // Positions per workgroup: the largest tile that still gives every CU about two workgroups; small images
