@@ -25,7 +25,8 @@ class Stencil(C.Structure):
                 ("nrefs", C.c_int), ("refs", Ref * MAX_REFS), ("nscal", C.c_int), ("scal", Ref * MAX_SCAL),
                 ("nins", C.c_int), ("ins", Ins * MAX_INS), ("nconst", C.c_int), ("consts", C.c_float * MAX_CONST),
                 ("count", C.c_long), ("nk", C.c_int), ("klo", C.c_int), ("nargs", C.c_int), ("ilo", C.c_int),
-                ("jlo", C.c_int), ("ni", C.c_int), ("nj", C.c_int), ("sx", C.c_int), ("cells", C.POINTER(C.c_int))]
+                ("jlo", C.c_int), ("ni", C.c_int), ("nj", C.c_int), ("sx", C.c_int), ("cells", C.POINTER(C.c_int)),
+                ("elt", C.c_int * MAX_ARRAYS), ("cdouble", C.c_int * MAX_CONST), ("dconsts", C.c_double * MAX_CONST)]
 
 
 class HostFacts(C.Structure):
@@ -79,6 +80,7 @@ PROTOTYPES = {
     "fortis_model_input": (vp, []), "fortis_model_output": (vp, []), "fortis_begin": (None, [i]),
     # stencil
     "fortis_stencil_check": (i, [C.POINTER(Stencil)]),
+    "fortis_stencil_route": (i, [C.POINTER(Stencil)]),
     "fortis_gather_config": (i, [C.POINTER(Stencil)]), "fortis_scatter_config": (i, [C.POINTER(Stencil)]),
     "fortis_gather_v": (None, [C.POINTER(i), C.POINTER(vp)]), "fortis_scatter_v": (None, [C.POINTER(i), C.POINTER(vp)]),
     "fortis_gather": (None, [vp, vp, vp, vp]), "fortis_scatter": (None, [i, vp, vp, vp, vp, vp]),

@@ -71,6 +71,12 @@ struct StencilDev {
 // Splits the straight-line program into per-cell code and a tv chain.  Returns -1 if tv is used
 // in a way that is not a single chain.
 int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out);
+// General kernels for everything else (stencil_generic.hip): fp64 arrays, double literals, the lifter's
+// functions, expressions that are not one chain.  dA: device array bases in descriptor order.
+int fortis_stencil_validate(const fortis_stencil_t* t);
+bool fortis_stencil_typed(const fortis_stencil_t* t);
+void fortis_launch_gather_generic(const fortis_stencil_t& t, const int* dcells, const void* const* dA, float* dX, hipStream_t s);
+void fortis_launch_scatter_generic(const fortis_stencil_t& t, const int* dcells, void* const* dA, const float* dY, int kk, hipStream_t s);
 
 // ---- elementwise / layout kernels (elementwise.hip) --------------------------------------
 void fortis_launch_scale(const float* src, float* dst, const float* vec, long rows, long n, int divide, hipStream_t s);

@@ -81,6 +81,8 @@ __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, c
 }
 
 // ---- lowering: straight-line program -> per-cell code + tv chain -----------------------------
+static bool g_lower_quiet = false;     // set while a table is only being tried for the fused kernels
+#define LOWER_ERR(...) do { if (!g_lower_quiet) fprintf(stderr, __VA_ARGS__); } while (0)
 int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
 {
     memset(out, 0, sizeof *out);
@@ -88,7 +90,7 @@ int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
         in->nscal < 0 || in->nscal > ST_SCAL_MAX || in->nins < 0 || in->nins > FORTIS_MAX_INS ||
         in->nconst < 0 || in->nconst > FORTIS_MAX_CONST || in->count < 1 || in->nk < 1 ||
         in->count * in->nk >= 4294967295L / FORTIS_MAX_REFS) {
-        fprintf(stderr, "fortis: stencil table out of range\n");
+        LOWER_ERR("fortis: stencil table out of range\n");
         return -1;
     }
     out->narrays = in->narrays;
@@ -99,8 +101,8 @@ int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
     for (int r = 0; r < in->nscal; r++) out->scal[r] = in->scal[r];
     for (int r = 0; r < in->nrefs + in->nscal; r++) {
         const fortis_ref_t& f = r < in->nrefs ? in->refs[r] : in->scal[r - in->nrefs];
-        if (f.array < 0 || f.array >= in->narrays) { fprintf(stderr, "fortis: stencil ref names array %d\n", f.array); return -1; }
-        if (f.si > 2147483647L || f.sj > 2147483647L || f.si < -2147483647L || f.sj < -2147483647L) { fprintf(stderr, "fortis: stencil stride out of range\n"); return -1; }
+        if (f.array < 0 || f.array >= in->narrays) { LOWER_ERR("fortis: stencil ref names array %d\n", f.array); return -1; }
+        if (f.si > 2147483647L || f.sj > 2147483647L || f.si < -2147483647L || f.sj < -2147483647L) { LOWER_ERR("fortis: stencil stride out of range\n"); return -1; }
     }
     for (int c = 0; c < in->nconst; c++) out->consts[c] = in->consts[c];
     out->count = in->count; out->nk = in->nk;
@@ -114,35 +116,48 @@ int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
         for (int s = 0; s < 2; s++) {
             const int c = codes[s];
             bool ok = c == 0 || (c >= 1 && c <= in->nscal) || (c >= 16 && c < 16 + in->nconst) || (c >= 32 && c < 32 + n);
-            if (!ok || I.op < 0 || I.op > 3) { fprintf(stderr, "fortis: bad stencil instruction %d\n", n); return -1; }
-            if (c == 0) { isdep[s] = 1; lowered[s] = 0; if (last_dep >= 0) { fprintf(stderr, "fortis: stencil expression re-reads the slot value after transforming it\n"); return -1; } }
-            else if (c >= 32 && dep[c - 32]) { isdep[s] = 1; lowered[s] = 0; if (c - 32 != last_dep) { fprintf(stderr, "fortis: stencil expression is not a single chain on the slot value\n"); return -1; } }
+            if (!ok || I.op < 0 || I.op > 3) { LOWER_ERR("fortis: bad stencil instruction %d\n", n); return -1; }
+            if (c == 0) { isdep[s] = 1; lowered[s] = 0; if (last_dep >= 0) { LOWER_ERR("fortis: stencil expression re-reads the slot value after transforming it\n"); return -1; } }
+            else if (c >= 32 && dep[c - 32]) { isdep[s] = 1; lowered[s] = 0; if (c - 32 != last_dep) { LOWER_ERR("fortis: stencil expression is not a single chain on the slot value\n"); return -1; } }
             else { isdep[s] = 0; lowered[s] = c >= 32 ? 32 + map[c - 32] : c; }
         }
-        if (isdep[0] && isdep[1]) { fprintf(stderr, "fortis: stencil expression combines the slot value with itself\n"); return -1; }
+        if (isdep[0] && isdep[1]) { LOWER_ERR("fortis: stencil expression combines the slot value with itself\n"); return -1; }
         if (isdep[0] || isdep[1]) {
             dep[n] = 1; map[n] = -1; last_dep = n;
             CellStep st = { I.op, isdep[0] ? lowered[1] : lowered[0], isdep[0] ? 1 : 0 };
-            if (out->nchain == ST_CHAIN_MAX) { fprintf(stderr, "fortis: stencil expression chains more than %d operations on the slot value\n", ST_CHAIN_MAX); return -1; }
+            if (out->nchain == ST_CHAIN_MAX) { LOWER_ERR("fortis: stencil expression chains more than %d operations on the slot value\n", ST_CHAIN_MAX); return -1; }
             out->chain[out->nchain++] = st;
         } else {
             dep[n] = 0; map[n] = out->ncell;
-            if (out->ncell == ST_CELL_MAX) { fprintf(stderr, "fortis: more than %d per-cell stencil instructions\n", ST_CELL_MAX); return -1; }
+            if (out->ncell == ST_CELL_MAX) { LOWER_ERR("fortis: more than %d per-cell stencil instructions\n", ST_CELL_MAX); return -1; }
             fortis_ins_t ci = { I.op, lowered[0], lowered[1] };
             out->cell[out->ncell++] = ci;
         }
     }
     if (in->nins > 0 && last_dep != in->nins - 1 && last_dep >= 0) {
-        fprintf(stderr, "fortis: the last stencil instruction must produce the slot value\n");
+        LOWER_ERR("fortis: the last stencil instruction must produce the slot value\n");
         return -1;
     }
-    if (in->nins > 0 && last_dep < 0) { fprintf(stderr, "fortis: stencil expressions never use the slot value\n"); return -1; }
+    if (in->nins > 0 && last_dep < 0) { LOWER_ERR("fortis: stencil expressions never use the slot value\n"); return -1; }
     return 0;
 }
 
 // ---- device copies of tables -----------------------------------------------------------------
+// 0: the table runs in the fused-form kernels (lowered into *low), 1: it takes the general kernels, -1: invalid.
+static int route_table(const fortis_stencil_t* t, StencilDev* low)
+{
+    if (fortis_stencil_validate(t) != 0) return -1;
+    if (fortis_stencil_typed(t)) return 1;
+    g_lower_quiet = true;
+    const int rc = fortis_stencil_lower(t, low);
+    g_lower_quiet = false;
+    return rc == 0 ? 0 : 1;
+}
+static inline size_t esz_of(const fortis_stencil_t& t, int a) { return t.elt[a] == 8 ? 8 : 4; }
+
 struct BoundStencil {
     bool ok = false;
+    bool generic = false;        // the table takes the general kernels
     fortis_stencil_t host;       // as configured (cells pointer not owned)
     StencilDev low;              // lowered table
     int* dcells = nullptr;       // device copy of the cell list
@@ -159,15 +174,17 @@ struct BoundStencil {
 };
 static BoundStencil g_gather, g_scatter;
 
+// Returns the table's route (see route_table) after copying its cell list to the device.
 static int upload_table(const fortis_stencil_t* t, StencilDev* low, int** dcells)
 {
-    if (fortis_stencil_lower(t, low) != 0) return -1;
+    const int route = route_table(t, low);
+    if (route < 0) return -1;
     if (t->cells) {
         HIP_OK(hipMalloc((void**)dcells, t->count * sizeof(int)));
         HIP_OK(hipMemcpy(*dcells, t->cells, t->count * sizeof(int), hipMemcpyHostToDevice));
-        low->cells = *dcells;
+        if (route == 0) low->cells = *dcells;
     }
-    return 0;
+    return route;
 }
 
 static void release(BoundStencil& b)
@@ -182,11 +199,13 @@ static void release(BoundStencil& b)
 static int config(BoundStencil& b, const fortis_stencil_t* t, bool is_scatter)
 {
     release(b);
-    if (upload_table(t, &b.low, &b.dcells) != 0) return -1;
+    const int route = upload_table(t, &b.low, &b.dcells);
+    if (route < 0) return -1;
+    b.generic = route == 1;
     b.host = *t;
     b.host.cells = nullptr;
-    if (is_scatter) {
-        for (int r = 0; r < t->nrefs; r++) b.written[t->refs[r].array] = true;
+    if (is_scatter) for (int r = 0; r < t->nrefs; r++) b.written[t->refs[r].array] = true;
+    if (is_scatter && !b.generic) {
         fortis_stencil_t all = *t;
         for (int r = 0; r < all.nrefs; r++)
             if (!all.refs[r].planar) { all.refs[r].planar = 1; all.plane[all.refs[r].array] = all.total[all.refs[r].array]; }
@@ -204,7 +223,7 @@ void fortis_stencil_reset_internal()
 }
 
 // cache of device tables for the device-resident API (keyed by table contents)
-struct CacheEnt { fortis_stencil_t key; const int* cells_key; int* dcells; StencilDev low; };
+struct CacheEnt { fortis_stencil_t key; const int* cells_key; int* dcells; StencilDev low; bool generic; };
 static CacheEnt g_cache[16];
 static int g_ncache = 0;
 static CacheEnt* cached(const fortis_stencil_t* t)
@@ -214,13 +233,26 @@ static CacheEnt* cached(const fortis_stencil_t* t)
         a.cells = b.cells = nullptr;
         if (!memcmp(&a, &b, sizeof a) && g_cache[i].cells_key == t->cells) return &g_cache[i];
     }
-    if (g_ncache == 16) { fprintf(stderr, "fortis: stencil table cache full\n"); return nullptr; }
-    CacheEnt* e = &g_cache[g_ncache];
+    CacheEnt* e;
+    const bool evict = g_ncache == 16;
+    if (evict) {
+        // full: the oldest entry is replaced in place (once nothing in flight can still read its cell list)
+        static int victim = 0;
+        e = &g_cache[victim];
+        victim = (victim + 1) % 16;
+        HIP_OK(hipStreamSynchronize(fortis_stream_get()));
+        if (e->dcells) HIP_OK(hipFree(e->dcells));
+        e->key.narrays = -1;            // matches no table until it is filled again
+    } else {
+        e = &g_cache[g_ncache];
+    }
     e->dcells = nullptr;
-    if (upload_table(t, &e->low, &e->dcells) != 0) return nullptr;
+    const int route = upload_table(t, &e->low, &e->dcells);
+    if (route < 0) return nullptr;
+    e->generic = route == 1;
     e->key = *t;
     e->cells_key = t->cells;
-    g_ncache++;
+    if (!evict) g_ncache++;
     return e;
 }
 
@@ -252,7 +284,13 @@ extern "C" {
 int fortis_stencil_check(const fortis_stencil_t* t)
 {
     StencilDev tmp;
-    return t ? fortis_stencil_lower(t, &tmp) : -1;
+    return t && route_table(t, &tmp) >= 0 ? 0 : -1;
+}
+// Test hook: 0 if the table runs in the fused-form kernels, 1 if it takes the general ones, -1 if invalid.
+int fortis_stencil_route(const fortis_stencil_t* t)
+{
+    StencilDev tmp;
+    return t ? route_table(t, &tmp) : -1;
 }
 int fortis_gather_config(const fortis_stencil_t* g) { return config(g_gather, g, false); }
 int fortis_scatter_config(const fortis_stencil_t* s) { return config(g_scatter, s, true); }
@@ -275,7 +313,7 @@ void fortis_gather_v(const int* a, const void* const* H)
     const bool kdist = t.nk > 1;
     if (!b.init) {
         for (int ai = 0; ai < t.narrays; ai++)
-            HIP_OK(hipMalloc(&b.darr[ai], (size_t)t.plane[ai] * t.nk * sizeof(float)));   // gather.cu:8-11
+            HIP_OK(hipMalloc(&b.darr[ai], (size_t)t.plane[ai] * t.nk * esz_of(t, ai)));   // gather.cu:8-11
         b.init = true;
     }
     const float* dptr[FORTIS_MAX_ARRAYS];
@@ -287,10 +325,14 @@ void fortis_gather_v(const int* a, const void* const* H)
         const bool planar3d = t.total[ai] > t.plane[ai];
         if (planar3d) off = kdist ? (long)(t.klo - 1) * t.plane[ai] : (long)((a ? a[0] : 1) - 1) * t.plane[ai];
         const long nelem = (kdist && planar3d) ? t.plane[ai] * t.nk : t.plane[ai];
-        HIP_OK(hipMemcpyAsync(b.darr[ai], (const float*)H[ai] + off, nelem * sizeof(float), hipMemcpyHostToDevice, s));
+        HIP_OK(hipMemcpyAsync(b.darr[ai], (const char*)H[ai] + off * esz_of(t, ai), nelem * esz_of(t, ai), hipMemcpyHostToDevice, s));
         dptr[ai] = (const float*)b.darr[ai];
     }
-    launch_gather(b.low, dptr, (float*)fortis_model_input(), s);
+    if (b.generic) {
+        fortis_launch_gather_generic(t, b.dcells, (const void* const*)dptr, (float*)fortis_model_input(), s);
+    } else {
+        launch_gather(b.low, dptr, (float*)fortis_model_input(), s);
+    }
 }
 
 void fortis_scatter_v(const int* a, void* const* H)
@@ -305,7 +347,7 @@ void fortis_scatter_v(const int* a, void* const* H)
     // per call (gather.cu:84-90); as copy commands from and to pageable memory those cost far more than the
     // kernel here (a pitched download is handled row by row).
     if (!b.init) {
-        for (int ai = 0; ai < t.narrays; ai++) HIP_OK(hipHostMalloc(&b.darr[ai], (size_t)t.plane[ai] * sizeof(float), hipHostMallocDefault));
+        for (int ai = 0; ai < t.narrays; ai++) HIP_OK(hipHostMalloc(&b.darr[ai], (size_t)t.plane[ai] * esz_of(t, ai), hipHostMallocDefault));
         b.host_planes = true;
         b.init = true;
     }
@@ -322,7 +364,7 @@ void fortis_scatter_v(const int* a, void* const* H)
     // compares its iteration's scalar planes with what was read then and, if they are the same bytes (the
     // normal case: they were inputs of the gather too), only copies its rows out -- no launch and no
     // synchronisation.  Any difference, or a new forward pass in between, takes the one-iteration path below.
-    if (t.nk > 1 && rects && !getenv("FORTIS_SCATTER_PER_CALL")) {
+    if (t.nk > 1 && rects && !b.generic && !getenv("FORTIS_SCATTER_PER_CALL")) {
         const int idx = k1 - t.klo;
         const long gen = fortis_step_generation();
         auto planes = [&](int ai) { return (t.total[ai] > t.plane[ai] || b.written[ai]) ? (long)t.nk : 1L; };
@@ -372,27 +414,29 @@ void fortis_scatter_v(const int* a, void* const* H)
         // inputs always; a written array only when its whole plane goes back (unvisited cells must survive)
         if (!b.written[ai] || whole_plane[ai]) {
             const long off = t.total[ai] > t.plane[ai] ? (long)(k1 - 1) * t.plane[ai] : 0;
-            memcpy(b.darr[ai], (const float*)H[ai] + off, t.plane[ai] * sizeof(float));
+            memcpy(b.darr[ai], (const char*)H[ai] + off * esz_of(t, ai), t.plane[ai] * esz_of(t, ai));
         }
     }
     // the staging holds ONE plane per array, so the kernel runs with plane index 0
     const long yoff = t.nk > 1 ? (long)(k1 - t.klo) * t.count * t.nrefs : 0;   // gather.cu:86
-    launch_scatter(b.low, dptr, (const float*)fortis_model_output() + yoff, 0, s);
+    if (b.generic) fortis_launch_scatter_generic(t, b.dcells, (void* const*)dptr, (const float*)fortis_model_output() + yoff, 0, s);
+    else launch_scatter(b.low, dptr, (const float*)fortis_model_output() + yoff, 0, s);
     HIP_OK(hipStreamSynchronize(s));
     for (int r = 0; r < t.nrefs; r++) {
         const int ai = t.refs[r].array;
+        const size_t es = esz_of(t, ai);
         const long off = t.total[ai] > t.plane[ai] ? (long)(k1 - 1) * t.plane[ai] : 0;
-        float* hbase = (float*)H[ai] + off;
-        const float* stage = (const float*)b.darr[ai];
+        char* hbase = (char*)H[ai] + off * es;
+        const char* stage = (const char*)b.darr[ai];
         if (whole_plane[ai]) {
             // cell list or non-unit inner stride: no rectangle to copy, return the whole plane
-            memcpy(hbase, stage, t.plane[ai] * sizeof(float));
+            memcpy(hbase, stage, t.plane[ai] * es);
         } else {
             // visited rectangle, pitch = stride of the j index (gather.cu:87-89; gather_emit.py:88-95)
             const long rect = t.refs[r].base + (long)t.ilo * t.refs[r].si + (long)t.jlo * t.refs[r].sj;
             const long pitch = t.refs[r].sj > 0 ? t.refs[r].sj : t.ni;
             const long nrow = t.nj > 0 ? t.nj : t.count / t.ni;
-            for (long j = 0; j < nrow; j++) memcpy(hbase + rect + j * pitch, stage + rect + j * pitch, (size_t)t.ni * sizeof(float));
+            for (long j = 0; j < nrow; j++) memcpy(hbase + (rect + j * pitch) * es, stage + (rect + j * pitch) * es, (size_t)t.ni * es);
         }
     }
 }
@@ -412,12 +456,14 @@ void fortis_stencil_gather_dev(const fortis_stencil_t* g, const float* const* dA
 {
     CacheEnt* e = cached(g);
     if (!e) return;
+    if (e->generic) { fortis_launch_gather_generic(*g, e->dcells, (const void* const*)dA, dX, fortis_stream_get()); return; }
     launch_gather(e->low, dA, dX, fortis_stream_get());
 }
 void fortis_stencil_scatter_dev(const fortis_stencil_t* sd, float* const* dA, const float* dY, int kk)
 {
     CacheEnt* e = cached(sd);
     if (!e) return;
+    if (e->generic) { fortis_launch_scatter_generic(*sd, e->dcells, (void* const*)dA, dY, kk, fortis_stream_get()); return; }
     launch_scatter(e->low, dA, dY, kk, fortis_stream_get());
 }
 
@@ -439,9 +485,15 @@ int fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t*
     fortis_stencil_t s2 = *sd;
     for (int r = 0; r < s2.nrefs; r++)
         if (!s2.refs[r].planar) { s2.refs[r].planar = 1; s2.plane[s2.refs[r].array] = s2.total[s2.refs[r].array]; }
-    CacheEnt* eg = cached(g);
     CacheEnt* es = cached(&s2);
+    CacheEnt* eg = cached(g);
+    if (eg && es && memcmp(&es->key, &s2, offsetof(fortis_stencil_t, cells)) != 0) es = cached(&s2);   // the second lookup replaced the first
     if (!eg || !es) return -1;
+    if (eg->generic || es->generic) {
+        fprintf(stderr, "fortis_stencil_step_fused: the tables need the general stencil kernels (fp64 arrays, functions or a "
+                        "non-chain expression); run gather, model and scatter as separate launches\n");
+        return -1;
+    }
     fortis_launch_chain_stencil(d, eg->low, es->low, g->count * g->nk, dG, dS, dY, fortis_stream_get());
     return 0;
 }

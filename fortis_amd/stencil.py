@@ -13,16 +13,40 @@ import numpy as np
 
 from ._lib import MAX_ARRAYS, MAX_CONST, MAX_INS, MAX_REFS, MAX_SCAL, Ins, Ref, Stencil
 
-_TOKEN = re.compile(r"\s*(tv|S\d+|(?:\d+\.\d*|\.\d+|\d+)(?:[eE][-+]?\d+)?f?|[()+\-*/])")
+_TOKEN = re.compile(r"\s*(tv|S\d+|sqrtf|expf|logf|tanhf|fmaxf|fminf|(?:\d+\.\d*|\.\d+|\d+)(?:[eE][-+]?\d+)?f?|[()+\-*/,])")
+_UNARY = {"sqrtf": 7, "expf": 8, "logf": 9, "tanhf": 10}
+_BINARY_FN = {"fmaxf": 4, "fminf": 5}
+INS_F64 = 0x100
+OP_NEG, OP_F32 = 6, 11
 
 
-def compile_exprs(exprs):
-    """C expression strings over `tv`, `S<n>` and float literals -> ([(op, a, b)], [consts]).
+def compile_exprs(exprs, scalar_f64=None):
+    """C expression strings as the reference's lifter writes them (driver/fortis_gather.py:89-121:
+    tv, S<n>, literals with or without an f suffix, + - * /, unary minus, sqrtf/expf/logf/tanhf,
+    fmaxf/fminf) -> ([(op, a, b)], [(value, is_double)]).
 
-    Operand codes: 0 tv, 1+n scalar S<n>, 16+n constant n, 32+n result n; op 0 add, 1 sub, 2 mul, 3 div.
-    Expressions apply in order, each replacing tv (driver/fortis_gather_emit.py:59-61, 79-80).
-    Evaluation order is the C parse: left-associative, * and / before + and -."""
-    ins, consts = [], []
+    Operand codes: 0 tv, 1+n scalar S<n>, 16+n constant n, 32+n result n.  Expressions apply in
+    order, each replacing tv (driver/fortis_gather_emit.py:59-61, 79-80).  Evaluation order is the
+    C parse: left-associative, * and / before + and -.  Types are C's: tv float, S<n> double where
+    scalar_f64[n], a literal double without its f suffix; an arithmetic result is double when an
+    operand is (INS_F64 in its op), the f-suffixed functions return float, and an expression of
+    type double ends in an explicit conversion, the assignment to the float tv."""
+    ins, consts, typ = [], [], {0: False}
+    for n in range(MAX_SCAL):     # without a scalar list every S<n> is taken as float
+        if scalar_f64 is None or n < len(scalar_f64):
+            typ[1 + n] = bool(scalar_f64[n]) if scalar_f64 is not None else False
+
+    def emit(op, a, b, f64):
+        ins.append((op | (INS_F64 if f64 else 0), a, b))
+        code = 32 + len(ins) - 1
+        typ[code] = f64
+        return code
+
+    def const(value, f64):
+        consts.append((float(value) if f64 else float(np.float32(value)), f64))
+        code = 16 + len(consts) - 1
+        typ[code] = f64
+        return code
 
     def parse_one(text, tvcode):
         toks = _TOKEN.findall(text)
@@ -35,49 +59,83 @@ def compile_exprs(exprs):
 
         def take():
             nonlocal pos
+            if pos >= len(toks):
+                raise ValueError(f"unexpected end of {text!r}")
             pos += 1
             return toks[pos - 1]
+
+        def expect(t):
+            if take() != t:
+                raise ValueError(f"expected {t!r} in {text!r}")
 
         def atom():
             t = take()
             if t == "(":
                 v = additive()
-                if take() != ")":
-                    raise ValueError(f"unbalanced parentheses in {text!r}")
+                expect(")")
                 return v
             if t == "tv":
                 return tvcode
+            if t in _UNARY:
+                expect("(")
+                v = additive()
+                expect(")")
+                return emit(_UNARY[t], v, v, False)
+            if t in _BINARY_FN:
+                expect("(")
+                v = additive()
+                expect(",")
+                w = additive()
+                expect(")")
+                return emit(_BINARY_FN[t], v, w, False)
             if t[0] == "S":
-                return 1 + int(t[1:])
-            if t in "+-*/)":
+                n = int(t[1:])
+                if 1 + n not in typ:
+                    raise ValueError(f"{t} is not a scalar of this descriptor ({text!r})")
+                return 1 + n
+            if t in "+-*/),":
                 raise ValueError(f"unexpected {t!r} in {text!r}")
-            consts.append(float(np.float32(float(t.rstrip("f")))))
-            return 16 + len(consts) - 1
+            return const(float(t.rstrip("f")), not t.endswith("f"))
+
+        def unary():
+            if peek() == "-":
+                take()
+                if peek() not in (None, "tv", "(", "-") and peek()[0] not in "Ssetf":
+                    t = take()       # a negated literal is the literal of the opposite sign, exactly
+                    return const(-float(t.rstrip("f")), not t.endswith("f"))
+                v = unary()
+                return emit(OP_NEG, v, v, typ[v])
+            return atom()
 
         def multiplicative():
-            v = atom()
+            v = unary()
             while peek() in ("*", "/"):
                 op = 2 if take() == "*" else 3
-                ins.append((op, v, atom()))
-                v = 32 + len(ins) - 1
+                w = unary()
+                v = emit(op, v, w, typ[v] or typ[w])
             return v
 
         def additive():
             v = multiplicative()
             while peek() in ("+", "-"):
                 op = 0 if take() == "+" else 1
-                ins.append((op, v, multiplicative()))
-                v = 32 + len(ins) - 1
+                w = multiplicative()
+                v = emit(op, v, w, typ[v] or typ[w])
             return v
 
         v = additive()
         if pos != len(toks):
             raise ValueError(f"trailing tokens in {text!r}")
+        if typ[v]:
+            v = emit(OP_F32, v, v, False)     # tv = <double expression>;
         return v
 
     cur = 0
     for e in exprs:
         cur = parse_one(e, cur)
+    if cur != 0 and cur < 32:
+        # an expression that is a bare operand ("S0"): materialise the assignment
+        cur = emit(OP_F32, cur, cur, False)
     if len(ins) > MAX_INS or len(consts) > MAX_CONST:
         raise ValueError("lifted expressions too long for the stencil table")
     return ins, consts
@@ -113,8 +171,8 @@ def build_table(desc, loop, kdist=None, role="gather", cells=None, sx=None):
     if not desc.get("ok", True):
         raise ValueError("descriptor says the lift was rejected")
     for a in desc["arrays"]:
-        if a["elt"] != "f32":
-            raise NotImplementedError("stencil arrays must be f32 (f64 host arrays are not lifted yet)")
+        if a["elt"] not in ("f32", "f64"):     # driver/fortis_gather_emit.py:13
+            raise ValueError(f"stencil array element type {a['elt']!r} is neither f32 nor f64")
     if len(desc["arrays"]) > MAX_ARRAYS:
         raise ValueError("too many arrays")
     t = Stencil()
@@ -134,6 +192,7 @@ def build_table(desc, loop, kdist=None, role="gather", cells=None, sx=None):
         nv = sum(1 for kind, _ in e["idx"] if kind == "v") if e else 0
         plane = int(np.prod(a["shape"][:len(a["shape"]) - nv]))
         t.total[ai], t.plane[ai] = total, plane
+        t.elt[ai] = 8 if a["elt"] == "f64" else 4
     t.nrefs = len(entries)
     for n, e in enumerate(entries):
         t.refs[n] = _ref(desc["arrays"], e)
@@ -142,13 +201,15 @@ def build_table(desc, loop, kdist=None, role="gather", cells=None, sx=None):
         if s["name"] != f"S{n}":
             raise ValueError("scalars must be named S0, S1, ... in order")
         t.scal[n] = _ref(desc["arrays"], s)
-    ins, consts = compile_exprs(desc["exprs"])
+    ins, consts = compile_exprs(desc["exprs"], [desc["arrays"][s["array"]]["elt"] == "f64" for s in desc["scalars"]])
     t.nins = len(ins)
     for n, (op, a, b) in enumerate(ins):
         t.ins[n] = Ins(op, a, b)
     t.nconst = len(consts)
-    for n, c in enumerate(consts):
+    for n, (c, f64) in enumerate(consts):
         t.consts[n] = c
+        t.cdouble[n] = 1 if f64 else 0
+        t.dconsts[n] = c
     # under loop distribution the gather loses its int args, the scatter keeps them (gather_emit.py:62, 84)
     t.nargs = 0 if (role == "gather" and nk > 1) else len(desc.get("args", []))
     t.nk, t.klo = nk, klo

@@ -146,12 +146,24 @@ void  fortis_begin(int count);
  * prints into the generated kernel. */
 typedef struct { int array; int planar; long base, si, sj; } fortis_ref_t;
 
-/* Lifted expressions as straight-line fp32 code: r[n] = operand(a) op operand(b).
- * operand: 0 = tv (the slot value), 1..8 = scalar S0..S7, 16+n = consts[n], 32+n = r[n].
- * op: 0 add, 1 sub, 2 mul, 3 div.  The last result replaces tv.  Each op is one IEEE fp32
- * operation, never fused (the reference compiles gather.cu with -fmad=false).  tv may enter
- * an instruction only as the running value of one chain (tv op c, c op tv). */
+/* Lifted expressions as straight-line code: r[n] = operand(a) op operand(b).
+ * operand: 0 = tv (the slot value), 1..8 = scalar S0..S7, 16+n = constant n, 32+n = r[n].
+ * op (low byte): 0 add, 1 sub, 2 mul, 3 div, 4 fmaxf, 5 fminf, and on operand a alone 6 negate,
+ * 7 sqrtf, 8 expf, 9 logf, 10 tanhf (the operator set of the reference's lifter,
+ * driver/fortis_gather.py:89-121) and 11 conversion to float.  The last result replaces tv.  Each op is one IEEE operation,
+ * never fused (the reference compiles gather.cu with -fmad=false).
+ * Types follow the C the reference's generator prints (driver/fortis_gather_emit.py:57-61, 76-81):
+ * tv is float, a scalar has its array's element type, a literal is float with an f suffix and
+ * double without; + - * / and negate have a double result when an operand is double, which the
+ * table builder marks with FORTIS_INS_F64 in op; the assignment back to tv at the end of an
+ * expression is an explicit conversion (op 11) where the expression's type is double; the
+ * f-suffixed functions convert their operands to float first.
+ * Tables whose expressions are one chain of + - * / on the slot value over fp32 arrays (tv op c,
+ * c op tv) run in the fused kernels; anything else takes the general kernels. */
 typedef struct { int op, a, b; } fortis_ins_t;
+#define FORTIS_INS_F64 0x100
+enum { FORTIS_OP_ADD = 0, FORTIS_OP_SUB, FORTIS_OP_MUL, FORTIS_OP_DIV, FORTIS_OP_MAX, FORTIS_OP_MIN,
+       FORTIS_OP_NEG, FORTIS_OP_SQRT, FORTIS_OP_EXP, FORTIS_OP_LOG, FORTIS_OP_TANH, FORTIS_OP_F32 };
 
 #define FORTIS_MAX_ARRAYS 8
 #define FORTIS_MAX_REFS 32
@@ -178,6 +190,10 @@ typedef struct {
     int  sx;                           /* leading dimension of the cell plane, for the cell list */
     const int* cells;                  /* optional host list of `count` 0-based cell indices (i-1)+(j-1)*sx;
                                           NULL = the rectangle.  Copied at config. */
+    int  elt[FORTIS_MAX_ARRAYS];       /* bytes per element of each host array: 4 (or 0) fp32, 8 fp64
+                                          (the descriptor's "elt", driver/fortis_gather_emit.py:13) */
+    int  cdouble[FORTIS_MAX_CONST];    /* constant n is a C double literal: its value is dconsts[n], not consts[n] */
+    double dconsts[FORTIS_MAX_CONST];
 } fortis_stencil_t;
 
 /* Validates a table without touching the GPU (ranges, and that the expressions form one chain on
@@ -199,6 +215,7 @@ void fortis_scatter(int a0, float* H0, float* H1, float* H2, float* H3, float* H
 
 /* Device-resident forms (arrays already in HBM; nothing is copied).  dA: device pointers in
  * descriptor order.  Asynchronous on the persistent stream. */
+/* (With fp64 arrays in the table the matching entries of dA point to doubles.) */
 void fortis_stencil_gather_dev(const fortis_stencil_t* g, const float* const* dA, float* dX);
 void fortis_stencil_scatter_dev(const fortis_stencil_t* s, float* const* dA, const float* dY, int kk);
 /* The whole lifted step in ONE kernel: gather (g) -> MLP chain (plan p, every op a linear or a
@@ -231,8 +248,11 @@ const char* fortis_plan_kernel_name(fortis_plan* p, int idx);
  * fortis_gemm_schedule: the persistent GEMM's work list for C[B][N] on `slots` resident workgroups, as
  *   (level, first 128 x 128 tile, items) triples, level 0 whole tiles, 1 halves (128 x 64), 2 quarters
  *   (64 x 64); returns the number of phases (at most 4), -1 on bad arguments.
- * fortis_magic_divmod: n / d and n % d by the exact multiply-shift the stencil kernels decode cells with. */
+ * fortis_magic_divmod: n / d and n % d by the exact multiply-shift the stencil kernels decode cells with.
+ * fortis_stencil_route: which kernels a stencil table takes: 0 the fused-form ones (fp32 arrays, one chain
+ *   of + - * / on the slot value), 1 the general ones, -1 the table is invalid. */
 int  fortis_gemm_schedule(long B, long N, long slots, long* triples);
+int  fortis_stencil_route(const fortis_stencil_t* t);
 void fortis_magic_divmod(unsigned n, unsigned d, unsigned* q, unsigned* r);
 
 #ifdef __cplusplus
