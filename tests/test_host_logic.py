@@ -134,11 +134,11 @@ def test_batch_already_multiplied_by_nk_is_accepted(golden):
 def test_expression_compiler():
     assert S.compile_exprs(["(((tv * S0) * S0) * S1)"])[0] == [(2, 0, 1), (2, 32, 1), (2, 33, 2)]
     ins, consts = S.compile_exprs(["(tv / (S0 + 1.000000e-30f))"])
-    assert ins == [(0, 1, 16), (3, 0, 32)] and consts == [float(np.float32(1e-30))]
+    assert ins == [(0, 1, 16), (3, 0, 32)] and consts == [(float(np.float32(1e-30)), False)]
     ins, _ = S.compile_exprs(["(tv * S0)", "(tv - 2.0f)"])   # two expressions in order, each replacing tv
     assert ins == [(2, 0, 1), (1, 32, 16)]
     with pytest.raises(ValueError):
-        S.compile_exprs(["sqrtf(tv)"])
+        S.compile_exprs(["cbrtf(tv)"])
 
 
 def _table_with(ins, nscal=2, nconst=1):
@@ -151,17 +151,29 @@ def _table_with(ins, nscal=2, nconst=1):
     return t
 
 
-def test_lowering_accepts_chains_and_rejects_the_rest(L, capfd):
-    ok = [[(0, 1, 16), (3, 0, 32)], [(2, 0, 1), (2, 32, 1), (2, 33, 2)], [(1, 16, 0)], []]
-    for ins in ok:
+def test_table_routing_chains_general_forms_and_invalid_tables(L, capfd):
+    """One chain of + - * / on the slot value runs in the fused-form kernels (route 0); other valid
+    programs take the general kernels (route 1); malformed tables are refused (route -1)."""
+    chains = [[(0, 1, 16), (3, 0, 32)], [(2, 0, 1), (2, 32, 1), (2, 33, 2)], [(1, 16, 0)], []]
+    for ins in chains:
+        assert L.fortis_stencil_route(C.byref(_table_with(ins))) == 0
         assert L.fortis_stencil_check(C.byref(_table_with(ins))) == 0
-    bad = [[(2, 0, 0)],                      # tv * tv
-           [(2, 0, 1), (0, 32, 0)],          # re-reads tv after transforming it
-           [(2, 0, 1), (0, 1, 2)],           # last instruction does not produce the slot value
-           [(0, 1, 2)],                      # never uses tv
-           [(7, 0, 1)],                      # unknown op
-           [(0, 0, 5)]]                      # scalar out of range
+    general = [[(2, 0, 0)],                  # tv * tv
+               [(2, 0, 1), (0, 32, 0)],      # re-reads tv after transforming it
+               [(2, 0, 1), (0, 1, 2)],       # last instruction does not involve the slot value
+               [(0, 1, 2)],                  # never uses tv
+               [(7, 0, 0)],                  # sqrtf
+               [(2 | 0x100, 0, 1), (11, 32, 32)]]   # double product, converted back
+    for ins in general:
+        assert L.fortis_stencil_route(C.byref(_table_with(ins))) == 1
+        assert L.fortis_stencil_check(C.byref(_table_with(ins))) == 0
+    bad = [[(12, 0, 1)],                     # unknown op
+           [(2 | 0x200, 0, 1)],              # unknown flag
+           [(0, 0, 5)],                      # scalar out of range
+           [(0, 0, 17)],                     # constant out of range
+           [(0, 0, 32)]]                     # result not yet computed
     for ins in bad:
+        assert L.fortis_stencil_route(C.byref(_table_with(ins))) == -1
         assert L.fortis_stencil_check(C.byref(_table_with(ins))) == -1
     capfd.readouterr()
 
