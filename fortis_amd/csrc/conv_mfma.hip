@@ -75,59 +75,67 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     const int sh = s.ups ? 1 : 0;
     const long srcW = s.W >> sh, sHW = (long)(s.H >> sh) * srcW, schan = (long)(s.D >> sh) * sHW;
 
-    // per-thread staging map of the input run (same for every chunk): global offset inside a chunk's
-    // channel group, c * schan + offset in the channel; -1: zero padding
-    int goff[NX];
+    // per-thread staging map of the input run (same for every chunk): byte offset inside a chunk's channel
+    // group, (c * schan + offset in the channel) * 4.  Padding elements load from offset 0 (goff) and carry
+    // the mark 0xffffffff in gchk, which the store compares with the chunk's limit.
+    unsigned goff[NX], gchk[NX];
 #pragma unroll
     for (int i = 0; i < NX; i++) {
         const int el = tid + i * CM_THREADS;
-        goff[i] = -1;
+        goff[i] = 0;
+        gchk[i] = 0xffffffffu;
         if (el < XCH) {
             unsigned c, rem, kd, r, yp, xp;
             st_divmod((unsigned)el, s.mKR, c, rem);
             st_divmod(rem, s.mR, kd, r);
             st_divmod((unsigned)(m0 + r), s.mP, yp, xp);
             const int zz = z + (int)kd - (KD / 2), yy = (int)yp - PADK, xx = (int)xp - PADK;
-            if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W)
-                goff[i] = (int)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh));
+            if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W) {
+                goff[i] = gchk[i] = (unsigned)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh)) * 4u;
+            }
         }
     }
 
-    // offsets at or beyond chunk_lim belong to channels past the last one (partial last chunk); as
-    // unsigned, the padding mark -1 is beyond it too
+    // byte offsets at or beyond chunk_lim belong to channels past the last one (only in a partial last chunk)
     auto chunk_lim = [&](int ch) {
         const int cleft = s.C - ch * CC;
-        return (unsigned)((cleft < CC ? cleft : CC) * schan);
+        return (unsigned)((cleft < CC ? cleft : CC) * schan) * 4u;
     };
-    cm_v4f rw[NW];
-    float rx[NX];
-    auto load_chunk = [&](int ch) {
+    // Two register sets: while LDS holds chunk k, set (k+1)&1 carries chunk k+1 (loaded one step ago) and
+    // set k&1 receives chunk k+2, so a chunk's global loads have two multiply phases to arrive in.
+    struct Regs { cm_v4f rw[NW]; float rx[NX]; };
+    Regs rg[2];
+    auto load_chunk = [&](Regs& r, int ch) {
         const cm_v4f* wsrc = (const cm_v4f*)(wp + ((long)fg * s.nchunks + ch) * WCH);
 #pragma unroll
         for (int i = 0; i < NW; i++) {
             const int f4 = tid + i * CM_THREADS;
-            rw[i] = wsrc[f4 < WCH / 4 ? f4 : 0];
+            r.rw[i] = wsrc[f4 < WCH / 4 ? f4 : 0];
         }
-        const float* xsrc = x + (long)ch * CC * schan;
-        const unsigned lim = chunk_lim(ch);
+        // uniform base + 32-bit byte offset per lane: no address arithmetic here.  Padding elements read
+        // offset 0 (a valid address); they are replaced by zero only when stored, so nothing waits here.
+        const char* xsrc = (const char*)(x + (long)ch * CC * schan);
+        if ((ch + 1) * CC <= s.C) {
 #pragma unroll
-        for (int i = 0; i < NX; i++)
-            // always load from a valid address (the element itself, or element 0 of a valid channel); the
-            // value is replaced by zero only when it is stored, so that nothing waits for the load here
-            rx[i] = xsrc[(unsigned)goff[i] < lim ? goff[i] : 0];
+            for (int i = 0; i < NX; i++) r.rx[i] = *(const float*)(xsrc + goff[i]);
+        } else {
+            const unsigned lim = chunk_lim(ch);      // partial last chunk: channels past the last one read offset 0 too
+#pragma unroll
+            for (int i = 0; i < NX; i++) r.rx[i] = *(const float*)(xsrc + (goff[i] < lim ? goff[i] : 0u));
+        }
     };
-    auto store_chunk = [&](int buf, int ch) {
+    auto store_chunk = [&](const Regs& r, int buf, int ch) {
         cm_v4f* wdst = (cm_v4f*)(sW + buf * WCH);
 #pragma unroll
         for (int i = 0; i < NW; i++) {
             const int f4 = tid + i * CM_THREADS;
-            if (f4 < WCH / 4) wdst[f4] = rw[i];
+            if (f4 < WCH / 4) wdst[f4] = r.rw[i];
         }
         float* xdst = sX + buf * XCHP + tid;
         const unsigned lim = chunk_lim(ch);
 #pragma unroll
         for (int i = 0; i < NX; i++)
-            if (i * CM_THREADS < XCHP) xdst[i * CM_THREADS] = (unsigned)goff[i] < lim ? rx[i] : 0.f;
+            if (i * CM_THREADS < XCHP) xdst[i * CM_THREADS] = gchk[i] < lim ? r.rx[i] : 0.f;
     };
 
     const int ft = wave % FW, mt0 = (wave / FW) * NMT;
@@ -141,12 +149,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
 
     const int ch0 = blockIdx.z * s.chunks_per;
     const int ch1 = ch0 + s.chunks_per < s.nchunks ? ch0 + s.chunks_per : s.nchunks;
-    load_chunk(ch0);
-    store_chunk(0, ch0);
-    cm_lds_barrier();
-    for (int ch = ch0; ch < ch1; ch++) {
-        const int buf = (ch - ch0) & 1;
-        if (ch + 1 < ch1) load_chunk(ch + 1);
+    auto multiply = [&](int buf) {
         const float* w = sW + buf * WCH + wbase;
         const float* xs = sX + buf * XCHP + xbase;
 #pragma unroll
@@ -164,8 +167,39 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
                         for (int j = 0; j < NMT; j++)
                             acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, xs[j * 32 + xoff], acc[j], 0, 0, 0);
                     }
-        if (ch + 1 < ch1) store_chunk(buf ^ 1, ch + 1);
+    };
+    // One step of the pipeline on chunk ch (LDS buffer buf): fetch chunk ch + 2 into `far`, multiply, move
+    // chunk ch + 1 from `near` into the other LDS buffer.  The steady-state form is unconditional: the
+    // compiler's wait insertion counts loads behind a branch as possibly absent and would then wait for
+    // the newest loads where only the oldest are needed.
+    auto step_full = [&](int ch, int buf, Regs& far, const Regs& near) {
+        load_chunk(far, ch + 2);
+        __builtin_amdgcn_sched_barrier(0);     // nothing of the store below (it waits for `near`) moves above the multiplies
+        multiply(buf);
+        __builtin_amdgcn_sched_barrier(0);
+        store_chunk(near, buf ^ 1, ch + 1);
         cm_lds_barrier();
+    };
+    auto step_tail = [&](int ch, int buf, Regs& far, const Regs& near) {
+        if (ch + 2 < ch1) load_chunk(far, ch + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(buf);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ch + 1 < ch1) store_chunk(near, buf ^ 1, ch + 1);
+        cm_lds_barrier();
+    };
+    load_chunk(rg[0], ch0);
+    store_chunk(rg[0], 0, ch0);
+    cm_lds_barrier();
+    load_chunk(rg[1], ch0 + 1 < ch1 ? ch0 + 1 : ch0);     // unconditional for the same reason (a lone chunk is fetched twice)
+    int ch = ch0;
+    for (; ch + 3 < ch1; ch += 2) {
+        step_full(ch, 0, rg[0], rg[1]);
+        step_full(ch + 1, 1, rg[1], rg[0]);
+    }
+    for (; ch < ch1; ch += 2) {
+        step_tail(ch, 0, rg[0], rg[1]);
+        if (ch + 1 < ch1) step_tail(ch + 1, 1, rg[1], rg[0]);
     }
 
     // epilogue: a lane holds one position and 16 output channels per m-tile
@@ -319,6 +353,7 @@ static int launch(const float* x, const float* wp, float* y, ConvMShape s, const
 {
     const long R = MT + (KS == 3 ? 2 * s.P + 2 : 0), xch = (long)cm_cc(KD * KS * KS) * KD * R;
     if (xch > (long)CM_THREADS * CM_NXMAX) return -1;     // run too long to stage
+    if ((long)cm_cc(KD * KS * KS) * s.D * s.H * s.W >= (1L << 30)) return -1;   // a chunk's byte offsets must fit 32 bits
     return xch <= CM_THREADS * 8 ? launch_nx<KD, KS, MT, FT, 8>(x, wp, y, s, e, st) : launch_nx<KD, KS, MT, FT, 16>(x, wp, y, s, e, st);
 }
 
