@@ -10,6 +10,10 @@ only (git-ignored).  Test infrastructure: run by tests/test_gpu_hosts.py, built 
                   LeakyReLU(0.1) on 1x3x16^3)
   zb_expert_hip   mom6_zb/zb_host_expert.f90    (per-layer hand-batched mlp_forward(xb(27,4736), yb(3,4736));
                   the model is mom6_zb/zb_nn.npz with its input and output norms)
+  zb_lifted_step.so   no host: the step file and the stencil tables + fortis_gather / fortis_scatter entries that
+                  the emitter writes for mom6_zb/gather.json, scatter.json, zb_loop_verdict.json, kdist.json (what
+                  links beside the lifted host mom6_zb/host_fissioned.fir; that FIR text is of a newer dialect than
+                  this flang parses, so the test drives the entries itself in the host's call order, :732-740)
 
 Each links: host.o + step file emitted by fortis_amd/emit.py + libfortis_rt.so."""
 import os
@@ -72,7 +76,19 @@ def main():
     c, _ = emit.emit_mlp_step(os.path.join(OUT, "zb_expert_step"), [W["A0"], W["A1"]], [W["b0"], W["b1"]], ["relu", None],
                               rows=4736, in_norms=W["in_norms"], out_norms=W["out_norms"])
     link(os.path.join(REF, "mom6_zb/zb_host_expert.f90"), c, "zb_expert_hip")
-    print("build_hosts: built toy_dev_hip, toy_call_hip, conv_dev_hip, conv_call_hip, zb_expert_hip in", OUT)
+    # the lifted ZB step: plan + tables + generated entries in one shared object
+    import json
+    g = os.path.join(ROOT, "tests", "golden")
+    desc = [json.load(open(os.path.join(g, "zb_%s.json" % n))) for n in ("gather", "scatter", "loop", "kdist")]
+    c, b = emit.emit_mlp_step(os.path.join(OUT, "zb_lifted_step"), [W["A0"], W["A1"]], [W["b0"], W["b1"]], ["relu", None],
+                              rows=71040, in_norms=W["in_norms"], out_norms=W["out_norms"], verdict="batched", expanded=True,
+                              count=71040, gather=True, scatter=True)
+    tc = emit.emit_stencil_tables(os.path.join(OUT, "zb_lifted_tables.c"), *desc)
+    run(["gcc", "-O2", "-shared", "-fPIC", "-I", os.path.join(ROOT, "include"), c, tc, "-L", os.path.join(ROOT, "fortis_amd"),
+         "-lfortis_rt", "-Wl,-rpath,$ORIGIN/../../fortis_amd", "-o", os.path.join(OUT, "zb_lifted_step.so")])
+    for f in (c, b, tc):
+        os.remove(f)
+    print("build_hosts: built toy_dev_hip, toy_call_hip, conv_dev_hip, conv_call_hip, zb_expert_hip, zb_lifted_step.so in", OUT)
     return 0
 
 

@@ -68,3 +68,45 @@ def test_zb_expert_host_matches_native_golden(gpu, tmp_path, golden):
             ref = G[name][n].astype(np.float64)
             got = raw[f, layer - 1]
             assert np.abs(got - ref).max() <= 5e-6 * np.abs(ref).max(), (name, layer)
+
+
+_LIFTED_CHILD = r"""
+import ctypes as C, os, sys
+import numpy as np
+root, golden = sys.argv[1], sys.argv[2]
+sys.path.insert(0, root)
+from oracle import oracle as O          # checker: field synthesis of the reference host only
+so = C.CDLL(os.path.join(root, "oracle", "_ref", "zb_lifted_step.so"))   # constructors: plan bound, tables configured
+G = np.load(os.path.join(golden, "zb_native_golden.npz"))
+F = O.zb_fields(); P = O.zb_prep(F)
+p = lambda a: a.ctypes.data_as(C.c_void_p)
+n3 = 68 * 78 * 15
+for step in range(2):
+    Txy_h, Txx, Tyy, Txy = np.zeros(68 * 78, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)
+    so.fortis_gather(p(P["sh_xy_h"]), p(F["sh_xx"]), p(P["vort_xy_h"]), p(P["norm_h"]))
+    so.mlp_forward_batched(None, None)
+    for k in range(1, 16):
+        so.fortis_scatter(C.c_int(k), p(P["norm_h"]), p(F["kappa_h"]), p(Txy_h), p(Txx), p(Tyy))
+        h, m = Txy_h.reshape(78, 68), F["mask2dBu"].reshape(78, 68)
+        Txy.reshape(15, 78, 68)[k - 1][2:75, 2:65] = np.float32(0.25) * ((h[3:76, 3:66] + h[2:75, 2:65]) + (h[2:75, 3:66] + h[3:76, 2:65])) * m[2:75, 2:65]
+    lay = G["layers"] - 1
+    for got, key in ((Txx, "Txx"), (Tyy, "Tyy"), (Txy, "Txy")):
+        ref = G[key].astype(np.float64)
+        err = np.abs(got.reshape(15, 78, 68)[lay] - ref).max() / np.abs(ref).max()
+        assert err < 1e-5, (key, err)
+    for n, a in enumerate((Txx, Tyy, Txy)):
+        assert abs(a.astype(np.float64).sum() - G["checksum"][n]) < 1e-5 * np.abs(a).sum()
+print("lifted step ok")
+"""
+
+
+def test_emitted_step_and_tables_drive_the_lifted_zb_step(gpu, golden, tmp_path):
+    """The files fortis_amd/emit.py writes for the lifted ZB host -- the step (plan + host facts) and the stencil
+    tables with their generated fortis_gather / fortis_scatter entries -- built into one shared object at build
+    time and driven in the lifted host's call order (mom6_zb/host_fissioned.fir:732-740), in a process of its
+    own because loading the object binds the step; results against the reference's native CPU build."""
+    root = os.path.dirname(REFBIN.rstrip("/")).rsplit("/oracle", 1)[0]
+    if not os.path.exists(os.path.join(REFBIN, "zb_lifted_step.so")):
+        pytest.skip("zb_lifted_step.so not built")
+    r = subprocess.run([os.sys.executable, "-c", _LIFTED_CHILD, root, golden], capture_output=True, text=True, timeout=180)
+    assert r.returncode == 0 and "lifted step ok" in r.stdout, r.stdout + r.stderr

@@ -107,3 +107,25 @@ def test_route_of_tables(golden):
     bad = S.build_table(gd, lp, kd, "gather")
     bad.elt[0] = 2
     assert L.fortis_stencil_route(C.byref(bad)) == -1
+
+
+def test_emitted_table_file_compiles_for_other_arities_and_types(golden, tmp_path):
+    """The C the emitter writes in place of gather.cu: entries with the generator's argument lists
+    (driver/fortis_gather_emit.py:62-64, 84) for a descriptor with fp64 arrays, functions and no loop
+    distribution (so the gather keeps its int argument); it must compile against the public header, and
+    the tables inside must be the ones build_table makes."""
+    import subprocess
+    from fortis_amd import emit
+    gd, sd, lp, kd = _zb_desc(golden)
+    gd, sd = copy.deepcopy(gd), copy.deepcopy(sd)
+    gd["arrays"][3]["elt"] = "f64"
+    gd["exprs"] = ["(tv / (S0 + 1.0e-30))", "sqrtf(fmaxf(tv, 0.0f))"]
+    sd["arrays"][3]["elt"] = sd["arrays"][4]["elt"] = "f64"
+    path = emit.emit_stencil_tables(str(tmp_path / "tables.c"), gd, sd, lp, None)
+    text = open(path).read()
+    assert "void fortis_gather(int a0, const float* H0, const float* H1, const float* H2, const double* H3)" in text
+    assert "void fortis_scatter(int a0, float* H0, float* H1, float* H2, double* H3, double* H4)" in text
+    assert ".elt = {4, 4, 4, 8}" in text and ".cdouble = {1, 0}" in text and "0x107" not in text and "{0x103, 0, 32}" in text
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    r = subprocess.run(["gcc", "-Wall", "-Werror", "-c", "-I", inc, path, "-o", str(tmp_path / "tables.o")], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
