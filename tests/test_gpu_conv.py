@@ -16,7 +16,12 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("C_,H,W,F,k,stride,pad", [(1, 16, 16, 4, 3, 1, 1), (5, 17, 13, 7, 3, 1, 1), (8, 32, 32, 16, 3, 2, 1),
-                                                    (32, 20, 24, 4, 1, 1, 0), (3, 9, 9, 9, 5, 1, 2), (64, 16, 16, 64, 3, 1, 1)])
+                                                    (32, 20, 24, 4, 1, 1, 0), (3, 9, 9, 9, 5, 1, 2), (64, 16, 16, 64, 3, 1, 1),
+                                                    # matrix-core path: channel counts that end in a partial staged chunk, a partial
+                                                    # output-channel group, ragged image sizes, an image wide enough for the
+                                                    # 16-round staging variant, and the single-tap form with its 16-channel chunks
+                                                    (6, 40, 36, 48, 3, 1, 1), (37, 70, 50, 16, 3, 1, 1), (20, 300, 260, 32, 3, 1, 1),
+                                                    (50, 33, 47, 40, 1, 1, 0), (130, 12, 12, 70, 3, 1, 1)])
 def test_conv2d_bias_act_vs_oracle(L, gpu, C_, H, W, F, k, stride, pad):
     rng = np.random.default_rng(0)
     x = rng.standard_normal((C_, H, W)).astype(np.float32)
@@ -119,7 +124,10 @@ def test_op_micro_suite(L, gpu):
 
 
 @pytest.mark.parametrize("C_,D,H,W,F,k,pad", [(3, 16, 16, 16, 8, 3, 1), (4, 9, 8, 7, 6, 3, 1), (2, 7, 7, 7, 3, 5, 2),
-                                               (64, 9, 9, 9, 64, 3, 1), (5, 6, 6, 6, 10, 1, 0), (3, 8, 8, 8, 4, 3, 0)])
+                                               (64, 9, 9, 9, 64, 3, 1), (5, 6, 6, 6, 10, 1, 0), (3, 8, 8, 8, 4, 3, 0),
+                                               # matrix-core path: odd channel count (partial 2-channel chunk), ragged extents,
+                                               # a partial output-channel group; a volume whose rows need the 16-round staging
+                                               (7, 12, 11, 10, 20, 3, 1), (6, 5, 90, 70, 80, 3, 1)])
 def test_conv3d_bias_act_residual_vs_oracle(L, gpu, C_, D, H, W, F, k, pad):
     rng = np.random.default_rng(1)
     x = rng.standard_normal((C_, D, H, W)).astype(np.float32)
