@@ -77,8 +77,7 @@ __device__ __forceinline__ void lds_barrier()
 // Schedule of one k slab (NKG groups of 8 k, one group = TM*TN*4 MFMAs per wave):
 //   top      global loads of the next slab -> staging registers (ra, rw)
 //   group g  LDS reads of the fragments of group g+1, then the MFMAs of group g
-//   before group NKG-2: staging registers -> other LDS buffer
-//   before the last group: barrier, LDS reads of the next slab's group 0
+//   before the last group: staging registers -> other LDS buffer, barrier, LDS reads of the next slab's group 0
 // so every LDS read has a whole group of MFMAs to arrive, and the barrier is followed by MFMAs that
 // were already fed.  The staging registers belong to the caller: when `preloaded`, they already hold
 // this tile's slab 0, and when `has_next`, the last slab's "next slab" is slab 0 of tile (m0n, n0n),
@@ -130,36 +129,38 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
             ow[t] = ((unsigned)(row < lastn ? row : lastn) * (unsigned)K + kq * 4) * 4u;
         }
     };
+    // Every staged chunk of a thread sits at the same k inside the slab (GM_THREADS is a multiple of F4R).
+    static_assert(GM_THREADS % F4R == 0, "a thread's chunks share their k position");
+    const int kq4 = (tid % F4R) * 4;
+    // ONE load site and ONE store site per slab, whatever the slab is (a full one, the one that runs past K,
+    // slab 0 of the next tile): the compiler otherwise merges the register sets of the different sites with
+    // copies placed right behind the loads, and every wave then waits for its loads before it multiplies.
+    // A chunk at or beyond K reads the row's chunk 0 instead (a valid address) and is zeroed when stored.
     auto load_slab = [&](const float* Ab, const float* Wb, const unsigned (&oa)[LA], const unsigned (&ow)[LW], long k0) __attribute__((always_inline)) {
         const char* ab = (const char*)(Ab + k0);
         const char* wb = (const char*)(Wb + k0);
-        if (k0 + GM_BK <= K) {
+        const unsigned adj = k0 + kq4 < K ? 0u : (unsigned)kq4 * 4u;
 #pragma unroll
-            for (int t = 0; t < LA; t++) ra[t] = *(const v4f*)(ab + oa[t]);
+        for (int t = 0; t < LA; t++) ra[t] = *(const v4f*)(ab + (oa[t] - adj));
 #pragma unroll
-            for (int t = 0; t < LW; t++) rw[t] = *(const v4f*)(wb + ow[t]);
-        } else {
-            // the slab that runs past K: chunks beyond K read the row's chunk 0 instead and become zeros
-            const v4f zero = (v4f)(0.f);
-#pragma unroll
-            for (int t = 0; t < LA; t++) {
-                const int kq = (tid + t * GM_THREADS) % F4R;
-                const bool ok = k0 + kq * 4 < K;
-                const v4f v = *(const v4f*)(ab + (oa[t] - (ok ? 0u : kq * 16u)));
-                ra[t] = ok ? v : zero;
-            }
-#pragma unroll
-            for (int t = 0; t < LW; t++) {
-                const int kq = (tid + t * GM_THREADS) % F4R;
-                const bool ok = k0 + kq * 4 < K;
-                const v4f v = *(const v4f*)(wb + (ow[t] - (ok ? 0u : kq * 16u)));
-                rw[t] = ok ? v : zero;
-            }
-        }
+        for (int t = 0; t < LW; t++) rw[t] = *(const v4f*)(wb + (ow[t] - adj));
     };
-    auto store_slab = [&](int buf) __attribute__((always_inline)) {
+    // k0: the slab the staging registers hold
+    auto store_slab = [&](int buf, long k0) __attribute__((always_inline)) {
         float* a = sA + buf * BM * GM_LDK;
         float* w = sW + buf * BN * GM_LDK;
+        if (k0 + GM_BK > K) {
+            // only the slab that runs past K comes here; the empty asm keeps this a branch (as a select it
+            // would cost every slab one instruction per staged register)
+            asm volatile("" ::: "memory");
+            if (k0 + kq4 >= K) {
+                const v4f zero = (v4f)(0.f);
+#pragma unroll
+                for (int t = 0; t < LA; t++) ra[t] = zero;
+#pragma unroll
+                for (int t = 0; t < LW; t++) rw[t] = zero;
+            }
+        }
 #pragma unroll
         for (int t = 0; t < LA; t++) {
             const int f = tid + t * GM_THREADS, row = f / F4R, kq = f % F4R;
@@ -198,26 +199,28 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     const float* Ab = A + m0 * K;
     const float* Wb = W + n0 * K;
     if (!preloaded) load_slab(Ab, Wb, oa, ow, 0);
-    store_slab(0);
+    store_slab(0, 0);
     lds_barrier();
     read_frag(0, 0, 0);
     for (int sl = 0; sl < nslab; sl++) {
         const int buf = sl & 1;
         const bool more = sl + 1 < nslab;
-        if (more) load_slab(Ab, Wb, oa, ow, (long)(sl + 1) * GM_BK);
-        else if (has_next) {
-            unsigned oan[LA], own[LW];
-            offsets(m0n, n0n, oan, own);
-            load_slab(A + m0n * K, W + n0n * K, oan, own, 0);
+        long knext = (long)(sl + 1) * GM_BK;
+        if (!more && has_next) {
+            // the staging registers now fetch slab 0 of the next tile: its offsets replace this tile's
+            offsets(m0n, n0n, oa, ow);
+            Ab = A + m0n * K;
+            Wb = W + n0n * K;
+            knext = 0;
         }
+        if (more || has_next) load_slab(Ab, Wb, oa, ow, knext);
 #pragma unroll
         for (int kg = 0; kg + 1 < NKG; kg++) {
             read_frag((kg + 1) & 1, buf, kg + 1);
-            // the staged slab goes to LDS one group before the barrier, so the writes drain behind MFMAs
-            if (kg == NKG - 2 && NKG > 2 && more) store_slab(buf ^ 1);
             multiply(kg & 1);
         }
-        if (NKG == 2 && more) store_slab(buf ^ 1);
+        // the staged slab goes to LDS as late as possible: its loads have had NKG - 1 groups of MFMAs to arrive
+        if (more) store_slab(buf ^ 1, knext);
         lds_barrier();
         if (more) read_frag(0, buf ^ 1, 0);
         multiply((NKG - 1) & 1);
