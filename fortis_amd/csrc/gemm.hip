@@ -139,11 +139,22 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     auto load_slab = [&](const float* Ab, const float* Wb, const unsigned (&oa)[LA], const unsigned (&ow)[LW], long k0) __attribute__((always_inline)) {
         const char* ab = (const char*)(Ab + k0);
         const char* wb = (const char*)(Wb + k0);
-        const unsigned adj = k0 + kq4 < K ? 0u : (unsigned)kq4 * 4u;
 #pragma unroll
-        for (int t = 0; t < LA; t++) ra[t] = *(const v4f*)(ab + (oa[t] - adj));
+        for (int t = 0; t < LA; t++) ra[t] = *(const v4f*)(ab + oa[t]);
 #pragma unroll
-        for (int t = 0; t < LW; t++) rw[t] = *(const v4f*)(wb + (ow[t] - adj));
+        for (int t = 0; t < LW; t++) rw[t] = *(const v4f*)(wb + ow[t]);
+    };
+    // Before the load of a slab that runs past K (the last one of a tile, after which these offsets are not
+    // used again): chunks at or beyond K are pointed at their row's chunk 0.
+    auto clamp_offsets = [&](long k0, unsigned (&oa)[LA], unsigned (&ow)[LW]) __attribute__((always_inline)) {
+        if (k0 + GM_BK > K) {
+            asm volatile("" ::: "memory");               // stays a branch
+            const unsigned adj = k0 + kq4 < K ? 0u : (unsigned)kq4 * 4u;
+#pragma unroll
+            for (int t = 0; t < LA; t++) oa[t] -= adj;
+#pragma unroll
+            for (int t = 0; t < LW; t++) ow[t] -= adj;
+        }
     };
     // k0: the slab the staging registers hold
     auto store_slab = [&](int buf, long k0) __attribute__((always_inline)) {
@@ -198,12 +209,16 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     offsets(m0, n0, oa, ow);
     const float* Ab = A + m0 * K;
     const float* Wb = W + n0 * K;
-    if (!preloaded) load_slab(Ab, Wb, oa, ow, 0);
+    if (!preloaded) {
+        clamp_offsets(0, oa, ow);
+        load_slab(Ab, Wb, oa, ow, 0);
+    }
     store_slab(0, 0);
     lds_barrier();
     read_frag(0, 0, 0);
-    for (int sl = 0; sl < nslab; sl++) {
-        const int buf = sl & 1;
+    // one k slab out of LDS buffer `buf` (a literal at both call sites, so every LDS address below is a
+    // constant offset from the thread's base and no address arithmetic is left in the loop)
+    auto slab = [&](int sl, int buf) __attribute__((always_inline)) {
         const bool more = sl + 1 < nslab;
         long knext = (long)(sl + 1) * GM_BK;
         if (!more && has_next) {
@@ -213,7 +228,10 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
             Wb = W + n0n * K;
             knext = 0;
         }
-        if (more || has_next) load_slab(Ab, Wb, oa, ow, knext);
+        if (more || has_next) {
+            clamp_offsets(knext, oa, ow);
+            load_slab(Ab, Wb, oa, ow, knext);
+        }
 #pragma unroll
         for (int kg = 0; kg + 1 < NKG; kg++) {
             read_frag((kg + 1) & 1, buf, kg + 1);
@@ -224,6 +242,10 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
         lds_barrier();
         if (more) read_frag(0, buf ^ 1, 0);
         multiply((NKG - 1) & 1);
+    };
+    for (int sl = 0; sl < nslab; sl += 2) {
+        slab(sl, 0);
+        if (sl + 1 < nslab) slab(sl + 1, 1);
     }
 
     // epilogue: lane holds column n = lr of 16 rows per MFMA tile.
