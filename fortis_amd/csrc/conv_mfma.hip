@@ -263,6 +263,22 @@ static int conv_cus()
     return n;
 }
 
+// Partial sums of channel-split launches: one buffer for every shape (launches on the library's stream run
+// one after the other).  It grows on the first, eager run of a plan; replays and captured runs find it in
+// place.  An outgrown buffer stays allocated: a graph captured earlier may still name it.
+static float* conv_split_scratch(size_t need)
+{
+    static float* scratch = nullptr;
+    static size_t cap = 0;
+    if (need > cap) {
+        float* p = nullptr;
+        if (hipMalloc((void**)&p, need) != hipSuccess) { fprintf(stderr, "fortis: no memory for %zu bytes of conv partial sums\n", need); return nullptr; }
+        scratch = p;
+        cap = need;
+    }
+    return scratch;
+}
+
 // Packs conv weights W[F][C][T] (T taps, row-major) into the kernel's order
 //   [F/FT][ceil(C/CC)][channel pair CC/2][tap T][half 2][FT channels], zero padded; CC = cm_cc(T)
 //   channels per chunk; FT = 32 when the GEMM has at most 32 output channels, else 64 (the launcher
@@ -326,16 +342,8 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     const long ospatial = (long)s.D * s.H * s.W * (s.mode ? 4 : 1);
     s.osize = (long)(s.mode ? s.F / 4 : s.F) * ospatial;
     if (s.ksplit > 1) {
-        // scratch grows on the first (eager) run of a plan; replays and captured runs find it in place
-        static float* scratch = nullptr;
-        static size_t cap = 0;
-        const size_t need = (size_t)s.ksplit * s.osize * sizeof(float);
-        if (need > cap) {
-            // an outgrown buffer stays allocated: a graph captured earlier may still name it
-            HIP_OK(hipMalloc((void**)&scratch, need));
-            cap = need;
-        }
-        s.part = scratch;
+        s.part = conv_split_scratch((size_t)s.ksplit * s.osize * sizeof(float));
+        if (!s.part) return -1;
     }
     dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);
     hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);

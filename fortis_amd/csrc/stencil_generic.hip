@@ -147,6 +147,33 @@ int fortis_stencil_validate(const fortis_stencil_t* t)
         const fortis_ref_t& f = r < t->nrefs ? t->refs[r] : t->scal[r - t->nrefs];
         if (f.array < 0 || f.array >= t->narrays) { fprintf(stderr, "fortis: stencil ref names array %d\n", f.array); return -1; }
     }
+    // Every element a kernel will touch must lie inside its array's plane: base + i*si + j*sj in [0, plane) for
+    // every visited cell (the plane index kk only adds whole planes).  A descriptor that fails this would make
+    // the kernels read or write outside the arrays.
+    const long ni = t->ni > 0 ? t->ni : 1, sx = t->sx > 0 ? t->sx : 1;
+    for (int r = 0; r < t->nrefs + t->nscal; r++) {
+        const fortis_ref_t& f = r < t->nrefs ? t->refs[r] : t->scal[r - t->nrefs];
+        long lo, hi;
+        if (t->cells) {
+            lo = hi = f.base + (1 + t->cells[0] % sx) * f.si + (1 + t->cells[0] / sx) * f.sj;
+            for (long c = 0; c < t->count; c++) {
+                if (t->cells[c] < 0) { fprintf(stderr, "fortis: negative entry in the stencil cell list\n"); return -1; }
+                const long e = f.base + (1 + t->cells[c] % sx) * f.si + (1 + t->cells[c] / sx) * f.sj;
+                lo = e < lo ? e : lo;
+                hi = e > hi ? e : hi;
+            }
+        } else {
+            const long i0 = t->ilo, i1 = t->ilo + (t->count < ni ? t->count : ni) - 1;
+            const long j0 = t->jlo, j1 = t->jlo + (t->count + ni - 1) / ni - 1;
+            lo = f.base + (f.si >= 0 ? i0 : i1) * f.si + (f.sj >= 0 ? j0 : j1) * f.sj;
+            hi = f.base + (f.si >= 0 ? i1 : i0) * f.si + (f.sj >= 0 ? j1 : j0) * f.sj;
+        }
+        if (lo < 0 || hi >= t->plane[f.array]) {
+            fprintf(stderr, "fortis: stencil %s %d reaches elements %ld..%ld of array %d, whose plane has %ld\n",
+                    r < t->nrefs ? "slot" : "scalar", r < t->nrefs ? r : r - t->nrefs, lo, hi, f.array, t->plane[f.array]);
+            return -1;
+        }
+    }
     for (int n = 0; n < t->nins; n++) {
         const int op = t->ins[n].op & 0xff, codes[2] = { t->ins[n].a, t->ins[n].b };
         bool ok = op <= FORTIS_OP_F32 && (t->ins[n].op & ~(0xff | FORTIS_INS_F64)) == 0;

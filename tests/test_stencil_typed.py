@@ -129,3 +129,29 @@ def test_emitted_table_file_compiles_for_other_arities_and_types(golden, tmp_pat
     inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
     r = subprocess.run(["gcc", "-Wall", "-Werror", "-c", "-I", inc, path, "-o", str(tmp_path / "tables.o")], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
+
+
+def test_tables_that_reach_outside_their_arrays_are_refused(golden, capfd):
+    """The kernels index the arrays with no bounds checks of their own, so a descriptor whose offsets or
+    rectangle leave an array's plane (as a range of memory: a column offset that merely wraps into the
+    neighbouring row is the lifter's business) is refused at configuration, on the host."""
+    L = fortis_amd.load()
+    gd, sd, lp, kd = _zb_desc(golden)
+
+    def route(fn, role="gather", cells=None):
+        g, s_, l = copy.deepcopy(gd), copy.deepcopy(sd), copy.deepcopy(lp)
+        fn(g, s_, l)
+        t = S.build_table(g if role == "gather" else s_, l, kd, role, cells=cells)
+        return L.fortis_stencil_route(C.byref(t))
+
+    assert route(lambda g, s_, l: None) == 0
+    assert route(lambda g, s_, l: g["slots"][0]["idx"][1].__setitem__(1, -3)) == -1          # A(i-1, j-3, k) with j from 3
+    assert route(lambda g, s_, l: g["slots"][26]["idx"][1].__setitem__(1, 3)) == -1          # A(..., j+3) with j up to 76 of 78
+    assert route(lambda g, s_, l: l["outer"].update(lo=10, hi=83)) == -1                     # rectangle shifted past the last row
+    assert route(lambda g, s_, l: s_["stores"][0]["idx"][1].__setitem__(1, 5), "scatter") == -1
+    assert route(lambda g, s_, l: g["scalars"][0]["idx"][1].__setitem__(1, -3)) == -1
+    ok_cells = np.array([1 + 1 * 68, 40 + 50 * 68], np.int32)
+    assert route(lambda g, s_, l: None, cells=ok_cells) == 0
+    assert route(lambda g, s_, l: None, cells=np.array([0], np.int32)) == -1                 # the corner has no i-1 neighbour
+    assert route(lambda g, s_, l: None, cells=np.array([67 + 77 * 68], np.int32)) == -1
+    assert "reaches elements" in capfd.readouterr().err
