@@ -15,11 +15,12 @@
 #include "stencil_dev.h"
 
 #define ST_THREADS 256
+typedef float st_v4f __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, float* __restrict__ X, unsigned rows)
 {
     __shared__ GatherArgs d;
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     params_to_lds(&d, ST_THREADS);
     const int n = st_u(d.nrefs);
     const int tid = threadIdx.x;
@@ -29,13 +30,24 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
         st_row(d, row, i, j, kk);
         // all slot loads are issued before any of them is consumed
         float tv[FORTIS_MAX_REFS];
-#pragma unroll
-        for (int q = 0; q < FORTIS_MAX_REFS; q++) {
-            const StSlotT<const float*> sl = d.refs[q < n ? q : 0];
-            tv[q] = st_g(sl.p)[st_off(sl, i, j, kk)];
-        }
         StCell cell;
-        st_prepare(d, i, j, kk, cell);
+        if (st_u(d.uniform)) {
+            // every slot and scalar has the same strides: one element offset per cell, and a slot is its
+            // pointer plus that offset (unused table entries repeat slot 0)
+            const long off = st_off(d.refs[0], i, j, kk);
+#pragma unroll
+            for (int q = 0; q < FORTIS_MAX_REFS; q++) tv[q] = st_g(d.refs[q].p)[off];
+#pragma unroll
+            for (int sI = 0; sI < ST_SCAL_MAX; sI++) cell.S[sI] = st_g(d.scal[sI].p)[off];
+            st_cell_program(d, cell);
+        } else {
+#pragma unroll
+            for (int q = 0; q < FORTIS_MAX_REFS; q++) {
+                const StSlotT<const float*> sl = d.refs[q < n ? q : 0];
+                tv[q] = st_g(sl.p)[st_off(sl, i, j, kk)];
+            }
+            st_prepare(d, i, j, kk, cell);
+        }
         st_chain_apply(d, cell, tv);
 #pragma unroll
         for (int q = 0; q < FORTIS_MAX_REFS; q++)
@@ -44,13 +56,21 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
     __syncthreads();
     const unsigned lim = (rows - row0 < ST_THREADS ? rows - row0 : ST_THREADS) * n;
     float* out = X + (size_t)row0 * n;
-    for (unsigned idx = tid; idx < lim; idx += ST_THREADS) out[idx] = lds[idx];
+    // the block's rows are one contiguous run of X, which starts on a 16-byte boundary when X does (256 rows
+    // of n floats each): written as 16-byte vectors, the last few floats of a ragged block one by one
+    if (((uintptr_t)X & 15) == 0) {
+        const unsigned lim4 = lim / 4;
+        for (unsigned idx = tid; idx < lim4; idx += ST_THREADS) ((st_v4f*)out)[idx] = ((const st_v4f*)lds)[idx];
+        for (unsigned idx = lim4 * 4 + tid; idx < lim; idx += ST_THREADS) out[idx] = lds[idx];
+    } else {
+        for (unsigned idx = tid; idx < lim; idx += ST_THREADS) out[idx] = lds[idx];
+    }
 }
 
 __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, const float* __restrict__ Y, int kk)
 {
     __shared__ ScatterArgs d;
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     params_to_lds(&d, ST_THREADS);
     const int n = st_u(d.nrefs);
     const int tid = threadIdx.x;
@@ -58,7 +78,13 @@ __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, c
     const unsigned lim = (d.count - col0 < ST_THREADS ? d.count - col0 : ST_THREADS) * n;
     kk += blockIdx.y;                                         // gridDim.y > 1: one enclosing-loop iteration per y
     const float* in = Y + ((size_t)blockIdx.y * d.count + col0) * n;
-    for (unsigned idx = tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
+    if (((uintptr_t)in & 15) == 0) {
+        const unsigned lim4 = lim / 4;
+        for (unsigned idx = tid; idx < lim4; idx += ST_THREADS) ((st_v4f*)lds)[idx] = ((const st_v4f*)in)[idx];
+        for (unsigned idx = lim4 * 4 + tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
+    } else {
+        for (unsigned idx = tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
+    }
     __syncthreads();
     if (col >= d.count) return;
     int i, j;
