@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused inference step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload climsim|zb|zb_ref|toy|unet|tsrgan|copy] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload climsim|zb|zb_ref|zb_unfused|toy|unet|tsrgan|copy] [--no-cpu]
 
 One "step" is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  Prints ONE JSON line: columns/s for the whole job, the roofline figure of the dominant
@@ -27,7 +27,8 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # same command (see profiles/), or None where no counter run has been made for the workload.
 MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((2482.4 * 2 + 936.6) * 1024),
-                    "zb_ref": int((2396.6 * 2 + 936.6) * 1024), "zb_1028x1028x15": int((331322.2 * 2 + 207387.3) * 1024), "toy": None}
+                    "zb_ref": int((2396.6 * 2 + 936.6) * 1024), "zb_1028x1028x15": int((331322.2 * 2 + 207387.3) * 1024), "toy": None,
+                    "zb_unfused_1028x1028x15": int((242224.0 * 2 + 1658880.0) * 1024)}
 
 
 def omp_threads():
@@ -128,6 +129,59 @@ def run_copy(L, args):
                roofline=dict(bound="hbm", kernel="copy_kernel", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
                              frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(avg, 5), bytes_per_launch=2 * n * 4, traffic=None))
     p.close()
+    return out
+
+
+def run_zb_unfused(L, args):
+    """The reference's structure of the ZB step: gather kernel -> X in HBM -> MLP -> Y in HBM -> one scatter launch
+    per layer (mom6_zb/gather.cu:50-57, 82-91), every part timed with HIP events on the library's stream.  The
+    gather is the memory-bound kernel of the path: the roofline block is its."""
+    from fortis_amd import configs, plan as P, stencil as S
+    sx, sy, nz = (int(v) for v in (args.grid or "1028x1028x15").lower().split("x"))
+    gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    gt, st = S.build_table(gd, lp, kd, "gather"), S.build_table(sd, lp, kd, "scatter")
+    A = configs.zb_arrays(sx, sy, nz)
+    rows, count, n3 = gt.count * gt.nk, int(gt.count), sx * sy * nz
+    net = configs.zb_mlp()
+    plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows)
+
+    def dev(a):
+        d = L.fortis_alloc(a.nbytes)
+        L.fortis_h2d(d, a.ctypes.data, a.nbytes)
+        return d
+    dG = (C.c_void_p * 4)(*[dev(A[k]) for k in ("sh_xy_h", "sh_xx", "vort_xy_h", "norm_h")])
+    dS = (C.c_void_p * 5)(dG[3], dev(A["kappa_h"]), dev(np.zeros(sx * sy, np.float32)), dev(np.zeros(n3, np.float32)), dev(np.zeros(n3, np.float32)))
+    dX = L.fortis_plan_tensor_ptr(plan.handle, plan.in_tensor)
+    dY = L.fortis_plan_tensor_ptr(plan.handle, plan.out_tensor)
+    CB = C.CFUNCTYPE(None, C.c_void_p)
+    gather_cb = CB(lambda _: L.fortis_stencil_gather_dev(C.byref(gt), dG, dX))
+
+    def scatter_all(_):
+        for kk in range(nz):
+            L.fortis_stencil_scatter_dev(C.byref(st), dS, C.c_void_p(dY + kk * count * 3 * 4), kk)
+    scatter_cb = CB(scatter_all)
+    for cb in (gather_cb, scatter_cb):
+        L.fortis_time_ms(cb, None, max(1, args.warmup))
+    plan.time_ms(max(1, args.warmup))
+    L.fortis_sync()
+    t0 = time.perf_counter()
+    g_ms = L.fortis_time_ms(gather_cb, None, args.steps) / args.steps
+    m_ms = plan.time_ms(args.steps) / args.steps
+    s_ms = L.fortis_time_ms(scatter_cb, None, args.steps) / args.steps
+    L.fortis_sync()
+    dt = time.perf_counter() - t0
+    g_bytes = 4 * (4 * n3 + 27 * rows)                     # 4 planes read once, X written
+    s_bytes = 4 * (3 * rows + n3 + nz * sx * sy + 3 * rows)  # Y read, norm + kappa read per layer, 3 outputs written
+    gbs = g_bytes / (g_ms * 1e-3) / 1e9
+    roof = dict(bound="hbm", kernel="gather_kernel (stencil gather with lifted expressions)", achieved=round(gbs, 1), peak=PEAK_HBM_GBS,
+                unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(g_ms, 5), bytes_per_launch=g_bytes,
+                scatter_GBs=round(s_bytes / (s_ms * 1e-3) / 1e9, 1), scatter_ms_all_layers=round(s_ms, 5), mlp_ms=round(m_ms, 5),
+                traffic=MEASURED_TRAFFIC.get("zb_unfused_%dx%dx%d" % (sx, sy, nz)))
+    out = dict(rows=rows, dt=(g_ms + m_ms + s_ms) * 1e-3 * args.steps, wall_dt=dt, dtype="f32",
+               config={"workload": "zb_unfused_gather_mlp_scatter_27_64_64_3_%dx%dx%d" % (sx, sy, nz), "columns": rows,
+                       "cells_per_layer": count, "layers": nz, "launches_per_step": 1 + nz + plan.num_kernels},
+               roofline=roof)
+    plan.close()
     return out
 
 
@@ -301,9 +355,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="climsim", choices=["climsim", "zb", "zb_ref", "toy", "copy", "unet", "tsrgan"])
+    ap.add_argument("--workload", default="climsim", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--grid", default=None, help="zb / zb_ref only: SXxSYxNZ grid instead of the reference's 68x78x15")
+    ap.add_argument("--grid", default=None, help="zb / zb_ref / zb_unfused only: SXxSYxNZ grid instead of the reference's 68x78x15 (zb_unfused: 1028x1028x15)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the fused step on ONE GPU; --gpus %d is not supported "
@@ -323,6 +377,8 @@ def main():
         r = run_copy(L, args)
     elif args.workload in ("unet", "tsrgan"):
         r = run_conv(L, args, args.workload)
+    elif args.workload == "zb_unfused":
+        r = run_zb_unfused(L, args)
     else:
         r = run_zb(L, args, reference_net=(args.workload == "zb_ref"))
     ms_per_step = r["dt"] / args.steps * 1e3
