@@ -16,6 +16,9 @@
 // (zero-filled outside the image), and every B operand is a single ds_read at lane base + constant.
 // Weights are re-packed once at plan time in exactly the order the kernel consumes them, so their
 // staging is a straight 16-byte copy.  Both are double buffered through registers.
+// On wide 2-D images that run is mostly halo (two whole rows for one tile's worth of positions), so 3 x 3
+// convs on images at least 64 wide use a second tiling (TILE2D): a workgroup's positions are MT / 32 rows of
+// 32 columns, staged with a one-pixel border at a fixed pitch of 34, tap (kh, kw) = element + kh*34 + kw.
 #include "stencil_dev.h"      // StMagic / st_divmod: exact division by a launch constant
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -31,6 +34,7 @@ static constexpr int cm_cc(int T) { return T >= 27 ? 2 : T >= 9 ? 4 : 16; }
 struct ConvMShape {
     int C, D, H, W, F;         // F = output channels of the GEMM (4x the real ones in transposed mode)
     int P, plane, tiles, nchunks, R;
+    int tiles_x;               // TILE2D: tiles along x
     int mode;                  // 0: convolution, 1: 2x2 stride-2 transposed conv scatter
     int ksplit, chunks_per;    // channel chunks are split over blockIdx.z; > 1: raw partial sums go to `part`
     float* part;               // [ksplit][output elements]
@@ -48,7 +52,8 @@ __device__ __forceinline__ void cm_lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <int KD, int KS, int MT, int FT, int NX>
+#define CM_TP 34       // TILE2D: pitch of a staged row (32 columns + border)
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D>
 __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
 {
@@ -60,16 +65,20 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     constexpr int NMT = MT / 32 / (4 / FW);                      // m-tiles per wave
     static_assert(NMT >= 1, "tile too small for the wave layout");
     constexpr int PADK = KS / 2;
+    constexpr int TH = MT / 32, R2 = (TH + 2) * CM_TP;           // TILE2D: rows per tile, staged elements per channel
+    static_assert(!TILE2D || (KD == 1 && KS == 3), "the 2-D tiling is for 3 x 3 convs");
     extern __shared__ float4 smem4[];
     float* sW = (float*)smem4;                                    // [2][WCH]
     float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R rounded up to the workgroup size]
-    const int XCH = CC * KD * s.R;
+    const int RR = TILE2D ? R2 : s.R;                             // staged elements per channel and kd
+    const int XCH = CC * KD * RR;
     const int XCHP = (XCH + CM_THREADS - 1) / CM_THREADS * CM_THREADS;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int z = blockIdx.x / s.tiles, tile = blockIdx.x - z * s.tiles;
     const int fg = blockIdx.y;
     const int m0 = tile * MT;
+    const int tyi = TILE2D ? tile / s.tiles_x : 0, y0 = tyi * TH, x0 = (tile - tyi * s.tiles_x) * 32;   // TILE2D: tile origin
     const long HW = (long)s.H * s.W, chan = (long)s.D * HW;
     // source geometry: the tensor itself, or the half-resolution tensor a fused nearest upsample reads
     const int sh = s.ups ? 1 : 0;
@@ -86,10 +95,16 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         gchk[i] = 0xffffffffu;
         if (el < XCH) {
             unsigned c, rem, kd, r, yp, xp;
-            st_divmod((unsigned)el, s.mKR, c, rem);
-            st_divmod(rem, s.mR, kd, r);
-            st_divmod((unsigned)(m0 + r), s.mP, yp, xp);
-            const int zz = z + (int)kd - (KD / 2), yy = (int)yp - PADK, xx = (int)xp - PADK;
+            int zz, yy, xx;
+            if (TILE2D) {
+                c = (unsigned)el / R2; r = (unsigned)el % R2;    // compile-time divisors
+                zz = z; yy = y0 + (int)(r / CM_TP) - 1; xx = x0 + (int)(r % CM_TP) - 1;
+            } else {
+                st_divmod((unsigned)el, s.mKR, c, rem);
+                st_divmod(rem, s.mR, kd, r);
+                st_divmod((unsigned)(m0 + r), s.mP, yp, xp);
+                zz = z + (int)kd - (KD / 2); yy = (int)yp - PADK; xx = (int)xp - PADK;
+            }
             if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W) {
                 goff[i] = gchk[i] = (unsigned)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh)) * 4u;
             }
@@ -140,7 +155,9 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
 
     const int ft = wave % FW, mt0 = (wave / FW) * NMT;
     const int wbase = (lane >> 5) * FT + ft * 32 + (lane & 31);
-    const int xbase = (lane >> 5) * KD * s.R + mt0 * 32 + (lane & 31);
+    // lane's element for tap (0, 0) of its first m-tile; an m-tile is 32 consecutive positions of the run, or
+    // (TILE2D) one row of the tile
+    const int xbase = (lane >> 5) * KD * RR + mt0 * (TILE2D ? CM_TP : 32) + (lane & 31);
     v16f acc[NMT];
 #pragma unroll
     for (int j = 0; j < NMT; j++)
@@ -162,10 +179,10 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
                     for (int kw = 0; kw < KS; kw++) {
                         const int tap = (kd * KS + kh) * KS + kw;
                         const float a = w[(cp * T + tap) * 2 * FT];
-                        const int xoff = (2 * cp * KD + kd) * s.R + kh * s.P + kw;
+                        const int xoff = (2 * cp * KD + kd) * RR + kh * (TILE2D ? CM_TP : s.P) + kw;
 #pragma unroll
                         for (int j = 0; j < NMT; j++)
-                            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, xs[j * 32 + xoff], acc[j], 0, 0, 0);
+                            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, xs[j * (TILE2D ? CM_TP : 32) + xoff], acc[j], 0, 0, 0);
                     }
     };
     // One step of the pipeline on chunk ch (LDS buffer buf): fetch chunk ch + 2 into `far`, multiply, move
@@ -206,10 +223,15 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     const long ospatial = s.mode ? 4 * chan : chan;
 #pragma unroll
     for (int j = 0; j < NMT; j++) {
-        const int m = m0 + (mt0 + j) * 32 + (lane & 31);
-        if (m >= s.plane) continue;
         unsigned yy, xx;
-        st_divmod((unsigned)m, s.mP, yy, xx);
+        if (TILE2D) {
+            yy = (unsigned)(y0 + mt0 + j); xx = (unsigned)(x0 + (lane & 31));
+            if ((int)yy >= s.H) continue;
+        } else {
+            const int m = m0 + (mt0 + j) * 32 + (lane & 31);
+            if (m >= s.plane) continue;
+            st_divmod((unsigned)m, s.mP, yy, xx);
+        }
         if ((int)xx >= s.W) continue;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -312,19 +334,24 @@ float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transpos
     return d;
 }
 
-template <int KD, int KS, int MT, int FT, int NX>
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D>
 static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {
     constexpr int T = KD * KS * KS;
     constexpr int CC = cm_cc(T);
     s.tiles = (int)cdiv(s.plane, MT);
     s.R = MT + (KS == 3 ? 2 * s.P + 2 : 0);
+    if (TILE2D) {
+        s.tiles_x = (int)cdiv(s.W, 32);
+        s.tiles = s.tiles_x * (int)cdiv(s.H, MT / 32);
+        s.R = (MT / 32 + 2) * CM_TP;
+    }
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
     const size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, CM_THREADS) * CM_THREADS) * sizeof(float);
     if (shmem > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
-        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         attr = shmem;
     }
     // A launch that leaves most CUs idle (deep, small images) is split over the input channels: each
@@ -346,7 +373,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
         if (!s.part) return -1;
     }
     dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);
-    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
     HIP_OK(hipGetLastError());
     if (s.ksplit > 1) {
         hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)cdiv(s.osize, 256)), dim3(256), 0, st, s.part, y, s.osize,
@@ -359,10 +386,18 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
 template <int KD, int KS, int MT, int FT>
 static int launch(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {
+    if ((long)cm_cc(KD * KS * KS) * s.D * s.H * s.W >= (1L << 30)) return -1;   // a chunk's byte offsets must fit 32 bits
+    if constexpr (KD == 1 && KS == 3) {
+        // image at least one tile wide whose width fills its 32-column tiles to 80 % or more: rows of 32
+        // columns with a one-pixel border; the staging rounds are a compile-time count
+        if (s.W >= 32 && cdiv(s.W, 32) * 32 * 4 <= 5L * s.W && getenv("FORTIS_CONV_LINEAR") == nullptr) {
+            constexpr int NX2 = (cm_cc(9) * (MT / 32 + 2) * CM_TP + CM_THREADS - 1) / CM_THREADS;
+            return launch_nx<1, 3, MT, FT, NX2, true>(x, wp, y, s, e, st);
+        }
+    }
     const long R = MT + (KS == 3 ? 2 * s.P + 2 : 0), xch = (long)cm_cc(KD * KS * KS) * KD * R;
     if (xch > (long)CM_THREADS * CM_NXMAX) return -1;     // run too long to stage
-    if ((long)cm_cc(KD * KS * KS) * s.D * s.H * s.W >= (1L << 30)) return -1;   // a chunk's byte offsets must fit 32 bits
-    return xch <= CM_THREADS * 8 ? launch_nx<KD, KS, MT, FT, 8>(x, wp, y, s, e, st) : launch_nx<KD, KS, MT, FT, 16>(x, wp, y, s, e, st);
+    return xch <= CM_THREADS * 8 ? launch_nx<KD, KS, MT, FT, 8, false>(x, wp, y, s, e, st) : launch_nx<KD, KS, MT, FT, 16, false>(x, wp, y, s, e, st);
 }
 
 // Positions per workgroup: the largest tile that still gives every CU about two workgroups; small images
@@ -387,7 +422,12 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
                             int KS, int kind, const ConvEpi& e, hipStream_t st)
 {
     if (C * D * H * Wd >= 2147483647L || F * D * H * Wd * (kind == 1 ? 4 : 1) >= 2147483647L) return -1;
-    ConvMShape s = { (int)C, (int)D, (int)H, (int)Wd, (int)(kind == 1 ? 4 * F : F), 0, 0, 0, 0, 0, kind == 1 ? 1 : 0, 1, 0, nullptr, 0, 0 };
+    ConvMShape s;
+    memset(&s, 0, sizeof s);
+    s.C = (int)C; s.D = (int)D; s.H = (int)H; s.W = (int)Wd;
+    s.F = (int)(kind == 1 ? 4 * F : F);
+    s.mode = kind == 1 ? 1 : 0;
+    s.ksplit = 1;
     s.ups = kind == 2 ? 1 : 0;
     if (kind == 2 && ((D | H | Wd) & 1)) return -1;
     const bool thin = conv_ft(s.F) == 32;

@@ -21,7 +21,10 @@ pytestmark = pytest.mark.gpu
                                                     # output-channel group, ragged image sizes, an image wide enough for the
                                                     # 16-round staging variant, and the single-tap form with its 16-channel chunks
                                                     (6, 40, 36, 48, 3, 1, 1), (37, 70, 50, 16, 3, 1, 1), (20, 300, 260, 32, 3, 1, 1),
-                                                    (50, 33, 47, 40, 1, 1, 0), (130, 12, 12, 70, 3, 1, 1)])
+                                                    (50, 33, 47, 40, 1, 1, 0), (130, 12, 12, 70, 3, 1, 1),
+                                                    # the 32-column tiling of wide images: ragged height, widths of one tile, of
+                                                    # whole tiles and with a mostly filled last tile, both channel-group widths
+                                                    (9, 45, 32, 24, 3, 1, 1), (16, 37, 96, 64, 3, 1, 1), (5, 130, 124, 33, 3, 1, 1)])
 def test_conv2d_bias_act_vs_oracle(L, gpu, C_, H, W, F, k, stride, pad):
     rng = np.random.default_rng(0)
     x = rng.standard_normal((C_, H, W)).astype(np.float32)
