@@ -70,7 +70,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     extern __shared__ float4 smem4[];
     float* sW = (float*)smem4;                                    // [2][WCH]
     float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R rounded up to the workgroup size]
-    const int RR = TILE2D ? R2 : s.R;                             // staged elements per channel and kd
+    const int RR = TILE2D ? R2 : KS == 1 ? MT : s.R;              // staged elements per channel and kd (s.R, a constant where it can be)
     const int XCH = CC * KD * RR;
     const int XCHP = (XCH + CM_THREADS - 1) / CM_THREADS * CM_THREADS;
 
