@@ -403,7 +403,9 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                 // matrix-core path for the shapes it takes; narrow outputs stay on the direct kernel
                 static int direct_only = -1;
                 if (direct_only < 0) direct_only = getenv("FORTIS_CONV_DIRECT") != 0;
-                const bool wide = o.F >= 16;
+                // enough output channels to fill a 32-channel MFMA group; a 1 x 1 conv always (it is a plain GEMM over
+                // the pixels whose cost is reading the input once, which the staged kernel does and the direct one does not)
+                const bool wide = o.F >= 16 || (o.kind == OP_CONV2D && o.KH == 1 && o.KW == 1);
                 bool ok = false;
                 int T = 0, tr = 0;
                 if (o.kind == OP_CONV2D) { ok = o.stride == 1 && o.KH == o.KW && (o.KH == 1 || o.KH == 3) && o.pad == o.KH / 2; T = (int)(o.KH * o.KW); }
