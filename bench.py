@@ -353,8 +353,8 @@ def run_zb(L, args, reference_net=False):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20, help="untimed steps first; the clocks need about ten steps of this size to settle")
     ap.add_argument("--workload", default="climsim", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--grid", default=None, help="zb / zb_ref / zb_unfused only: SXxSYxNZ grid instead of the reference's 68x78x15 (zb_unfused: 1028x1028x15)")
