@@ -157,6 +157,10 @@ def test_boundary_pre_post_bit_exact(L, gpu, dtype, NI, NK):
     (12000, 1100, 36, "relu"),     # 846 tiles: whole rounds + a round of halves + quarters
     (16384, 512, 64, None),        # 512 tiles: whole rounds only, no activation
     (257, 385, 4, "leaky"),        # one row / one column past a tile edge, a single 4-wide k slab
+    (70000, 300, 20, "relu"),      # several whole rounds with K below one slab: every tile's only slab runs past K,
+                                   # also when it is fetched ahead as the next tile's first slab
+    (66000, 264, 32, None),        # K of exactly one slab
+    (40000, 384, 76, "leaky"),     # two full slabs and a 12-wide tail, three rounds
 ])
 def test_gemm_schedule_phases(L, gpu, B, N, K, act):
     """The persistent GEMM hands out whole 128 x 128 tiles round by round and cuts the remainder into
