@@ -341,13 +341,47 @@ def run_zb(L, args, reference_net=False):
                        "launches_per_step": 1},
                roofline=roof)
     if not args.no_cpu:
-        from oracle import oracle as O
-        X = O.stencil_gather(gd, garr, int(gt.count), int(gt.nk), 3, 3, 64)
-        case = dict(net, rows=rows)
-        out["cpu_baseline"] = cpu_baseline_mlp(case, rows, X, min_seconds=5.0, **extra)
-        out["cpu_baseline"]["sample"] += " (MLP part only; the gather and scatter loops of the host are not included)"
+        ref = cpu_baseline_zb_reference() if (reference_net and not args.grid) else None
+        if ref:
+            out["cpu_baseline"] = ref
+        else:
+            from oracle import oracle as O
+            X = O.stencil_gather(gd, garr, int(gt.count), int(gt.nk), 3, 3, 64)
+            case = dict(net, rows=rows)
+            out["cpu_baseline"] = cpu_baseline_mlp(case, rows, X, min_seconds=5.0, **extra)
+            out["cpu_baseline"]["sample"] += " (MLP part only; the gather and scatter loops of the host are not included)"
     plan.close()
     return out
+
+
+def cpu_baseline_zb_reference(min_seconds=10.0):
+    """The reference's own CPU path for this very step: its native Fortran host (mom6_zb/zb_host.f90 with
+    fwd_native_zb.f90, compiled unchanged by oracle/build_ref.sh) on the reference geometry and network,
+    which times 10 steps itself ('per-step ms').  Single-threaded, as the reference runs it.  None if the
+    binary was not built."""
+    import re
+    import subprocess
+    import tempfile
+    exe = os.path.join(ROOT, "oracle", "_ref", "zb_native4")
+    if not os.path.exists(exe):
+        return None
+    W = np.load(os.path.join(ROOT, "tests", "golden", "zb_nn.npz"))
+    ms, runs, t0 = [], 0, time.perf_counter()
+    with tempfile.TemporaryDirectory() as td:
+        with open(os.path.join(td, "zb_nn.bin"), "wb") as o:      # layout of mom6_zb/make_zb_weights.py:12-17
+            for a in (W["A0"].T, W["b0"], W["A1"].T, W["b1"], W["in_norms"], W["out_norms"]):
+                o.write(np.ascontiguousarray(a, dtype=np.float32).tobytes())
+        while time.perf_counter() - t0 < min_seconds:
+            r = subprocess.run([exe], cwd=td, capture_output=True, text=True, timeout=120)
+            m = re.search(r"per-step ms:\s*([-0-9.Ee+]+)", r.stdout)
+            if r.returncode != 0 or not m:
+                return None
+            ms.append(float(m.group(1)))
+            runs += 1
+    per_step = float(np.median(ms))
+    return {"value": 71040 / (per_step * 1e-3), "unit": "columns/s", "cores": 1, "kind": "reference",
+            "sample": "%d runs of the reference's native Fortran ZB host (zb_host.f90 + fwd_native_zb.f90, flang -O2), each timing 10 whole "
+                      "steps (stencil packing, 27->20->3 forward, de-scaling and stores on 71040 cells); median %.2f ms per step" % (runs, per_step)}
 
 
 def main():
