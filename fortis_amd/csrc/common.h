@@ -93,6 +93,7 @@ struct ConvEpi {
     int act;
     float alpha;
     const float* res;    // residual tensor added after the activation (same shape as output), or null
+    float* pool;         // conv2d only: also receives the 2 x 2 stride-2 max pool of the output (H, W even), or null
 };
 int fortis_launch_conv2d(const float* x, const float* w, float* y, long C, long H, long Wd, long F, long KH,
                          long KW, long Ho, long Wo, long sh, long sw, long ph, long pw, const ConvEpi& e,

@@ -273,6 +273,40 @@ __global__ void conv_split_reduce_kernel(const float* __restrict__ part, float* 
     y[idx] = v;
 }
 
+// The same for a 2-D conv whose output also goes through a 2 x 2 stride-2 max pool: a thread owns one pooled
+// position, i.e. a 2 x 2 block of the output, writes its four values and their maximum.
+__global__ void conv_split_reduce_pool_kernel(const float* __restrict__ part, float* __restrict__ y, float* __restrict__ pool,
+                                              int F, int H, int W, long osize, int ksplit, ConvEpi e)
+{
+    const int Ho = H / 2, Wo = W / 2;
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long)F * Ho * Wo) return;
+    const int xo = (int)(idx % Wo), yo = (int)((idx / Wo) % Ho);
+    const long f = idx / ((long)Wo * Ho);
+    const float sc = e.scale ? e.scale[f] : 1.f, sf = e.shift ? e.shift[f] : 0.f;
+    float m = -INFINITY;
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        const long row = (f * H + 2 * yo + a) * W + 2 * xo;        // even: the pair is 8-byte aligned
+        float2 v = *(const float2*)(part + row);
+        for (int k = 1; k < ksplit; k++) { const float2 q = *(const float2*)(part + k * osize + row); v.x += q.x; v.y += q.y; }
+        float o[2] = { v.x, v.y };
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            float t = o[b];
+            if (e.scale) t = t * sc;
+            if (e.shift) t = t + sf;
+            if (e.act == FORTIS_ACT_RELU) t = t > 0.f ? t : 0.f;
+            else if (e.act == FORTIS_ACT_LEAKY) t = t > 0.f ? t : e.alpha * t;
+            if (e.res) t = t + e.res[row + b];
+            o[b] = t;
+            m = t > m ? t : m;
+        }
+        *(float2*)(y + row) = make_float2(o[0], o[1]);
+    }
+    pool[idx] = m;
+}
+
 // ---- host side ---------------------------------------------------------------------------------------
 static inline long conv_ft(long Fg) { return Fg <= 32 ? 32 : 64; }
 static int conv_cus()
@@ -375,10 +409,19 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);
     hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
     HIP_OK(hipGetLastError());
-    if (s.ksplit > 1) {
+    const bool pooled = e.pool != nullptr;
+    if (pooled && (s.mode || s.D != 1 || (s.H & 1) || (s.W & 1) || (((uintptr_t)y | (uintptr_t)s.part) & 7))) return -1;   // the plan only asks for it on 2-D convs
+    if (s.ksplit > 1 && pooled) {
+        const long n = (long)s.F * (s.H / 2) * (s.W / 2);
+        hipLaunchKernelGGL(conv_split_reduce_pool_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, st, s.part, y, e.pool, s.F, s.H, s.W,
+                           s.osize, s.ksplit, e);
+        HIP_OK(hipGetLastError());
+    } else if (s.ksplit > 1) {
         hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)cdiv(s.osize, 256)), dim3(256), 0, st, s.part, y, s.osize,
                            ospatial, s.ksplit, e);
         HIP_OK(hipGetLastError());
+    } else if (pooled) {
+        fortis_launch_maxpool2d(y, e.pool, s.F, s.H, s.W, 2, st);
     }
     return 0;
 }

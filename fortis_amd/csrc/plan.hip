@@ -39,6 +39,7 @@ struct Exec {
     const Op* op = nullptr;
     ConvEpi epi = { nullptr, nullptr, 0, 0.f, nullptr };
     const float* Wmfma = nullptr;   // weights packed for the MFMA implicit-GEMM kernel, when the shape qualifies
+    int pool_dst = -1;              // conv2d: tensor that receives the 2 x 2 max pool folded into this conv
 };
 
 struct fortis_plan {
@@ -416,6 +417,17 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                     p->owned.push_back(wp);
                     ex.Wmfma = wp;
                 }
+                // A 2 x 2 max pool that directly follows and reads this conv's whole output is written by the conv's
+                // own last stage (the reduce of a channel-split launch, else a pool launch from the conv launcher).
+                if (o.kind == OP_CONV2D && ex.Wmfma && i + 1 < ops.size() && ops[i + 1].kind == OP_MAXPOOL && ops[i + 1].src == o.dst &&
+                    ops[i + 1].KH == 2 && ops[i + 1].C == o.F && ops[i + 1].H == o.H && ops[i + 1].W == o.W && o.coff == 0 &&
+                    (o.ctot == 0 || o.ctot == o.F) && !(o.H & 1) && !(o.W & 1) && ops[i + 1].dst != o.dst) {
+                    ex.pool_dst = ops[i + 1].dst;
+                    p->exec.push_back(ex);
+                    p->exec_skip++;
+                    i += adv + 1;
+                    continue;
+                }
                 break;
             }
             case OP_MAXPOOL: ex.kind = EX_MAXPOOL; break;
@@ -477,10 +489,14 @@ void fortis_plan_run(fortis_plan* p)
             case EX_POST: fortis_launch_boundary_post(src, p->tptr[e.dst], e.rows, e.N, e.p0, e.flag, s); break;
             case EX_CONV2D: {
                 const long Ho = (o->H + 2 * o->pad - o->KH) / o->stride + 1, Wo = (o->W + 2 * o->pad - o->KW) / o->stride + 1;
-                rc = e.Wmfma ? fortis_launch_conv_mfma(src, e.Wmfma, dst + o->coff * Ho * Wo, o->C, 1, o->H, o->W, o->F, 1, (int)o->KH, 0, e.epi, s) : -1;
-                if (rc != 0)
+                ConvEpi epi = e.epi;
+                epi.pool = e.pool_dst >= 0 ? (float*)p->tptr[e.pool_dst] : nullptr;
+                rc = e.Wmfma ? fortis_launch_conv_mfma(src, e.Wmfma, dst + o->coff * Ho * Wo, o->C, 1, o->H, o->W, o->F, 1, (int)o->KH, 0, epi, s) : -1;
+                if (rc != 0) {
                     rc = fortis_launch_conv2d(src, e.W, dst, o->C, o->H, o->W, o->F, o->KH, o->KW, Ho, Wo, o->stride, o->stride,
                                               o->pad, o->pad, e.epi, o->coff, o->ctot, s);
+                    if (rc == 0 && epi.pool) fortis_launch_maxpool2d(dst, epi.pool, o->F, Ho, Wo, 2, s);
+                }
                 break;
             }
             case EX_CONVT2D: {
