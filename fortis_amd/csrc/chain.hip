@@ -275,6 +275,7 @@ void chain_wave_kernel(ChainParams params)
     const gfloat* out_mul = st_g(d.out_mul);
     const bool g_uniform = STENCIL && st_u(g.uniform) != 0;
     const bool s_uniform = STENCIL && st_u(sc.uniform) != 0;
+    const bool s_refs_uniform = STENCIL && st_u(sc.refs_uniform) != 0;     // one store offset per cell
     // gather and scatter usually visit the same cells in the same order: decode a row once
     const bool same_cells = STENCIL && st_u((int)(g.count == sc.count && g.ni == sc.ni && g.ilo == sc.ilo && g.jlo == sc.jlo &&
                                                   g.sx == sc.sx && g.cells == sc.cells)) != 0;
@@ -436,7 +437,7 @@ void chain_wave_kernel(ChainParams params)
                     const int n = nt * 16 + 4 * lq + r;
                     if (valid && n < NO) {
                         const StSlotT<float*> sl = sc.refs[n];
-                        st_g(sl.p)[s_uniform ? soff : st_off(sl, in.si, in.sj, in.skk)] = ov[r];
+                        st_g(sl.p)[s_refs_uniform ? soff : st_off(sl, in.si, in.sj, in.skk)] = ov[r];
                     }
                 }
             }

@@ -68,7 +68,8 @@ struct alignas(16) StencilArgsT {
     const int* cells;
     StMagic mcount, mni, msx;   // exact division by count, ni, sx
     int uniform;                // every slot and scalar has the same (si, sj, plane): one offset per cell
-    int pad_[3];
+    int refs_uniform;           // every slot does (the scalars may differ, e.g. a 2-D plane among 3-D arrays)
+    int pad_[2];
 };
 typedef StencilArgsT<const float*> GatherArgs;
 typedef StencilArgsT<float*> ScatterArgs;
@@ -218,6 +219,7 @@ static inline void st_make_args(const StencilDev& low, const int* dcells, P cons
     a->uniform = 1;
     for (int r = 0; r < low.nrefs; r++)
         if (a->refs[r].si != a->refs[0].si || a->refs[r].sj != a->refs[0].sj || a->refs[r].plane != a->refs[0].plane) a->uniform = 0;
+    a->refs_uniform = a->uniform;
     for (int r = 0; r < low.nscal; r++)
         if (a->scal[r].si != a->refs[0].si || a->scal[r].sj != a->refs[0].sj || a->scal[r].plane != a->refs[0].plane) a->uniform = 0;
 }
