@@ -109,6 +109,12 @@ int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long 
 float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats);
 int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, long D, long H, long Wd, long F, int KD,
                             int KS, int kind, const ConvEpi& e, hipStream_t s);
+// Partial sums of a conv whose input channels are split over workgroups: the library's one buffer for them
+// (grown on demand, null when the device has no memory left) and the kernel that adds ksplit slices of
+// osize floats and applies the epilogue.
+float* fortis_conv_split_scratch(size_t bytes);
+int fortis_launch_conv_split_reduce(const float* part, float* y, long osize, long ospatial, int ksplit, const ConvEpi& e,
+                                    hipStream_t s);
 void fortis_launch_maxpool2d(const float* x, float* y, long C, long H, long Wd, long k, hipStream_t s);
 void fortis_launch_upsample(const float* x, float* y, long C, long D, long H, long Wd, long sfac, int nd, hipStream_t s);
 void fortis_launch_concat_copy(const float* x, float* y, long C, long S, long coff, hipStream_t s);

@@ -115,72 +115,76 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_direct_kernel(const float* 
 
 // 3x3x3, stride 1, pad 1 convolution with at most CT_F output channels (image-space heads such as
 // 64 -> 3): the matrix cores would multiply 32-row tiles that are nine tenths padding, so this one runs on
-// the vector ALUs, which have the same fp32 peak on this part.
+// the vector ALUs.
 // Positions of one z-plane are linearised with pitch P = W + 1 (tap (kh, kw) of position m is element
 // m + kh*P + kw of the zero-padded plane, a lane-independent offset).  A workgroup takes CT_MT positions,
 // a thread CT_PT consecutive ones times all output channels in registers; per chunk of CT_CC input
-// channels the three z-planes' runs are staged in LDS (double buffered through registers), and the
-// chunk's weights [channel][tap][output channel] next to them; a weight read has the same address in
-// every lane (LDS broadcast) and fetches one tap for all output channels.
+// channels the three z-planes' runs are staged in LDS (double buffered through registers).  A weight has
+// the same address in every lane, so the weights are read through the scalar cache into scalar registers
+// (LDS broadcast reads of them took more LDS time than the inputs).  With few workgroups per compute unit
+// the input channels are split over blockIdx.y and a reduce kernel adds the slices.
 #define CT_F 4
 #define CT_PT 2
 #define CT_MT (CONV_THREADS * CT_PT)
 #define CT_CC 2
-#define CT_NX 16     // staged elements per thread per chunk, at most
+#define CT_NR 3      // staging rounds of a (channel, z-plane) run: it has at most CT_NR * CONV_THREADS elements
 
 template <int NF>      // output channels computed: 3 (F <= 3) or 4
 __global__ __launch_bounds__(CONV_THREADS) void conv3d_thin_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                                    float* __restrict__ y, int C, int D, int H, int W, int F,
-                                                                   int P, int plane, int tiles, int R, ConvEpi e)
+                                                                   int P, int plane, int tiles, int R, int cps, ConvEpi e)
 {
-    extern __shared__ float ct_lds[];                       // [2][CT_CC][3][R] inputs, then [2][CT_CC][27][CT_F] weights
+    // blockIdx.y: slice of the input channels (cps chunks each); with more than one slice, slice k writes
+    // its raw sums to y + k * F*D*H*W and a reduce kernel applies the epilogue
+    extern __shared__ float ct_lds[];                       // [2][CT_CC][3][R] inputs
     const int tid = threadIdx.x;
     const int z = blockIdx.x / tiles, tile = blockIdx.x - z * tiles;
     const int m0 = tile * CT_MT;
     const long HW = (long)H * W, chan = (long)D * HW;
     const int XCH = CT_CC * 3 * R;
 
-    // staging map (the same for every chunk): offset of the element inside a CT_CC-channel group, or -1
-    int goff[CT_NX];
+    // staging map: every (channel, z-plane) run of a chunk holds the same R pixels, so a thread keeps the
+    // in-plane offset of pixel tid + j * CONV_THREADS (or -1 outside the image) and the run's base is uniform
+    unsigned poff[CT_NR];       // byte offset inside the plane (0 for padding)
+    bool pin[CT_NR];            // inside the image
 #pragma unroll
-    for (int i = 0; i < CT_NX; i++) {
-        const int el = tid + i * CONV_THREADS;
-        goff[i] = -1;
-        if (el < XCH) {
-            const int c = el / (3 * R), rem = el - c * (3 * R), kd = rem / R, r = rem - kd * R;
-            const int v = m0 + r, yp = v / P, xp = v - yp * P;
-            const int zz = z + kd - 1, yy = yp - 1, xx = xp - 1;
-            if (zz >= 0 && zz < D && yy >= 0 && yy < H && xx >= 0 && xx < W)
-                goff[i] = (int)(c * chan + zz * HW + (long)yy * W + xx);
-        }
+    for (int j = 0; j < CT_NR; j++) {
+        const int r = tid + j * CONV_THREADS;
+        const int v = m0 + r, yp = v / P, xp = v - yp * P;
+        const int yy = yp - 1, xx = xp - 1;
+        pin[j] = r < R && yy >= 0 && yy < H && xx >= 0 && xx < W;
+        poff[j] = pin[j] ? (unsigned)(yy * W + xx) * 4u : 0u;
     }
-    float rx[CT_NX];
-    float rwt = 0.f;
-    float* wl = ct_lds + 2 * XCH;
-    // weight element this thread stages: (cc, tap, f) -> w[f][c][tap]
-    const int wcc = tid / (27 * CT_F), wtap = (tid / CT_F) % 27, wf = tid % CT_F;
-    auto load_chunk = [&](int ch) __attribute__((always_inline)) {
-        if (tid < CT_CC * 27 * CT_F) {
-            const int c = ch * CT_CC + wcc;
-            rwt = (wf < F && c < C) ? w[((long)wf * C + c) * 27 + wtap] : 0.f;
-        }
-        const float* xsrc = x + (long)ch * CT_CC * chan;
-#pragma unroll
-        for (int i = 0; i < CT_NX; i++) {
-            const int el = tid + i * CONV_THREADS;
-            const bool ok = goff[i] >= 0 && ch * CT_CC + el / (3 * R) < C;
-            const float v = xsrc[ok ? goff[i] : 0];
-            rx[i] = ok ? v : 0.f;
-        }
+    float rx[CT_CC * 3][CT_NR];
+    // run (cc, kd) of chunk ch lies inside the tensor
+    auto run_ok = [&](int ch, int cc, int kd) __attribute__((always_inline)) {
+        const int zz = z + kd - 1;
+        return ch * CT_CC + cc < C && zz >= 0 && zz < D;
     };
-    auto store_chunk = [&](int buf) __attribute__((always_inline)) {
-        if (tid < CT_CC * 27 * CT_F) wl[buf * CT_CC * 27 * CT_F + tid] = rwt;
+    auto load_chunk = [&](int ch) __attribute__((always_inline)) {
+#pragma unroll
+        for (int cc = 0; cc < CT_CC; cc++)
+#pragma unroll
+            for (int kd = 0; kd < 3; kd++) {
+                // runs outside the tensor read the tensor's first plane and are zeroed when stored
+                const char* src = (const char*)(run_ok(ch, cc, kd) ? x + (long)(ch * CT_CC + cc) * chan + (long)(z + kd - 1) * HW : x);
+#pragma unroll
+                for (int j = 0; j < CT_NR; j++) rx[cc * 3 + kd][j] = *(const float*)(src + poff[j]);
+            }
+    };
+    auto store_chunk = [&](int buf, int ch) __attribute__((always_inline)) {
         float* dst = ct_lds + buf * XCH;
 #pragma unroll
-        for (int i = 0; i < CT_NX; i++) {
-            const int el = tid + i * CONV_THREADS;
-            if (el < XCH) dst[el] = rx[i];
-        }
+        for (int cc = 0; cc < CT_CC; cc++)
+#pragma unroll
+            for (int kd = 0; kd < 3; kd++) {
+                const bool ok = run_ok(ch, cc, kd);
+#pragma unroll
+                for (int j = 0; j < CT_NR; j++) {
+                    const int r = tid + j * CONV_THREADS;
+                    if (r < R) dst[(cc * 3 + kd) * R + r] = (ok && pin[j]) ? rx[cc * 3 + kd][j] : 0.f;
+                }
+            }
     };
 
     float acc[NF][CT_PT];
@@ -189,12 +193,13 @@ __global__ __launch_bounds__(CONV_THREADS) void conv3d_thin_kernel(const float* 
 #pragma unroll
         for (int p = 0; p < CT_PT; p++) acc[f][p] = 0.f;
 
-    const int nchunks = (C + CT_CC - 1) / CT_CC;
-    load_chunk(0);
-    store_chunk(0);
+    const int nall = (C + CT_CC - 1) / CT_CC;
+    const int ch0 = blockIdx.y * cps, nchunks = ch0 + cps < nall ? ch0 + cps : nall;
+    load_chunk(ch0);
+    store_chunk(0, ch0);
     __syncthreads();
-    for (int ch = 0; ch < nchunks; ch++) {
-        const int buf = ch & 1;
+    for (int ch = ch0; ch < nchunks; ch++) {
+        const int buf = (ch - ch0) & 1;
         if (ch + 1 < nchunks) load_chunk(ch + 1);
         const float* xs = ct_lds + buf * XCH + tid * CT_PT;
 #pragma unroll
@@ -202,25 +207,33 @@ __global__ __launch_bounds__(CONV_THREADS) void conv3d_thin_kernel(const float* 
             const int c = ch * CT_CC + cc;
             if (c >= C) break;
 #pragma unroll
-            for (int kd = 0; kd < 3; kd++)
+            for (int kd = 0; kd < 3; kd++) {
+                // the plane's nine weights of every output channel: the address is the same in all lanes, so they
+                // come through the scalar cache into scalar registers and cost no LDS or vector traffic
+                // (channels beyond F repeat the last one; their sums are not stored)
+                float wk[NF][9];
+#pragma unroll
+                for (int f = 0; f < NF; f++) {
+                    const float* wr = w + ((long)(f < F ? f : F - 1) * C + c) * 27 + kd * 9;
+#pragma unroll
+                    for (int t = 0; t < 9; t++) wk[f][t] = wr[t];
+                }
 #pragma unroll
                 for (int kh = 0; kh < 3; kh++) {
                     float in[CT_PT + 2];
                     const float* row = xs + (cc * 3 + kd) * R + kh * P;
 #pragma unroll
                     for (int t = 0; t < CT_PT + 2; t++) in[t] = row[t];
-                    // the three taps' weights for all output channels: same address in every lane (LDS broadcast)
-                    const float4* wt = (const float4*)(wl + ((buf * CT_CC + cc) * 27 + (kd * 3 + kh) * 3) * CT_F);
-                    const float4 w0 = wt[0], w1 = wt[1], w2 = wt[2];
-                    const float wa[3][CT_F] = { { w0.x, w0.y, w0.z, w0.w }, { w1.x, w1.y, w1.z, w1.w }, { w2.x, w2.y, w2.z, w2.w } };
 #pragma unroll
                     for (int f = 0; f < NF; f++)
 #pragma unroll
                         for (int p = 0; p < CT_PT; p++)
-                            acc[f][p] = fmaf(in[p + 2], wa[2][f], fmaf(in[p + 1], wa[1][f], fmaf(in[p], wa[0][f], acc[f][p])));
+                            acc[f][p] = fmaf(in[p + 2], wk[f][kh * 3 + 2],
+                                             fmaf(in[p + 1], wk[f][kh * 3 + 1], fmaf(in[p], wk[f][kh * 3], acc[f][p])));
                 }
+            }
         }
-        if (ch + 1 < nchunks) store_chunk(buf ^ 1);
+        if (ch + 1 < nchunks) store_chunk(buf ^ 1, ch + 1);
         __syncthreads();
     }
 #pragma unroll
@@ -230,9 +243,16 @@ __global__ __launch_bounds__(CONV_THREADS) void conv3d_thin_kernel(const float* 
         const int yy = m / P, xx = m - yy * P;
         if (xx >= W) continue;
         const long opos = ((long)z * H + yy) * W + xx;
+        if (gridDim.y > 1) {
+            float* part = y + (long)blockIdx.y * F * chan;
 #pragma unroll
-        for (int f = 0; f < NF; f++)
-            if (f < F) y[f * chan + opos] = conv_epilogue(acc[f][p], f, opos, chan, e);
+            for (int f = 0; f < NF; f++)
+                if (f < F) part[f * chan + opos] = acc[f][p];
+        } else {
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+                if (f < F) y[f * chan + opos] = conv_epilogue(acc[f][p], f, opos, chan, e);
+        }
     }
 }
 
@@ -326,6 +346,16 @@ static void launch_direct(const float* x, const float* w, float* y, const ConvSh
     }
 }
 
+static int thin_cus()
+{
+    static int cus = 0;
+    if (!cus) {
+        hipDeviceProp_t prop;
+        cus = hipGetDeviceProperties(&prop, 0) == hipSuccess ? prop.multiProcessorCount : 256;
+    }
+    return cus;
+}
+
 int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long D, long H, long Wd, long F, long KD,
                          long KH, long KW, long Do, long Ho, long Wo, long pd, long ph, long pw, const ConvEpi& e,
                          hipStream_t s)
@@ -334,21 +364,36 @@ int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long 
     if (Do != D + 2 * pd - KD + 1 || Ho != H + 2 * ph - KH + 1 || Wo != Wd + 2 * pw - KW + 1) return -1;
     if (KD == 3 && KH == 3 && KW == 3 && pd == 1 && ph == 1 && pw == 1 && F <= CT_F) {
         const int P = (int)Wd + 1, plane = (int)H * P, tiles = (int)cdiv(plane, CT_MT), R = CT_MT + 2 * P + 2;
-        const size_t shmem = (size_t)2 * (CT_CC * 3 * R + CT_CC * 27 * CT_F) * sizeof(float);
-        if ((long)CT_CC * 3 * R <= (long)CONV_THREADS * CT_NX && shmem <= 160 * 1024) {
+        const size_t shmem = (size_t)2 * CT_CC * 3 * R * sizeof(float);
+        if (R <= CONV_THREADS * CT_NR && shmem <= 160 * 1024) {
             static size_t attr = 0;
             if (shmem > attr) {
                 HIP_OK(hipFuncSetAttribute((const void*)conv3d_thin_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
                 HIP_OK(hipFuncSetAttribute((const void*)conv3d_thin_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
                 attr = shmem;
             }
+            // a workgroup's chunks run one after another, each waiting for its loads: with few workgroups
+            // per compute unit the input channels are split so that about eight are in flight on each
+            const int nall = (int)cdiv(C, CT_CC);
+            int ksplit = 1;
+            while (ksplit < 8 && D * tiles * ksplit < 8L * thin_cus() && nall / (ksplit * 2) >= 4) ksplit *= 2;
+            const int cps = (int)cdiv(nall, ksplit);
+            ksplit = (int)cdiv(nall, cps);
+            const long osize = F * D * H * Wd;
+            float* dst = y;
+            if (ksplit > 1) {
+                dst = fortis_conv_split_scratch((size_t)ksplit * osize * sizeof(float));
+                if (!dst) return -1;
+            }
+            const dim3 grid((unsigned)(D * tiles), (unsigned)ksplit);
             if (F <= 3)
-                hipLaunchKernelGGL(conv3d_thin_kernel<3>, dim3((unsigned)(D * tiles)), dim3(CONV_THREADS), shmem, s, x, w, y, (int)C,
-                                   (int)D, (int)H, (int)Wd, (int)F, P, plane, tiles, R, e);
+                hipLaunchKernelGGL(conv3d_thin_kernel<3>, grid, dim3(CONV_THREADS), shmem, s, x, w, dst, (int)C, (int)D, (int)H,
+                                   (int)Wd, (int)F, P, plane, tiles, R, cps, e);
             else
-                hipLaunchKernelGGL(conv3d_thin_kernel<4>, dim3((unsigned)(D * tiles)), dim3(CONV_THREADS), shmem, s, x, w, y, (int)C,
-                                   (int)D, (int)H, (int)Wd, (int)F, P, plane, tiles, R, e);
+                hipLaunchKernelGGL(conv3d_thin_kernel<4>, grid, dim3(CONV_THREADS), shmem, s, x, w, dst, (int)C, (int)D, (int)H,
+                                   (int)Wd, (int)F, P, plane, tiles, R, cps, e);
             HIP_OK(hipGetLastError());
+            if (ksplit > 1) return fortis_launch_conv_split_reduce(dst, y, osize, D * H * Wd, ksplit, e, s);
             return 0;
         }
     }

@@ -322,7 +322,7 @@ static int conv_cus()
 // Partial sums of channel-split launches: one buffer for every shape (launches on the library's stream run
 // one after the other).  It grows on the first, eager run of a plan; replays and captured runs find it in
 // place.  An outgrown buffer stays allocated: a graph captured earlier may still name it.
-static float* conv_split_scratch(size_t need)
+float* fortis_conv_split_scratch(size_t need)
 {
     static float* scratch = nullptr;
     static size_t cap = 0;
@@ -333,6 +333,15 @@ static float* conv_split_scratch(size_t need)
         cap = need;
     }
     return scratch;
+}
+
+int fortis_launch_conv_split_reduce(const float* part, float* y, long osize, long ospatial, int ksplit, const ConvEpi& e,
+                                    hipStream_t st)
+{
+    hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)cdiv(osize, 256)), dim3(256), 0, st, part, y, osize, ospatial,
+                       ksplit, e);
+    HIP_OK(hipGetLastError());
+    return 0;
 }
 
 // Packs conv weights W[F][C][T] (T taps, row-major) into the kernel's order
@@ -403,7 +412,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     const long ospatial = (long)s.D * s.H * s.W * (s.mode ? 4 : 1);
     s.osize = (long)(s.mode ? s.F / 4 : s.F) * ospatial;
     if (s.ksplit > 1) {
-        s.part = conv_split_scratch((size_t)s.ksplit * s.osize * sizeof(float));
+        s.part = fortis_conv_split_scratch((size_t)s.ksplit * s.osize * sizeof(float));
         if (!s.part) return -1;
     }
     dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);

@@ -130,7 +130,10 @@ def test_op_micro_suite(L, gpu):
                                                (64, 9, 9, 9, 64, 3, 1), (5, 6, 6, 6, 10, 1, 0), (3, 8, 8, 8, 4, 3, 0),
                                                # matrix-core path: odd channel count (partial 2-channel chunk), ragged extents,
                                                # a partial output-channel group; a volume whose rows need the 16-round staging
-                                               (7, 12, 11, 10, 20, 3, 1), (6, 5, 90, 70, 80, 3, 1)])
+                                               (7, 12, 11, 10, 20, 3, 1), (6, 5, 90, 70, 80, 3, 1),
+                                               # image-space heads (at most 4 output channels) whose input channels are split
+                                               # over workgroups: even slices, and an odd channel count with a shorter last slice
+                                               (32, 8, 20, 20, 3, 3, 1), (17, 6, 10, 12, 4, 3, 1), (64, 5, 30, 33, 1, 3, 1)])
 def test_conv3d_bias_act_residual_vs_oracle(L, gpu, C_, D, H, W, F, k, pad):
     rng = np.random.default_rng(1)
     x = rng.standard_normal((C_, D, H, W)).astype(np.float32)
