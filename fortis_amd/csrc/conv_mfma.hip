@@ -256,21 +256,58 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
 }
 
 // Sums the partial results of a channel-split launch in split order (deterministic) and applies the
-// epilogue.  ospatial = elements per output channel.
+// epilogue.  ospatial = elements per output channel.  V = 4: a thread takes four consecutive elements of one
+// channel (ospatial a multiple of 4, all pointers 16-byte aligned).
+template <int V>
 __global__ void conv_split_reduce_kernel(const float* __restrict__ part, float* __restrict__ y, long osize, long ospatial,
                                          int ksplit, ConvEpi e)
 {
-    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long idx = ((long)blockIdx.x * blockDim.x + threadIdx.x) * V;
     if (idx >= osize) return;
-    float v = part[idx];
-    for (int k = 1; k < ksplit; k++) v += part[k * osize + idx];
+    float v[V];
+    if constexpr (V == 4) {
+        float4 a = *(const float4*)(part + idx);
+        for (int k = 1; k < ksplit; k++) {
+            const float4 q = *(const float4*)(part + k * osize + idx);
+            a.x += q.x; a.y += q.y; a.z += q.z; a.w += q.w;
+        }
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    } else {
+        v[0] = part[idx];
+        for (int k = 1; k < ksplit; k++) v[0] += part[k * osize + idx];
+    }
     const long fo = idx / ospatial;
-    if (e.scale) v = v * e.scale[fo];
-    if (e.shift) v = v + e.shift[fo];
-    if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
-    else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
-    if (e.res) v = v + e.res[idx];
-    y[idx] = v;
+    const float sc = e.scale ? e.scale[fo] : 1.f, sf = e.shift ? e.shift[fo] : 0.f;
+    float r[V];
+    if constexpr (V == 4) {
+        const float4 q = e.res ? *(const float4*)(e.res + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+        r[0] = q.x; r[1] = q.y; r[2] = q.z; r[3] = q.w;
+    } else {
+        r[0] = e.res ? e.res[idx] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        float t = v[i];
+        if (e.scale) t = t * sc;
+        if (e.shift) t = t + sf;
+        if (e.act == FORTIS_ACT_RELU) t = t > 0.f ? t : 0.f;
+        else if (e.act == FORTIS_ACT_LEAKY) t = t > 0.f ? t : e.alpha * t;
+        if (e.res) t = t + r[i];
+        v[i] = t;
+    }
+    if constexpr (V == 4) *(float4*)(y + idx) = make_float4(v[0], v[1], v[2], v[3]);
+    else y[idx] = v[0];
+}
+
+static void launch_split_reduce(const float* part, float* y, long osize, long ospatial, int ksplit, const ConvEpi& e, hipStream_t st)
+{
+    const bool v4 = ospatial % 4 == 0 && (((uintptr_t)part | (uintptr_t)y | (uintptr_t)e.res) & 15) == 0;
+    if (v4)
+        hipLaunchKernelGGL(conv_split_reduce_kernel<4>, dim3((unsigned)cdiv(osize / 4, 256)), dim3(256), 0, st, part, y, osize,
+                           ospatial, ksplit, e);
+    else
+        hipLaunchKernelGGL(conv_split_reduce_kernel<1>, dim3((unsigned)cdiv(osize, 256)), dim3(256), 0, st, part, y, osize, ospatial,
+                           ksplit, e);
 }
 
 // The same for a 2-D conv whose output also goes through a 2 x 2 stride-2 max pool: a thread owns one pooled
@@ -338,8 +375,7 @@ float* fortis_conv_split_scratch(size_t need)
 int fortis_launch_conv_split_reduce(const float* part, float* y, long osize, long ospatial, int ksplit, const ConvEpi& e,
                                     hipStream_t st)
 {
-    hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)cdiv(osize, 256)), dim3(256), 0, st, part, y, osize, ospatial,
-                       ksplit, e);
+    launch_split_reduce(part, y, osize, ospatial, ksplit, e, st);
     HIP_OK(hipGetLastError());
     return 0;
 }
@@ -426,8 +462,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
                            s.osize, s.ksplit, e);
         HIP_OK(hipGetLastError());
     } else if (s.ksplit > 1) {
-        hipLaunchKernelGGL(conv_split_reduce_kernel, dim3((unsigned)cdiv(s.osize, 256)), dim3(256), 0, st, s.part, y, s.osize,
-                           ospatial, s.ksplit, e);
+        launch_split_reduce(s.part, y, s.osize, ospatial, s.ksplit, e, st);
         HIP_OK(hipGetLastError());
     } else if (pooled) {
         fortis_launch_maxpool2d(y, e.pool, s.F, s.H, s.W, 2, st);
