@@ -484,6 +484,12 @@ static int launch(const float* x, const float* wp, float* y, ConvMShape s, const
     }
     const long R = MT + (KS == 3 ? 2 * s.P + 2 : 0), xch = (long)cm_cc(KD * KS * KS) * KD * R;
     if (xch > (long)CM_THREADS * CM_NXMAX) return -1;     // run too long to stage
+    if constexpr (KD == 3 && MT == 128) {
+        // volumes: the staging rounds are paid for in matrix time, so the common widths get their exact count
+        if (xch <= CM_THREADS * 5) return launch_nx<KD, KS, MT, FT, 5, false>(x, wp, y, s, e, st);
+        if (xch <= CM_THREADS * 6) return launch_nx<KD, KS, MT, FT, 6, false>(x, wp, y, s, e, st);
+        if (xch <= CM_THREADS * 7) return launch_nx<KD, KS, MT, FT, 7, false>(x, wp, y, s, e, st);
+    }
     return xch <= CM_THREADS * 8 ? launch_nx<KD, KS, MT, FT, 8, false>(x, wp, y, s, e, st) : launch_nx<KD, KS, MT, FT, 16, false>(x, wp, y, s, e, st);
 }
 
