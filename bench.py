@@ -139,8 +139,15 @@ def run_zb_unfused(L, args):
     from fortis_amd import configs, plan as P, stencil as S
     sx, sy, nz = (int(v) for v in (args.grid or "1028x1028x15").lower().split("x"))
     gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    # --f64: every host array is double precision (an E3SM-style host), which takes the general stencil
+    # kernels (typed expression evaluation) instead of the fp32 form
+    esz, ft = (8, np.float64) if args.f64 else (4, np.float32)
+    if args.f64:
+        for d in (gd, sd):
+            for a in d["arrays"]:
+                a["elt"] = "f64"
     gt, st = S.build_table(gd, lp, kd, "gather"), S.build_table(sd, lp, kd, "scatter")
-    A = configs.zb_arrays(sx, sy, nz)
+    A = {k: np.ascontiguousarray(v, dtype=ft) for k, v in configs.zb_arrays(sx, sy, nz).items()}
     rows, count, n3 = gt.count * gt.nk, int(gt.count), sx * sy * nz
     net = configs.zb_mlp()
     plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows)
@@ -150,7 +157,7 @@ def run_zb_unfused(L, args):
         L.fortis_h2d(d, a.ctypes.data, a.nbytes)
         return d
     dG = (C.c_void_p * 4)(*[dev(A[k]) for k in ("sh_xy_h", "sh_xx", "vort_xy_h", "norm_h")])
-    dS = (C.c_void_p * 5)(dG[3], dev(A["kappa_h"]), dev(np.zeros(sx * sy, np.float32)), dev(np.zeros(n3, np.float32)), dev(np.zeros(n3, np.float32)))
+    dS = (C.c_void_p * 5)(dG[3], dev(A["kappa_h"]), dev(np.zeros(sx * sy, ft)), dev(np.zeros(n3, ft)), dev(np.zeros(n3, ft)))
     dX = L.fortis_plan_tensor_ptr(plan.handle, plan.in_tensor)
     dY = L.fortis_plan_tensor_ptr(plan.handle, plan.out_tensor)
     CB = C.CFUNCTYPE(None, C.c_void_p)
@@ -170,15 +177,16 @@ def run_zb_unfused(L, args):
     s_ms = L.fortis_time_ms(scatter_cb, None, args.steps) / args.steps
     L.fortis_sync()
     dt = time.perf_counter() - t0
-    g_bytes = 4 * (4 * n3 + 27 * rows)                     # 4 planes read once, X written
-    s_bytes = 4 * (3 * rows + n3 + nz * sx * sy + 3 * rows)  # Y read, norm + kappa read per layer, 3 outputs written
+    g_bytes = esz * 4 * n3 + 4 * 27 * rows                 # 4 planes read once, X written
+    s_bytes = 4 * 3 * rows + esz * (n3 + nz * sx * sy + 3 * rows)  # Y read, norm + kappa read per layer, 3 outputs written
     gbs = g_bytes / (g_ms * 1e-3) / 1e9
-    roof = dict(bound="hbm", kernel="gather_kernel (stencil gather with lifted expressions)", achieved=round(gbs, 1), peak=PEAK_HBM_GBS,
+    kname = "gather_generic_kernel (typed stencil gather, fp64 host arrays)" if args.f64 else "gather_kernel (stencil gather with lifted expressions)"
+    roof = dict(bound="hbm", kernel=kname, achieved=round(gbs, 1), peak=PEAK_HBM_GBS,
                 unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(g_ms, 5), bytes_per_launch=g_bytes,
                 scatter_GBs=round(s_bytes / (s_ms * 1e-3) / 1e9, 1), scatter_ms_all_layers=round(s_ms, 5), mlp_ms=round(m_ms, 5),
-                traffic=MEASURED_TRAFFIC.get("zb_unfused_%dx%dx%d" % (sx, sy, nz)))
+                traffic=None if args.f64 else MEASURED_TRAFFIC.get("zb_unfused_%dx%dx%d" % (sx, sy, nz)))
     out = dict(rows=rows, dt=(g_ms + m_ms + s_ms) * 1e-3 * args.steps, wall_dt=dt, dtype="f32",
-               config={"workload": "zb_unfused_gather_mlp_scatter_27_64_64_3_%dx%dx%d" % (sx, sy, nz), "columns": rows,
+               config={"workload": "zb_unfused_gather_mlp_scatter_27_64_64_3_%dx%dx%d%s" % (sx, sy, nz, "_f64_arrays" if args.f64 else ""), "columns": rows,
                        "cells_per_layer": count, "layers": nz, "launches_per_step": 1 + nz + plan.num_kernels},
                roofline=roof)
     plan.close()
@@ -391,6 +399,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20, help="untimed steps first; the clocks need about ten steps of this size to settle")
     ap.add_argument("--workload", default="climsim", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--f64", action="store_true", help="zb_unfused only: double-precision host arrays (the general stencil kernels)")
     ap.add_argument("--grid", default=None, help="zb / zb_ref / zb_unfused only: SXxSYxNZ grid instead of the reference's 68x78x15 (zb_unfused: 1028x1028x15)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -11,18 +11,25 @@
 #include "stencil_dev.h"
 
 #define SG_THREADS 256
+#define SG_CHAIN_MAX 8
 
 struct GenSlot { const void* p; long si, sj, plane; int f64, pad_; };   // p: array base with the element offset folded in
 struct alignas(16) GenArgs {
-    int nrefs, nscal, nins, pad0_;
+    int nrefs, nscal, nins, cellmask;      // cellmask: bit n set = instruction n does not depend on the slot value
     GenSlot refs[FORTIS_MAX_REFS];
     GenSlot scal[FORTIS_MAX_SCAL];
     int op[FORTIS_MAX_INS], a[FORTIS_MAX_INS], b[FORTIS_MAX_INS];
     double consts[FORTIS_MAX_CONST];
     unsigned count;
-    int ilo, jlo, ni, sx, pad1_;
+    int ilo, jlo, ni, sx, uniform;          // uniform: every slot has the strides of slot 0
     const int* cells;
     StMagic mcount, mni, msx;
+    int slotkind;                           // slot arrays: 0 all fp32, 1 all fp64, 2 mixed
+    // Chain form of the slot-dependent instructions (nchain < 0: not of that form): step s applies ch_op[s] to the
+    // running slot value and one operand that is the same for every slot of the row (ch_other[s], an operand
+    // code, -1 for a unary operator); ch_left[s]: the running value is the left operand.
+    int nchain, pad_[2];
+    int ch_op[SG_CHAIN_MAX], ch_other[SG_CHAIN_MAX], ch_left[SG_CHAIN_MAX];
 };
 
 typedef __attribute__((address_space(1))) double gdouble;
@@ -38,21 +45,18 @@ __device__ __forceinline__ void sg_store(const GenSlot& s, long off, float v)
 }
 
 // Runs the instruction list on one slot value.  r: this thread's column of the result scratch in LDS.
-__device__ __forceinline__ float sg_eval(const GenArgs& d, float tv, const double (&S)[FORTIS_MAX_SCAL],
-                                         double (*r)[SG_THREADS], int tid)
+// Instructions that do not depend on the slot value (bit set in d.cellmask) are the same for every slot of a
+// row: phase 1 runs those once per row, phase 0 the others once per slot; both leave their results in r.
+// The row's scalars are rows nins .. nins + nscal - 1 of r, so that an operand of any kind is one read.
+__device__ __forceinline__ float sg_eval(const GenArgs& d, float tv, double (*r)[SG_THREADS], int tid, int phase)
 {
-    const int nins = st_u(d.nins);
-    double last = (double)tv;
+    const int nins = st_u(d.nins), cellmask = st_u(d.cellmask);
     for (int n = 0; n < nins; n++) {
+        if (((cellmask >> n) & 1) != phase) continue;
         const int opw = st_u(d.op[n]), ca = st_u(d.a[n]), cb = st_u(d.b[n]);
         auto operand = [&](int code) -> double {
             if (code == 0) return (double)tv;
-            if (code < 16) {
-                double v = S[0];
-#pragma unroll
-                for (int s = 1; s < FORTIS_MAX_SCAL; s++) v = (code == 1 + s) ? S[s] : v;
-                return v;
-            }
+            if (code < 16) return r[nins + code - 1][tid];
             if (code < 32) return d.consts[code - 16];
             return r[code - 32][tid];
         };
@@ -75,57 +79,165 @@ __device__ __forceinline__ float sg_eval(const GenArgs& d, float tv, const doubl
             default: v = (double)xf; break;          // FORTIS_OP_F32
         }
         r[n][tid] = v;
-        last = v;
     }
-    return (float)last;
+    return nins ? (float)r[nins - 1][tid] : tv;
 }
 
+// An operand that does not involve the slot value: a scalar of the row, a constant, or an earlier result.
+__device__ __forceinline__ double sg_cell_operand(const GenArgs& d, double (*r)[SG_THREADS], int tid, int code)
+{
+    const int nins = st_u(d.nins);
+    if (code < 16) return r[nins + code - 1][tid];
+    if (code < 32) return d.consts[code - 16];
+    return r[code - 32][tid];
+}
+
+template <typename F>
+__device__ __forceinline__ void sg_apply(float* mine, int n, bool left, double c, F f)
+{
+    if (left) for (int q = 0; q < n; q++) mine[q] = (float)f((double)mine[q], c);
+    else for (int q = 0; q < n; q++) mine[q] = (float)f(c, (double)mine[q]);
+}
+
+// One step of the chain form on all n slot values of the row: the operator is decoded once, not once per slot.
+// Same arithmetic as sg_eval: operands as doubles, an fp32 operation converts them to float first.
+__device__ __forceinline__ void sg_chain_step(int opw, bool left, double c, float* mine, int n)
+{
+    const bool f64 = (opw & FORTIS_INS_F64) != 0;
+    switch (opw & 0xff) {
+        case FORTIS_OP_ADD:
+            if (f64) sg_apply(mine, n, left, c, [](double x, double y) { return __dadd_rn(x, y); });
+            else sg_apply(mine, n, left, c, [](double x, double y) { return (double)__fadd_rn((float)x, (float)y); });
+            break;
+        case FORTIS_OP_SUB:
+            if (f64) sg_apply(mine, n, left, c, [](double x, double y) { return __dsub_rn(x, y); });
+            else sg_apply(mine, n, left, c, [](double x, double y) { return (double)__fsub_rn((float)x, (float)y); });
+            break;
+        case FORTIS_OP_MUL:
+            if (f64) sg_apply(mine, n, left, c, [](double x, double y) { return __dmul_rn(x, y); });
+            else sg_apply(mine, n, left, c, [](double x, double y) { return (double)__fmul_rn((float)x, (float)y); });
+            break;
+        case FORTIS_OP_DIV:
+            if (f64) sg_apply(mine, n, left, c, [](double x, double y) { return __ddiv_rn(x, y); });
+            else sg_apply(mine, n, left, c, [](double x, double y) { return (double)__fdiv_rn((float)x, (float)y); });
+            break;
+        case FORTIS_OP_MAX: sg_apply(mine, n, left, c, [](double x, double y) { return (double)fmaxf((float)x, (float)y); }); break;
+        case FORTIS_OP_MIN: sg_apply(mine, n, left, c, [](double x, double y) { return (double)fminf((float)x, (float)y); }); break;
+        case FORTIS_OP_NEG: sg_apply(mine, n, true, c, [](double x, double) { return (double)(-(float)x); }); break;   // exact in either type
+        case FORTIS_OP_SQRT: sg_apply(mine, n, true, c, [](double x, double) { return (double)__builtin_sqrtf((float)x); }); break;
+        case FORTIS_OP_EXP: sg_apply(mine, n, true, c, [](double x, double) { return (double)expf((float)x); }); break;
+        case FORTIS_OP_LOG: sg_apply(mine, n, true, c, [](double x, double) { return (double)logf((float)x); }); break;
+        case FORTIS_OP_TANH: sg_apply(mine, n, true, c, [](double x, double) { return (double)tanhf((float)x); }); break;
+        default: break;                                        // FORTIS_OP_F32: the running value is a float already
+    }
+}
+
+// Loads the row's scalars into their rows of r.
+__device__ __forceinline__ void sg_scalars(const GenArgs& d, double (*r)[SG_THREADS], int tid, int i, int j, int kk)
+{
+    const int nins = st_u(d.nins), nscal = st_u(d.nscal);
+    for (int s = 0; s < nscal; s++)
+        r[nins + s][tid] = sg_load(d.scal[s], (long)i * d.scal[s].si + (long)j * d.scal[s].sj + (long)kk * d.scal[s].plane);
+}
+// Element offset of slot sl at cell (i, j, kk); off0 serves every slot when they share their strides.
+__device__ __forceinline__ long sg_off(const GenArgs& d, const GenSlot& sl, long off0, int i, int j, int kk)
+{
+    return st_u(d.uniform) ? off0 : (long)i * sl.si + (long)j * sl.sj + (long)kk * sl.plane;
+}
+
+// Loads the row's n slot values into mine[], four loads in flight at a time.  T: element type of every slot's array.
+template <typename T>
+__device__ __forceinline__ void sg_load_slots(const GenArgs& d, float* mine, int n, long off0, int i, int j, int kk)
+{
+    typedef __attribute__((address_space(1))) T gT;
+    int q = 0;
+    for (; q + 4 <= n; q += 4) {
+        T v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const GenSlot& sl = d.refs[q + u];
+            v[u] = ((const gT*)sl.p)[sg_off(d, sl, off0, i, j, kk)];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) mine[q + u] = (float)v[u];          // float tv = A[...]
+    }
+    for (; q < n; q++) {
+        const GenSlot& sl = d.refs[q];
+        mine[q] = (float)((const gT*)sl.p)[sg_off(d, sl, off0, i, j, kk)];
+    }
+}
+
+// One thread per row.  The row's slot values are loaded first (independent loads, several in flight), then
+// evaluated in place in the workgroup's tile of X in LDS; the tile -- SG_THREADS consecutive rows, contiguous
+// in X -- is written out with coalesced 16-byte stores (a thread storing its own row strides by the row length).
+// Dynamic LDS: [nins + nscal][SG_THREADS] doubles (expression results, then the row's scalars), then the tile [SG_THREADS][nrefs] floats.
 __global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args, float* __restrict__ X, unsigned rows)
 {
     __shared__ GenArgs d;
-    __shared__ double r[FORTIS_MAX_INS][SG_THREADS];
+    extern __shared__ double sg_dyn[];
     params_to_lds(&d, SG_THREADS);
     const int tid = threadIdx.x;
-    const unsigned row = blockIdx.x * SG_THREADS + tid;
-    if (row >= rows) return;
-    int i, j, kk;
-    st_row(d, row, i, j, kk);
-    double S[FORTIS_MAX_SCAL];
-#pragma unroll
-    for (int s = 0; s < FORTIS_MAX_SCAL; s++) {
-        S[s] = 0.0;
-        if (s < d.nscal) S[s] = sg_load(d.scal[s], (long)i * d.scal[s].si + (long)j * d.scal[s].sj + (long)kk * d.scal[s].plane);
+    const int n = st_u(d.nrefs), nins = st_u(d.nins);
+    double (*r)[SG_THREADS] = (double (*)[SG_THREADS])sg_dyn;
+    float* tile = (float*)(sg_dyn + (size_t)(nins + st_u(d.nscal)) * SG_THREADS);
+    const unsigned row0 = blockIdx.x * SG_THREADS, row = row0 + tid;
+    if (row < rows) {
+        int i, j, kk;
+        st_row(d, row, i, j, kk);
+        sg_scalars(d, r, tid, i, j, kk);
+        const long off0 = (long)i * d.refs[0].si + (long)j * d.refs[0].sj + (long)kk * d.refs[0].plane;
+        float* mine = tile + tid * n;
+        const int kind = st_u(d.slotkind);
+        if (kind == 1) sg_load_slots<double>(d, mine, n, off0, i, j, kk);
+        else if (kind == 0) sg_load_slots<float>(d, mine, n, off0, i, j, kk);
+        else
+            for (int q = 0; q < n; q++) {
+                const GenSlot& sl = d.refs[q];
+                mine[q] = (float)sg_load(sl, sg_off(d, sl, off0, i, j, kk));   // float tv = A[...]
+            }
+        sg_eval(d, 0.f, r, tid, 1);
+        const int nchain = st_u(d.nchain);
+        if (nchain >= 0) {
+            for (int c = 0; c < nchain; c++) {
+                const int other = st_u(d.ch_other[c]);
+                sg_chain_step(st_u(d.ch_op[c]), st_u(d.ch_left[c]) != 0, other >= 0 ? sg_cell_operand(d, r, tid, other) : 0.0, mine, n);
+            }
+        } else {
+            for (int q = 0; q < n; q++) mine[q] = sg_eval(d, mine[q], r, tid, 0);
+        }
     }
-    const int n = st_u(d.nrefs);
-    float* out = X + (size_t)row * n;
-    for (int q = 0; q < n; q++) {
-        const GenSlot& sl = d.refs[q];
-        const float tv = (float)sg_load(sl, (long)i * sl.si + (long)j * sl.sj + (long)kk * sl.plane);   // float tv = A[...]
-        out[q] = sg_eval(d, tv, S, r, tid);
+    __syncthreads();
+    const unsigned nr = rows - row0 < SG_THREADS ? rows - row0 : SG_THREADS, total = nr * n;
+    float* dst = X + (size_t)row0 * n;
+    if (((uintptr_t)dst & 15) == 0) {
+        const unsigned t4 = total / 4;
+        for (unsigned v = tid; v < t4; v += SG_THREADS) ((float4*)dst)[v] = ((const float4*)tile)[v];
+        for (unsigned e = t4 * 4 + tid; e < total; e += SG_THREADS) dst[e] = tile[e];
+    } else {
+        for (unsigned e = tid; e < total; e += SG_THREADS) dst[e] = tile[e];
     }
 }
 
+// One thread per cell of layer kk.  Dynamic LDS: [nins + nscal][SG_THREADS] doubles (expression results, scalars).
 __global__ __launch_bounds__(SG_THREADS) void scatter_generic_kernel(GenArgs args, const float* __restrict__ Y, int kk)
 {
     __shared__ GenArgs d;
-    __shared__ double r[FORTIS_MAX_INS][SG_THREADS];
+    extern __shared__ double sg_dyn[];
     params_to_lds(&d, SG_THREADS);
+    double (*r)[SG_THREADS] = (double (*)[SG_THREADS])sg_dyn;
     const int tid = threadIdx.x;
     const unsigned col = blockIdx.x * SG_THREADS + tid;
     if (col >= d.count) return;
     int i, j;
     st_cell(d, col, i, j);
-    double S[FORTIS_MAX_SCAL];
-#pragma unroll
-    for (int s = 0; s < FORTIS_MAX_SCAL; s++) {
-        S[s] = 0.0;
-        if (s < d.nscal) S[s] = sg_load(d.scal[s], (long)i * d.scal[s].si + (long)j * d.scal[s].sj + (long)kk * d.scal[s].plane);
-    }
+    sg_scalars(d, r, tid, i, j, kk);
+    const long off0 = (long)i * d.refs[0].si + (long)j * d.refs[0].sj + (long)kk * d.refs[0].plane;
     const int n = st_u(d.nrefs);
     const float* in = Y + (size_t)col * n;
+    sg_eval(d, 0.f, r, tid, 1);
     for (int q = 0; q < n; q++) {
         const GenSlot& sl = d.refs[q];
-        sg_store(sl, (long)i * sl.si + (long)j * sl.sj + (long)kk * sl.plane, sg_eval(d, in[q], S, r, tid));
+        sg_store(sl, sg_off(d, sl, off0, i, j, kk), sg_eval(d, in[q], r, tid, 0));
     }
 }
 
@@ -207,8 +319,42 @@ static void sg_make_args(const fortis_stencil_t& t, const int* dcells, const voi
         s.plane = f.planar ? t.plane[f.array] : 0;
         s.f64 = sg_esz(t, f.array) == 8;
     }
-    for (int n = 0; n < t.nins; n++) { g->op[n] = t.ins[n].op; g->a[n] = t.ins[n].a; g->b[n] = t.ins[n].b; }
+    for (int n = 0; n < t.nins; n++) {
+        g->op[n] = t.ins[n].op; g->a[n] = t.ins[n].a; g->b[n] = t.ins[n].b;
+        // depends on the slot value: reads it, or reads the result of an instruction that does
+        auto dep = [&](int code) { return code == 0 || (code >= 32 && !((g->cellmask >> (code - 32)) & 1)); };
+        const bool binary = (t.ins[n].op & 0xff) <= FORTIS_OP_MIN;
+        if (!dep(t.ins[n].a) && !(binary && dep(t.ins[n].b))) g->cellmask |= 1 << n;
+    }
     for (int c = 0; c < t.nconst; c++) g->consts[c] = t.cdouble[c] ? t.dconsts[c] : (double)t.consts[c];
+    // Chain form: every slot-dependent instruction combines the previous one's result (the slot value for the
+    // first) with an operand that is the same for all slots, the last instruction is the last step, and no fp64
+    // step feeds another fp64 step (the running values are kept as floats).
+    {
+        int prev = -1, nch = 0;
+        bool ok = t.nins == 0 || !((g->cellmask >> (t.nins - 1)) & 1);
+        for (int n = 0; n < t.nins && ok; n++) {
+            if ((g->cellmask >> n) & 1) continue;
+            const int op = t.ins[n].op & 0xff, a = t.ins[n].a, b = t.ins[n].b, run = prev < 0 ? 0 : 32 + prev;
+            const bool binary = op <= FORTIS_OP_MIN;
+            auto dep = [&](int code) { return code == 0 || (code >= 32 && !((g->cellmask >> (code - 32)) & 1)); };
+            if (nch == SG_CHAIN_MAX) { ok = false; break; }
+            if (a == run && !(binary && dep(b))) { g->ch_left[nch] = 1; g->ch_other[nch] = binary ? b : -1; }
+            else if (binary && b == run && !dep(a)) { g->ch_left[nch] = 0; g->ch_other[nch] = a; }
+            else { ok = false; break; }
+            // a double handed from one fp64 step to the next would be cut to a float (an fp32 step converts its
+            // operands to float anyway)
+            if (prev >= 0 && (t.ins[prev].op & FORTIS_INS_F64) && (t.ins[n].op & FORTIS_INS_F64)) { ok = false; break; }
+            g->ch_op[nch++] = t.ins[n].op;
+            prev = n;
+        }
+        g->nchain = ok ? nch : -1;
+    }
+    g->slotkind = g->refs[0].f64;
+    for (int r = 1; r < t.nrefs; r++) if (g->refs[r].f64 != g->refs[0].f64) g->slotkind = 2;
+    g->uniform = 1;
+    for (int r = 1; r < t.nrefs; r++)
+        if (g->refs[r].si != g->refs[0].si || g->refs[r].sj != g->refs[0].sj || g->refs[r].plane != g->refs[0].plane) g->uniform = 0;
     g->count = (unsigned)t.count;
     g->ilo = t.ilo; g->jlo = t.jlo; g->ni = t.ni > 0 ? t.ni : 1; g->sx = t.sx > 0 ? t.sx : 1;
     g->cells = dcells;
@@ -222,13 +368,21 @@ void fortis_launch_gather_generic(const fortis_stencil_t& t, const int* dcells, 
     GenArgs g;
     sg_make_args(t, dcells, dA, &g);
     const unsigned rows = (unsigned)(t.count * t.nk);
-    hipLaunchKernelGGL(gather_generic_kernel, dim3((unsigned)cdiv(rows, SG_THREADS)), dim3(SG_THREADS), 0, s, g, dX, rows);
+    const size_t shmem = (size_t)SG_THREADS * ((t.nins + t.nscal) * sizeof(double) + t.nrefs * sizeof(float));   // at most 72 KB
+    static bool sized = false;
+    if (!sized) {
+        HIP_OK(hipFuncSetAttribute((const void*)gather_generic_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   SG_THREADS * (int)((FORTIS_MAX_INS + FORTIS_MAX_SCAL) * sizeof(double) + FORTIS_MAX_REFS * sizeof(float))));
+        sized = true;
+    }
+    hipLaunchKernelGGL(gather_generic_kernel, dim3((unsigned)cdiv(rows, SG_THREADS)), dim3(SG_THREADS), shmem, s, g, dX, rows);
     HIP_OK(hipGetLastError());
 }
 void fortis_launch_scatter_generic(const fortis_stencil_t& t, const int* dcells, void* const* dA, const float* dY, int kk, hipStream_t s)
 {
     GenArgs g;
     sg_make_args(t, dcells, (const void* const*)dA, &g);
-    hipLaunchKernelGGL(scatter_generic_kernel, dim3((unsigned)cdiv(t.count, SG_THREADS)), dim3(SG_THREADS), 0, s, g, dY, kk);
+    hipLaunchKernelGGL(scatter_generic_kernel, dim3((unsigned)cdiv(t.count, SG_THREADS)), dim3(SG_THREADS),
+                       (size_t)SG_THREADS * (t.nins + t.nscal) * sizeof(double), s, g, dY, kk);
     HIP_OK(hipGetLastError());
 }

@@ -65,6 +65,15 @@ def _gather(L, gd, lp, kd, garr):
     (["((tv * tv) + tv)"], ()),                                  # not a chain on the slot value
     (["(sqrtf(fmaxf(tv, 0.0f)) * S0)", "(fminf(tv, 2.0f) - (-S0))"], ()),
     (["((-tv) / -3.0f)"], (1,)),
+    # the slot value as the right operand of a step, in float and in double
+    (["(S0 / tv)", "(2.0 - tv)"], (3,)),
+    # one fp64 step feeding another: the running value cannot be cut to a float between them
+    (["((tv * S0) * S0)"], (3,)),
+    # a per-cell subexpression beside the chain on the slot value
+    (["(sqrtf(fmaxf(tv, 0.0f)) / ((S0 * S0) + 1.0f))"], ()),
+    (["((tv - S0) / ((S0 * S0) + 1.0f))"], (3,)),
+    # more steps than the chain form holds
+    (["(((((((((tv + 1.0f) * 2.0f) - 3.0f) * 0.5f) + S0) * S0) - 1.0f) * 2.0f) + 0.25f)"], ()),
 ])
 def test_general_gather_bit_exact(L, gpu, exprs, g64):
     gd, sd, lp, kd, garr, _ = _case(gexprs=exprs, g64=g64)
