@@ -158,6 +158,57 @@ def test_fused_step_config2_network(L, gpu, golden, hidden):
     plan.close()
 
 
+def test_bench_grid_fused_equals_unfused_and_layer_vs_oracle(L, gpu):
+    """The benchmark grid, 1028 x 1028 x 15 (15.7 M columns), through properties that do not need the oracle at
+    that size: the one-launch fused step and the reference's structure (gather kernel -> X -> MLP -> Y -> one
+    scatter per layer) run the same arithmetic and must agree bit for bit in Y and in every written field; one
+    layer of X and its scatter are checked against the oracle on that layer's planes."""
+    sx, sy, nz = 1028, 1028, 15
+    gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    gt, st = S.build_table(gd, lp, kd, "gather"), S.build_table(sd, lp, kd, "scatter")
+    A = configs.zb_arrays(sx, sy, nz)
+    count, n2, n3 = (sx - 4) * (sy - 4), sx * sy, sx * sy * nz
+    rows = count * nz
+    net = configs.zb_mlp()
+    plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows)
+    garr = [A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"]]
+    host = [A["norm_h"], A["kappa_h"], np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+    fused_out, fused_Y = _fused(L, gt, st, plan, garr, host, rows)
+    # the reference's structure
+    gb = [DevBuf(L, a) for a in garr]
+    sb = [DevBuf(L, a) for a in host]
+    dX = L.fortis_plan_tensor_ptr(plan.handle, plan.in_tensor)
+    dY = L.fortis_plan_tensor_ptr(plan.handle, plan.out_tensor)
+    L.fortis_stencil_gather_dev(C.byref(gt), ptrs(gb), C.c_void_p(dX))
+    plan.run()
+    for kk in range(nz):
+        L.fortis_stencil_scatter_dev(C.byref(st), ptrs(sb), C.c_void_p(dY + kk * count * 3 * 4), kk)
+    L.fortis_sync()
+    Y = np.empty((rows, 3), np.float32)
+    L.fortis_d2h(Y.ctypes.data, C.c_void_p(dY), Y.nbytes)
+    assert bits_equal(Y, fused_Y)
+    for q in (3, 4):
+        assert bits_equal(sb[q].get(host[q].shape), fused_out[q])
+    # the 2-D Txy_h: the layer-by-layer scatters leave the last layer in it, the fused step keeps one plane per layer
+    assert bits_equal(sb[2].get((n2,)), fused_out[2].reshape(nz, n2)[nz - 1])
+    # layer kk against the oracle: X rows of that layer, and the scatter of the GPU's own Y for it
+    kk = 7
+    Xk = np.empty((count, 27), np.float32)
+    L.fortis_d2h(Xk.ctypes.data, C.c_void_p(dX + kk * count * 27 * 4), Xk.nbytes)
+    plane = lambda a: np.ascontiguousarray(a.reshape(nz, n2)[kk])
+    gd1, sd1, _, _ = configs.zb_descriptors(sx, sy, 1)
+    assert bits_equal(Xk, O.stencil_gather(gd1, [plane(a) for a in garr], count, 1, 3, 3, sx - 4))
+    ref = [plane(A["norm_h"]), A["kappa_h"], np.zeros(n2, np.float32), np.zeros(n2, np.float32), np.zeros(n2, np.float32)]
+    O.stencil_scatter(sd1, ref, Y[kk * count:(kk + 1) * count], count, 0, 3, 3, sx - 4)
+    assert bits_equal(plane(fused_out[3]), ref[3]) and bits_equal(plane(fused_out[4]), ref[4])
+    # the fp64-accumulated network on a seeded sample of that layer's rows
+    idx = np.random.default_rng(6).choice(count, 512, replace=False)
+    assert maxrel(Y[kk * count + idx], O.mlp_f64(net["Ws"], net["bs"], net["acts"], Xk[idx])) < TOL
+    for b in gb + sb:
+        b.free()
+    plan.close()
+
+
 def test_fused_step_rejects_mismatched_tables(L, gpu, golden, capfd):
     gt, st, gd, sd, lp, kd = golden_tables(golden)
     net = configs.toy_mlp(64)
