@@ -504,7 +504,9 @@ static int launch_mt(const float* x, const float* wp, float* y, ConvMShape s, co
     const long want = 2L * conv_cus(), groups = (long)s.D * cdiv(s.F, FT);
     constexpr int MTMIN = FT == 64 ? 64 : 128;
     if (KD == 1 && groups * cdiv(s.plane, 256) >= want && launch<KD, KS, 256, FT>(x, wp, y, s, e, st) == 0) return 0;
-    if (2 * groups * cdiv(s.plane, 128) >= want || MTMIN == 128) return launch<KD, KS, 128, FT>(x, wp, y, s, e, st);
+    // images: 128 positions only if that alone fills the chip (a smaller tile beats a channel split with its
+    // reduce kernel); volumes keep 128 positions down to half of that (their chunks are long enough to split)
+    if ((KD == 1 ? 1 : 2) * groups * cdiv(s.plane, 128) >= want || MTMIN == 128) return launch<KD, KS, 128, FT>(x, wp, y, s, e, st);
     return launch<KD, KS, MTMIN, FT>(x, wp, y, s, e, st);
 }
 
