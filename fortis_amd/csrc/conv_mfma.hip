@@ -413,6 +413,42 @@ float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transpos
     return d;
 }
 
+// The same packing on the device, for callers that hold raw weights in device memory and give them anew with
+// every call (the runtime-tier conv entries): W[F][C][T] -> a buffer of the library (one for all shapes,
+// grown on demand and kept; launches on the library's stream run one after the other).
+__global__ void conv_pack_kernel(const float* __restrict__ W, float* __restrict__ P, long F, long C, int T, int FT, int CC, long nch,
+                                 long n)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    const int NCP = CC / 2;
+    long r = idx;
+    const int fl = (int)(r % FT); r /= FT;
+    const int hh = (int)(r % 2); r /= 2;
+    const int t = (int)(r % T); r /= T;
+    const int cp = (int)(r % NCP); r /= NCP;
+    const long ch = r % nch, fgi = r / nch;
+    const long f = fgi * FT + fl, c = ch * CC + cp * 2 + hh;
+    P[idx] = (f < F && c < C) ? W[(f * C + c) * T + t] : 0.f;
+}
+
+const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, hipStream_t st)
+{
+    static float* buf = nullptr;
+    static size_t cap = 0;
+    const long FT = conv_ft(F), CC = cm_cc(T);
+    const long nch = cdiv(C, CC), n = cdiv(F, FT) * nch * (CC / 2) * T * 2 * FT;
+    if ((size_t)n * sizeof(float) > cap) {
+        float* p = nullptr;
+        if (hipMalloc((void**)&p, (size_t)n * sizeof(float)) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        buf = p;                                   // an outgrown buffer stays: a captured graph may name it
+        cap = (size_t)n * sizeof(float);
+    }
+    hipLaunchKernelGGL(conv_pack_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, st, dW, buf, F, C, T, (int)FT, (int)CC, nch, n);
+    HIP_OK(hipGetLastError());
+    return buf;
+}
+
 template <int KD, int KS, int MT, int FT, int NX, bool TILE2D>
 static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {

@@ -98,6 +98,22 @@ void fortis_gemm(float* Aa, float* A, long Ao, long As0, long As1, long At0, lon
 }
 
 // ---- conv entries (runtime/fortis_rt.c:108-156, runtime/fortis_fft.cu:66-79, 131-146) -------
+// Shapes the matrix-core kernel takes (stride 1, K = 1 or 3 with same padding, enough output channels to fill a
+// 32-channel group) go to it: the raw weights are packed on the device with every call (the reference reads the
+// weights it is given on every call, so nothing is cached by pointer).  FORTIS_CONV_DIRECT=1 keeps the direct
+// kernels.  Returns -1 when the shape is not taken.
+static int conv_entry_mfma(const float* x, const float* w, float* y, long C, long D, long H, long Wd, long F, long KD, long KS)
+{
+    static int direct_only = -1;
+    if (direct_only < 0) direct_only = getenv("FORTIS_CONV_DIRECT") != nullptr;
+    if (direct_only || !(F >= 16 || (KD == 1 && KS == 1))) return -1;
+    hipStream_t s = fortis_stream_get();
+    const float* wp = fortis_conv_mfma_pack_dev(w, F, C, (int)(KD * KS * KS), s);
+    if (!wp) return -1;
+    ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
+    return fortis_launch_conv_mfma(x, wp, y, C, D, H, Wd, F, (int)KD, (int)KS, 0, e, s);
+}
+
 void fortis_conv2d(float* xa, float* x, long xo, long x0, long x1, long x2, long x3, long xt0, long xt1, long xt2, long xt3,
                    float* wa, float* w, long wo, long w0, long w1, long w2, long w3, long wt0, long wt1, long wt2, long wt3,
                    float* ya, float* y, long yo, long y0, long y1, long y2, long y3, long yt0, long yt1, long yt2, long yt3,
@@ -108,7 +124,9 @@ void fortis_conv2d(float* xa, float* x, long xo, long x0, long x1, long x2, long
     (void)wa; (void)w0; (void)w1; (void)w2; (void)w3; (void)wt0; (void)wt1; (void)wt2; (void)wt3;
     (void)ya; (void)y0; (void)y1; (void)y2; (void)y3; (void)yt0; (void)yt1; (void)yt2; (void)yt3;
     ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
+    const bool same = sh == 1 && sw == 1 && KH == KW && (KH == 1 || KH == 3) && ph == KH / 2 && pw == KW / 2 && Hout == Hin && Wout == Win;
     for (long n = 0; n < N; n++) {
+        if (same && conv_entry_mfma(x + xo + n * C * Hin * Win, w + wo, y + yo + n * F * Hout * Wout, C, 1, Hin, Win, F, 1, KH) == 0) continue;
         int rc = fortis_launch_conv2d(x + xo + n * C * Hin * Win, w + wo, y + yo + n * F * Hout * Wout, C, Hin, Win, F,
                                       KH, KW, Hout, Wout, sh, sw, ph, pw, e, 0, F, fortis_stream_get());
         if (rc != 0) {
@@ -124,6 +142,9 @@ static void conv3d_any(const char* who, float* x, long xo, float* w, long wo, fl
                        long Wout, long sd, long sh, long sw, long pd, long ph, long pw)
 {
     if (N != 1 || sd != 1 || sh != 1 || sw != 1) { fprintf(stderr, "%s: unsupported shape\n", who); return; }
+    if (KD == 3 && KH == 3 && KW == 3 && pd == 1 && ph == 1 && pw == 1 && Dout == Din && Hout == Hin && Wout == Win &&
+        conv_entry_mfma(x + xo, w + wo, y + yo, C, Din, Hin, Win, F, 3, 3) == 0)
+        return;
     ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
     if (fortis_launch_conv3d(x + xo, w + wo, y + yo, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, pd, ph, pw, e,
                              fortis_stream_get()) != 0)

@@ -213,6 +213,38 @@ def test_memref_conv_entries(L, gpu, capfd):
         d.free()
 
 
+def test_memref_conv_entries_wide_shapes(L, gpu):
+    """The runtime-tier entries on shapes the matrix-core kernel takes (raw weights packed on the device per call):
+    a batch of two 3x3 images, a 1x1 conv, a 3x3x3 volume; a second call with other weights in the same buffer
+    must use them (nothing is cached by pointer)."""
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((2, 24, 40, 36)).astype(np.float32)
+    for k in (3, 1):
+        w = (rng.standard_normal((48, 24, k, k)) / np.sqrt(24 * k * k)).astype(np.float32)
+        ref = O.conv2d(x, w, (1, 1), (k // 2, k // 2))
+        dx, dw, dy = DevBuf(L, x), DevBuf(L, w), DevBuf(L, nbytes=ref.nbytes)
+        args = [2, 24, 40, 36, 48, k, k, 40, 36, 1, 1, k // 2, k // 2]
+        L.fortis_conv2d(*_memref(dx, x.shape), *_memref(dw, w.shape), *_memref(dy, ref.shape), *args)
+        assert maxrel(dy.get(ref.shape), ref) < TOL
+        w2 = (rng.standard_normal(w.shape) / np.sqrt(24 * k * k)).astype(np.float32)
+        L.fortis_h2d(dw.ptr, w2.ctypes.data, w2.nbytes)
+        L.fortis_conv2d(*_memref(dx, x.shape), *_memref(dw, w.shape), *_memref(dy, ref.shape), *args)
+        assert maxrel(dy.get(ref.shape), O.conv2d(x, w2, (1, 1), (k // 2, k // 2))) < TOL
+        for d in (dx, dw, dy):
+            d.free()
+    x3 = rng.standard_normal((1, 10, 9, 14, 11)).astype(np.float32)
+    w3 = (rng.standard_normal((20, 10, 3, 3, 3)) / np.sqrt(270)).astype(np.float32)
+    ref3 = O.conv3d(x3, w3, pad=(1, 1, 1))
+    dx3, dw3, dy3 = DevBuf(L, x3), DevBuf(L, w3), DevBuf(L, nbytes=ref3.nbytes)
+    tail = [1, 10, 9, 14, 11, 20, 3, 3, 3, 9, 14, 11, 1, 1, 1, 1, 1, 1]
+    for fn in (L.fortis_conv3d, L.fortis_conv3d_direct):
+        L.fortis_d2d(dy3.ptr, dx3.ptr, 16)
+        fn(*_memref(dx3, x3.shape), *_memref(dw3, w3.shape), *_memref(dy3, ref3.shape), *tail)
+        assert maxrel(dy3.get(ref3.shape), ref3) < TOL
+    for d in (dx3, dw3, dy3):
+        d.free()
+
+
 @pytest.mark.parametrize("H,chans", [(32, (8, 16, 24, 32)), (256, (32, 64, 128, 256))])
 def test_config4_unet(L, gpu, H, chans):
     case = configs.unet(H=H, chans=chans)
