@@ -28,7 +28,11 @@ PEAK_HBM_GBS = 8000.0
 # same command (see profiles/), or None where no counter run has been made for the workload.
 MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((2482.4 * 2 + 936.6) * 1024),
                     "zb_ref": int((2396.6 * 2 + 936.6) * 1024), "zb_1028x1028x15": int((331322.2 * 2 + 207387.3) * 1024), "toy": None,
-                    "zb_unfused_1028x1028x15": int((242224.0 * 2 + 1658880.0) * 1024)}
+                    "zb_unfused_1028x1028x15": int((242224.0 * 2 + 1658880.0) * 1024),
+                    "zb_unfused_1028x1028x15_f64": int((457592.4 * 2 + 1658880.0) * 1024),
+                    # conv workloads: every conv, split-reduce and thin-head dispatch of a step summed, divided by the
+                    # step's conv operations (18 and 19), like flop_per_launch
+                    "unet": int((4443827968 - 7 * (4124.1 * 2 + 2048.0) * 1024) / 7 / 18), "tsrgan": int(13291334624 / 7 / 19)}
 
 
 def omp_threads():
@@ -184,7 +188,7 @@ def run_zb_unfused(L, args):
     roof = dict(bound="hbm", kernel=kname, achieved=round(gbs, 1), peak=PEAK_HBM_GBS,
                 unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(g_ms, 5), bytes_per_launch=g_bytes,
                 scatter_GBs=round(s_bytes / (s_ms * 1e-3) / 1e9, 1), scatter_ms_all_layers=round(s_ms, 5), mlp_ms=round(m_ms, 5),
-                traffic=None if args.f64 else MEASURED_TRAFFIC.get("zb_unfused_%dx%dx%d" % (sx, sy, nz)))
+                traffic=MEASURED_TRAFFIC.get("zb_unfused_%dx%dx%d%s" % (sx, sy, nz, "_f64" if args.f64 else "")))
     out = dict(rows=rows, dt=(g_ms + m_ms + s_ms) * 1e-3 * args.steps, wall_dt=dt, dtype="f32",
                config={"workload": "zb_unfused_gather_mlp_scatter_27_64_64_3_%dx%dx%d%s" % (sx, sy, nz, "_f64_arrays" if args.f64 else ""), "columns": rows,
                        "cells_per_layer": count, "layers": nz, "launches_per_step": 1 + nz + plan.num_kernels},
@@ -224,7 +228,8 @@ def run_conv(L, args, which):
                        "ms_per_step_by_kernel": {k: round(v, 4) for k, v in kern.items()}},
                roofline=dict(bound="mfma", kernel=dom + " (+ fused BN/bias/activation/residual epilogue)", achieved=round(achieved, 3),
                              peak=PEAK_F32_MFMA_TFLOPS, unit="TFLOP/s", frac=round(achieved / PEAK_F32_MFMA_TFLOPS, 4),
-                             avg_launch_ms=round(conv_ms / nconv, 5), flop_per_launch=case["flops"] / nconv, traffic=None))
+                             avg_launch_ms=round(conv_ms / nconv, 5), flop_per_launch=case["flops"] / nconv,
+                             traffic=MEASURED_TRAFFIC.get(which)))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_conv(case, which)
     plan.close()
