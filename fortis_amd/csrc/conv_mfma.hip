@@ -36,7 +36,8 @@ struct ConvMShape {
     int P, plane, tiles, nchunks, R;
     int tiles_x;               // TILE2D: tiles along x
     int mode;                  // 0: convolution, 1: 2x2 stride-2 transposed conv scatter
-    int ksplit, chunks_per;    // channel chunks are split over blockIdx.z; > 1: raw partial sums go to `part`
+    int ksplit;                // channel chunks are split over blockIdx.z; > 1: raw partial sums go to `part`
+    int cb[17];                // slice k takes chunks cb[k] .. cb[k+1]-1 (larger slices first: they are dispatched first)
     float* part;               // [ksplit][output elements]
     int ups;                   // 1: the input tensor is (D/2, H/2, W/2) and is read through a nearest x2 upsample
     long osize;                // output elements
@@ -54,7 +55,8 @@ __device__ __forceinline__ void cm_lds_barrier()
 
 #define CM_TP 34       // TILE2D: pitch of a staged row (32 columns + border)
 template <int KD, int KS, int MT, int FT, int NX, bool TILE2D>
-__global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
+__global__ __launch_bounds__(CM_THREADS) __attribute__((amdgpu_waves_per_eu(KD == 3 && MT == 128 && FT == 64 && NX <= 8 ? 4 : 1)))
+void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
 {
     constexpr int T = KD * KS * KS;
@@ -69,10 +71,10 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
     static_assert(!TILE2D || (KD == 1 && KS == 3), "the 2-D tiling is for 3 x 3 convs");
     extern __shared__ float4 smem4[];
     float* sW = (float*)smem4;                                    // [2][WCH]
-    float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R rounded up to the workgroup size]
+    float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R rounded up to a wave's 64 lanes]
     const int RR = TILE2D ? R2 : KS == 1 ? MT : s.R;              // staged elements per channel and kd (s.R, a constant where it can be)
     const int XCH = CC * KD * RR;
-    const int XCHP = (XCH + CM_THREADS - 1) / CM_THREADS * CM_THREADS;
+    const int XCHP = (XCH + 63) / 64 * 64;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int z = blockIdx.x / s.tiles, tile = blockIdx.x - z * s.tiles;
@@ -148,9 +150,10 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
         }
         float* xdst = sX + buf * XCHP + tid;
         const unsigned lim = chunk_lim(ch);
+        const int el0 = st_u(tid & ~63);          // the wave's first element of round 0: the bound check is per wave
 #pragma unroll
         for (int i = 0; i < NX; i++)
-            if (i * CM_THREADS < XCHP) xdst[i * CM_THREADS] = gchk[i] < lim ? r.rx[i] : 0.f;
+            if (i * CM_THREADS + el0 < XCHP) xdst[i * CM_THREADS] = gchk[i] < lim ? r.rx[i] : 0.f;
     };
 
     const int ft = wave % FW, mt0 = (wave / FW) * NMT;
@@ -164,8 +167,7 @@ __global__ __launch_bounds__(CM_THREADS) void conv_mfma_kernel(const float* __re
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
-    const int ch0 = blockIdx.z * s.chunks_per;
-    const int ch1 = ch0 + s.chunks_per < s.nchunks ? ch0 + s.chunks_per : s.nchunks;
+    const int ch0 = s.cb[blockIdx.z], ch1 = s.cb[blockIdx.z + 1];
     auto multiply = [&](int buf) {
         const float* w = sW + buf * WCH + wbase;
         const float* xs = sX + buf * XCHP + xbase;
@@ -462,7 +464,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
         s.R = (MT / 32 + 2) * CM_TP;
     }
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
-    const size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, CM_THREADS) * CM_THREADS) * sizeof(float);
+    const size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, 64) * 64) * sizeof(float);
     if (shmem > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
@@ -473,13 +475,16 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     // split writes raw partial sums, a second kernel adds them in order and applies the epilogue.
     const long wgs = (long)s.D * s.tiles * cdiv(s.F, FT);
     s.ksplit = 1;
-    s.chunks_per = s.nchunks;
+    s.cb[0] = 0; s.cb[1] = s.nchunks;
     if (2 * wgs < 3 * conv_cus() && s.C >= 32) {
-        long k = cdiv(2L * conv_cus(), wgs);
+        // volumes aim at three workgroups per CU (their chunks are long: 27 taps), images at two
+        long k = cdiv((KD == 3 ? 3L : 2L) * conv_cus(), wgs);
         if (k > s.C / 16) k = s.C / 16;               // at least 16 input channels per split
         if (k > 16) k = 16;
-        s.chunks_per = (int)cdiv(s.nchunks, k);
-        s.ksplit = (int)cdiv(s.nchunks, s.chunks_per);
+        // slices in chunks, the remainder spread over the first ones: the larger slices are dispatched first
+        const int base = (int)(s.nchunks / k), extra = (int)(s.nchunks % k);
+        s.ksplit = (int)k;
+        for (int i = 0; i < s.ksplit; i++) s.cb[i + 1] = s.cb[i] + base + (i < extra ? 1 : 0);
     }
     const long ospatial = (long)s.D * s.H * s.W * (s.mode ? 4 : 1);
     s.osize = (long)(s.mode ? s.F / 4 : s.F) * ospatial;
