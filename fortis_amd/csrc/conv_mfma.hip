@@ -477,8 +477,9 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     s.ksplit = 1;
     s.cb[0] = 0; s.cb[1] = s.nchunks;
     if (2 * wgs < 3 * conv_cus() && s.C >= 32) {
-        // volumes aim at three workgroups per CU (their chunks are long: 27 taps), images at two
-        long k = cdiv((KD == 3 ? 3L : 2L) * conv_cus(), wgs);
+        // volumes aim at three workgroups per CU (their chunks are long: 27 taps), images at one (measured on the
+        // UNet levels: a finer split costs more in partial sums than it gains in occupancy)
+        long k = cdiv((KD == 3 ? 3L : 1L) * conv_cus(), wgs);
         if (k > s.C / 16) k = s.C / 16;               // at least 16 input channels per split
         if (k > 16) k = 16;
         // slices in chunks, the remainder spread over the first ones: the larger slices are dispatched first
