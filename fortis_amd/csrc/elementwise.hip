@@ -5,6 +5,7 @@
 // fortis_pre_k / fortis_post_k, trt_backend/e3sm_boundary.cu:9-20, are one-thread-per-element and
 // strided on one side).
 #include "common.h"
+#include <type_traits>
 
 #define EW_THREADS 256
 
@@ -55,10 +56,45 @@ __global__ void transpose_kernel(const TI* __restrict__ src, TO* __restrict__ ds
         if (r < R && c < Cc) dst[c * R + r] = tile[threadIdx.x][y];
     }
 }
+// The same for fp32 on both sides with R and Cc multiples of 4 and 16-byte aligned arrays: 64 x 64 tiles, 256
+// threads, 16-byte loads along the source rows and 16-byte stores along the destination rows.
+template <typename F>
+__global__ __launch_bounds__(256) void transpose4_kernel(const float* __restrict__ src, float* __restrict__ dst, long R, long Cc, F f)
+{
+    __shared__ float tile[64][65];
+    const long c0 = (long)blockIdx.x * 64, r0 = (long)blockIdx.y * 64;
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int idx = tid + u * 256, row = idx >> 4, c4 = (idx & 15) * 4;
+        const long r = r0 + row, c = c0 + c4;
+        if (r < R && c < Cc) {
+            const float4 v = *(const float4*)(src + r * Cc + c);
+            tile[row][c4] = f(v.x, r, c); tile[row][c4 + 1] = f(v.y, r, c + 1);
+            tile[row][c4 + 2] = f(v.z, r, c + 2); tile[row][c4 + 3] = f(v.w, r, c + 3);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int idx = tid + u * 256, crow = idx >> 4, r4 = (idx & 15) * 4;
+        const long c = c0 + crow, r = r0 + r4;
+        if (r < R && c < Cc)
+            *(float4*)(dst + c * R + r) = make_float4(tile[r4][crow], tile[r4 + 1][crow], tile[r4 + 2][crow], tile[r4 + 3][crow]);
+    }
+}
+
 template <typename TI, typename TO, typename F>
 static void launch_transpose(const TI* src, TO* dst, long R, long Cc, F f, hipStream_t s)
 {
     if (R <= 0 || Cc <= 0) return;
+    if constexpr (std::is_same<TI, float>::value && std::is_same<TO, float>::value) {
+        if (R % 4 == 0 && Cc % 4 == 0 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+            hipLaunchKernelGGL((transpose4_kernel<F>), dim3((unsigned)cdiv(Cc, 64), (unsigned)cdiv(R, 64)), dim3(256), 0, s, src, dst, R, Cc, f);
+            HIP_OK(hipGetLastError());
+            return;
+        }
+    }
     hipLaunchKernelGGL((transpose_kernel<TI, TO, F>), dim3((unsigned)cdiv(Cc, 32), (unsigned)cdiv(R, 32)), dim3(32, 8), 0, s,
                        src, dst, R, Cc, f);
     HIP_OK(hipGetLastError());
