@@ -24,7 +24,7 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
     params_to_lds(&d, ST_THREADS);
     const int n = st_u(d.nrefs);
     const int tid = threadIdx.x;
-    const unsigned row0 = blockIdx.x * ST_THREADS, row = row0 + tid;
+    const unsigned row0 = st_xcd_band_block() * ST_THREADS, row = row0 + tid;
     if (row < rows) {
         int i, j, kk;
         st_row(d, row, i, j, kk);

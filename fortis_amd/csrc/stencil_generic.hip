@@ -180,7 +180,7 @@ __global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args
     const int n = st_u(d.nrefs), nins = st_u(d.nins);
     double (*r)[SG_THREADS] = (double (*)[SG_THREADS])sg_dyn;
     float* tile = (float*)(sg_dyn + (size_t)(nins + st_u(d.nscal)) * SG_THREADS);
-    const unsigned row0 = blockIdx.x * SG_THREADS, row = row0 + tid;
+    const unsigned row0 = st_xcd_band_block() * SG_THREADS, row = row0 + tid;
     if (row < rows) {
         int i, j, kk;
         st_row(d, row, i, j, kk);
