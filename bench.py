@@ -32,7 +32,7 @@ MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((2482.4 * 2 + 
                     "zb_unfused_1028x1028x15_f64": int((248700.0 * 2 + 1658880.0) * 1024),
                     # conv workloads: every conv, split-reduce and thin-head dispatch of a step summed, divided by the
                     # step's conv operations (18 and 19), like flop_per_launch
-                    "unet": int((1163560.2 * 2 + 727552.0) * 1024 / 7 / 18), "tsrgan": int((5122972.1 * 2 + 5358390.3) * 1024 / 7 / 19)}
+                    "unet": int((1163560.2 * 2 + 727552.0) * 1024 / 7 / 18), "tsrgan": int((3255367.7 * 2 + 5167927.1) * 1024 / 7 / 19)}
 
 
 def omp_threads():

@@ -87,6 +87,18 @@ void fortis_launch_boundary_post(const float* Y, void* B, long NI, long NK, cons
 void fortis_launch_permute(const float* src, float* dst, long C, long S, int to_channels_first, hipStream_t s);
 
 // ---- convolution family (conv.hip) ---------------------------------------------------------
+// Workgroups are dealt to the chip's eight XCDs round-robin (workgroup b of a row of the grid runs on XCD
+// (b + constant) % 8), each XCD with its own L2.  Kernels whose neighbouring workgroups read overlapping input
+// (stencil rows, conv halos and z-planes) number their work through this map, which gives each XCD a contiguous
+// band of the nb items instead of every eighth one (the last nb % 8 items keep their index).
+#ifdef __HIPCC__
+__device__ __forceinline__ unsigned fortis_xcd_band(unsigned b, unsigned nb)
+{
+    const unsigned per = nb / 8;
+    return b < per * 8 ? (b % 8) * per + b / 8 : b;
+}
+#endif
+
 struct ConvEpi {
     const float* scale;  // per output channel multiplier (folded BatchNorm), or null
     const float* shift;  // per output channel additive term (bias, folded BatchNorm), or null

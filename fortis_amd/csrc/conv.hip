@@ -138,7 +138,8 @@ __global__ __launch_bounds__(CONV_THREADS) void conv3d_thin_kernel(const float* 
     // its raw sums to y + k * F*D*H*W and a reduce kernel applies the epilogue
     extern __shared__ float ct_lds[];                       // [2][CT_CC][3][R] inputs
     const int tid = threadIdx.x;
-    const int z = blockIdx.x / tiles, tile = blockIdx.x - z * tiles;
+    const int bx = (int)fortis_xcd_band(blockIdx.x, gridDim.x);       // neighbouring tiles and planes on one XCD
+    const int z = bx / tiles, tile = bx - z * tiles;
     const int m0 = tile * CT_MT;
     const long HW = (long)H * W, chan = (long)D * HW;
     const int XCH = CT_CC * 3 * R;

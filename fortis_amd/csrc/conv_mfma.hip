@@ -77,7 +77,10 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     const int XCHP = (XCH + 63) / 64 * 64;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int z = blockIdx.x / s.tiles, tile = blockIdx.x - z * s.tiles;
+    // volumes: neighbouring tiles and planes on one XCD (input fetched once instead of 2-3 times; on images the
+    // banded order measured 2 % slower)
+    const int bx = KD == 3 ? (int)fortis_xcd_band(blockIdx.x, gridDim.x) : (int)blockIdx.x;
+    const int z = bx / s.tiles, tile = bx - z * s.tiles;
     const int fg = blockIdx.y;
     const int m0 = tile * MT;
     const int tyi = TILE2D ? tile / s.tiles_x : 0, y0 = tyi * TH, x0 = (tile - tyi * s.tiles_x) * 32;   // TILE2D: tile origin

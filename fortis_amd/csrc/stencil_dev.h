@@ -28,15 +28,7 @@ __device__ __forceinline__ void params_to_lds(T* dst, int nthreads)
     for (int i = threadIdx.x; i < (int)(sizeof(T) / 16); i += nthreads) ((float4*)dst)[i] = src[i];
     __syncthreads();
 }
-// Workgroups are dealt to the chip's eight XCDs round-robin (workgroup b runs on XCD b % 8), each XCD with its own
-// L2.  A stencil row is read by the workgroups of three neighbouring grid rows: with consecutive workgroups on
-// consecutive XCDs every input row is fetched from HBM by two L2s.  This map gives each XCD a contiguous band of
-// workgroups instead (the last gridDim % 8 workgroups keep their index).
-__device__ __forceinline__ unsigned st_xcd_band_block()
-{
-    const unsigned nb = gridDim.x, per = nb / 8, b = blockIdx.x;
-    return b < per * 8 ? (b % 8) * per + b / 8 : b;
-}
+__device__ __forceinline__ unsigned st_xcd_band_block() { return fortis_xcd_band(blockIdx.x, gridDim.x); }
 // A pointer read back from LDS has lost its address space; device arrays are global memory.
 typedef __attribute__((address_space(1))) float gfloat;
 __device__ __forceinline__ const gfloat* st_g(const float* p) { return (const gfloat*)p; }
