@@ -2,6 +2,8 @@
 // binding, and the host-facing entry points of the generated shim (driver/fortis_shim.py:54-135):
 // buffer ownership, upload/download choreography, pack/unpack staging, graph capture on the
 // second call and replay afterwards, with an eager fallback.
+#include <atomic>
+#include <thread>
 #include <vector>
 #include "common.h"
 
@@ -699,25 +701,97 @@ void mlp_forward_dev(void)
     }
 }
 
-void mlp_upload(void* in)
-{
-    if (!bound("mlp_upload")) return;
-    HIP_OK(hipMemcpyAsync(g_step.din, in, (size_t)g_step.h.n_in * g_step.h.in_esz, hipMemcpyHostToDevice, fortis_stream_get()));
-}
-void mlp_download(void* out)
-{
-    if (!bound("mlp_download")) return;
-    hipStream_t s = fortis_stream_get();
-    HIP_OK(hipMemcpyAsync(out, g_step.dout, (size_t)g_step.h.n_out * g_step.h.out_esz, hipMemcpyDeviceToHost, s));
-    HIP_OK(hipStreamSynchronize(s));
-}
-
 static void setup_xy()
 {
     // page-locked staging is allocated, never registered over existing host memory
     HIP_OK(hipHostMalloc(&g_step.X, (size_t)g_step.h.n_in * g_step.h.in_esz, hipHostMallocDefault));
     HIP_OK(hipHostMalloc(&g_step.Y, (size_t)g_step.h.n_out * g_step.h.out_esz, hipHostMallocDefault));
 }
+
+// ---- large host arrays: copies through page-locked staging, filled and drained by a few host threads --------
+// A copy straight from or to pageable host memory runs at about 20 GB/s here (the runtime stages it on one
+// thread) and existing host memory cannot be page-locked in place.  Arrays of 8 MB and more therefore go in
+// chunks through the page-locked staging buffers (g_step.X / g_step.Y): worker threads copy chunks between
+// the host array and staging while the DMA engine moves the chunks already copied.
+// FORTIS_NO_STAGED_COPY=1 keeps the plain copies.
+#define STAGE_CHUNK ((size_t)4 << 20)
+#define STAGE_THREADS 4
+static bool staged_copies(size_t n)
+{
+    return n >= 2 * STAGE_CHUNK && getenv("FORTIS_NO_STAGED_COPY") == nullptr;
+}
+static void staged_h2d(void* dev, const void* host, void* stage, size_t n, hipStream_t s)
+{
+    const size_t nchunks = (n + STAGE_CHUNK - 1) / STAGE_CHUNK;
+    std::atomic<size_t> next(0);
+    auto work = [&]() {
+        for (size_t c = next.fetch_add(1); c < nchunks; c = next.fetch_add(1)) {
+            const size_t o = c * STAGE_CHUNK, len = o + STAGE_CHUNK < n ? STAGE_CHUNK : n - o;
+            memcpy((char*)stage + o, (const char*)host + o, len);
+            HIP_OK(hipMemcpyAsync((char*)dev + o, (char*)stage + o, len, hipMemcpyHostToDevice, s));
+        }
+    };
+    std::thread th[STAGE_THREADS - 1];
+    for (auto& t : th) t = std::thread(work);
+    work();
+    for (auto& t : th) t.join();       // every chunk's copy is enqueued: what follows on the stream sees the whole array
+}
+static void staged_d2h(void* host, const void* dev, void* stage, size_t n, hipStream_t s)
+{
+    const size_t nchunks = (n + STAGE_CHUNK - 1) / STAGE_CHUNK;
+    static std::vector<hipEvent_t> ev;
+    while (ev.size() < nchunks) {
+        hipEvent_t e;
+        HIP_OK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        ev.push_back(e);
+    }
+    for (size_t c = 0; c < nchunks; c++) {
+        const size_t o = c * STAGE_CHUNK, len = o + STAGE_CHUNK < n ? STAGE_CHUNK : n - o;
+        HIP_OK(hipMemcpyAsync((char*)stage + o, (const char*)dev + o, len, hipMemcpyDeviceToHost, s));
+        HIP_OK(hipEventRecord(ev[c], s));
+    }
+    std::atomic<size_t> next(0);
+    auto work = [&]() {
+        for (size_t c = next.fetch_add(1); c < nchunks; c = next.fetch_add(1)) {
+            const size_t o = c * STAGE_CHUNK, len = o + STAGE_CHUNK < n ? STAGE_CHUNK : n - o;
+            HIP_OK(hipEventSynchronize(ev[c]));
+            memcpy((char*)host + o, (const char*)stage + o, len);
+        }
+    };
+    std::thread th[STAGE_THREADS - 1];
+    for (auto& t : th) t = std::thread(work);
+    work();
+    for (auto& t : th) t.join();
+}
+
+void mlp_upload(void* in)
+{
+    if (!bound("mlp_upload")) return;
+    const size_t n = (size_t)g_step.h.n_in * g_step.h.in_esz;
+    hipStream_t s = fortis_stream_get();
+    if (staged_copies(n)) {
+        if (!g_step.X) setup_xy();
+        // the staging buffer is reused: the previous call's chunks must have left it
+        HIP_OK(hipStreamSynchronize(s));
+        staged_h2d(g_step.din, in, g_step.X, n, s);
+        return;
+    }
+    HIP_OK(hipMemcpyAsync(g_step.din, in, n, hipMemcpyHostToDevice, s));
+}
+void mlp_download(void* out)
+{
+    if (!bound("mlp_download")) return;
+    hipStream_t s = fortis_stream_get();
+    const size_t n = (size_t)g_step.h.n_out * g_step.h.out_esz;
+    if (staged_copies(n)) {
+        if (!g_step.Y) setup_xy();
+        staged_d2h(out, g_step.dout, g_step.Y, n, s);
+        return;
+    }
+    HIP_OK(hipMemcpyAsync(out, g_step.dout, n, hipMemcpyDeviceToHost, s));
+    HIP_OK(hipStreamSynchronize(s));
+}
+
 void fortis_pack(void* row, int col)
 {
     if (!bound("fortis_pack")) return;

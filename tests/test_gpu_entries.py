@@ -40,6 +40,39 @@ def test_whole_array_call_and_resident_entries(L, gpu):
     assert bits_equal(y, y2)
 
 
+def test_whole_array_call_large_arrays(L, gpu, monkeypatch):
+    """Host arrays of 8 MB and more travel in chunks through page-locked staging, copied by several host threads:
+    the result must be the one of the plain copies (FORTIS_NO_STAGED_COPY=1), bit for bit, on arrays whose size
+    is not a multiple of the chunk; a sample of rows is checked against the oracle."""
+    rows = 41003
+    rng = np.random.default_rng(11)
+    Ws = [(rng.standard_normal((96, 64)) / 8).astype(np.float32), (rng.standard_normal((72, 96)) / 10).astype(np.float32)]
+    bs = [rng.standard_normal(96).astype(np.float32), rng.standard_normal(72).astype(np.float32)]
+    X = rng.standard_normal((rows, 64)).astype(np.float32)                 # 10.5 MB in, 11.8 MB out
+    plan = P.mlp_plan(Ws, bs, ["relu", None], rows)
+    ST.bind(plan, X.size, rows * 72)
+    y = np.zeros((rows, 72), np.float32)
+    ST.mlp_forward(X, y)
+    idx = rng.choice(rows, 256, replace=False)
+    assert maxrel(y[idx], O.mlp_f64(Ws, bs, ["relu", None], X[idx])) < TOL
+    y2 = np.zeros_like(y)
+    ST.mlp_upload(X)
+    ST.mlp_forward_dev()
+    ST.mlp_download(y2)
+    assert bits_equal(y, y2)
+    # a second call with other data reuses the staging buffers
+    X2 = rng.standard_normal((rows, 64)).astype(np.float32)
+    y3 = np.zeros_like(y)
+    ST.mlp_forward(X2, y3)
+    monkeypatch.setenv("FORTIS_NO_STAGED_COPY", "1")
+    ST.reset()
+    plan = P.mlp_plan(Ws, bs, ["relu", None], rows)
+    ST.bind(plan, X.size, rows * 72)
+    y4 = np.zeros_like(y)
+    ST.mlp_forward(X2, y4)
+    assert bits_equal(y3, y4) and not bits_equal(y3, y)
+
+
 def test_graph_capture_on_second_call_and_replay(L, gpu, monkeypatch):
     """fortis.graph set: call 1 eager, call 2 captures and launches, later calls replay
     (driver/fortis_shim.py:82-90).  Every replay must equal the eager result, with eager work and
