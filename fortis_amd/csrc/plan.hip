@@ -825,8 +825,12 @@ void mlp_forward_batched(void* in, void* out)
         return;
     }
     if (h.step == 1 && h.minc == 1) {
-        HIP_OK(hipMemcpyAsync(g_step.din, in, NIN * h.count, hipMemcpyHostToDevice, s));
+        const bool big_in = staged_copies(NIN * h.count), big_out = staged_copies(NOUT * h.count);
+        if ((big_in || big_out) && !g_step.X) setup_xy();
+        if (big_in) { HIP_OK(hipStreamSynchronize(s)); staged_h2d(g_step.din, in, g_step.X, NIN * h.count, s); }
+        else HIP_OK(hipMemcpyAsync(g_step.din, in, NIN * h.count, hipMemcpyHostToDevice, s));
         mlp_forward_dev();
+        if (big_out) { staged_d2h(out, g_step.dout, g_step.Y, NOUT * h.count, s); return; }
         HIP_OK(hipMemcpyAsync(out, g_step.dout, NOUT * h.count, hipMemcpyDeviceToHost, s));
         HIP_OK(hipStreamSynchronize(s));
         return;

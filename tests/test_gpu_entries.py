@@ -71,6 +71,14 @@ def test_whole_array_call_large_arrays(L, gpu, monkeypatch):
     y4 = np.zeros_like(y)
     ST.mlp_forward(X2, y4)
     assert bits_equal(y3, y4) and not bits_equal(y3, y)
+    # the batched slice form on the same arrays takes the same route
+    monkeypatch.delenv("FORTIS_NO_STAGED_COPY")
+    ST.reset()
+    plan = P.mlp_plan(Ws, bs, ["relu", None], rows)
+    ST.bind(plan, X.size, rows * 72, verdict="batched", count=rows, lo=1, step=1, minc=1)
+    y5 = np.zeros_like(y)
+    ST.mlp_forward_batched(X2, y5)
+    assert bits_equal(y5, y4)
 
 
 def test_graph_capture_on_second_call_and_replay(L, gpu, monkeypatch):
