@@ -230,3 +230,18 @@ def test_magic_divmod_is_exact():
         for n_ in (v for v in ns if 0 <= v < 2**32):
             L.fortis_magic_divmod(n_, d, C.byref(q), C.byref(r))
             assert (q.value, r.value) == (n_ // d, n_ % d), (n_, d)
+
+
+def test_bench_contract_without_a_gpu():
+    """bench.py refuses more than one GPU with a message (the path has no exchange step to measure), and its
+    measured-traffic table has an entry for every workload that reports a roofline against measured HBM bytes."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "ONE GPU" in (r.stderr + r.stdout)
+    sys.path.insert(0, root)
+    import bench
+    for key in ("climsim", "zb", "zb_ref", "zb_1028x1028x15", "zb_unfused_1028x1028x15", "zb_unfused_1028x1028x15_f64", "unet", "tsrgan"):
+        assert bench.MEASURED_TRAFFIC[key] > 0
+    assert bench.PEAK_HBM_GBS == 8000.0 and bench.PEAK_F32_MFMA_TFLOPS == 157.3
