@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 # same command (see profiles/), or None where no counter run has been made for the workload.
 MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((2482.4 * 2 + 936.6) * 1024),
                     "zb_ref": int((2396.6 * 2 + 936.6) * 1024), "zb_1028x1028x15": int((331322.2 * 2 + 207387.3) * 1024), "toy": None,
-                    "zb_unfused_1028x1028x15": int((123744.8 * 2 + 1658880.0) * 1024),
+                    "zb_unfused_1028x1028x15": int((242224.0 * 2 + 1658880.0) * 1024),
                     "zb_unfused_1028x1028x15_f64": int((248700.0 * 2 + 1658880.0) * 1024),
                     # conv workloads: every conv, split-reduce and thin-head dispatch of a step summed, divided by the
                     # step's conv operations (18 and 19), like flop_per_launch
