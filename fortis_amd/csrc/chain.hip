@@ -532,8 +532,14 @@ int fortis_chain_build(ChainDesc* d, int nlayers, const float* const* W, const f
         if (b && b[l]) memcpy(h + L.boff, b[l], L.N * sizeof(float));
     }
     float* dev = nullptr;
-    HIP_OK(hipMalloc((void**)&dev, total * sizeof(float)));
-    HIP_OK(hipMemcpy(dev, h, total * sizeof(float), hipMemcpyHostToDevice));
+    if (fortis_dev_malloc((void**)&dev, total * sizeof(float), "MLP chain weights") != 0) { free(h); return -1; }
+    if (hipMemcpy(dev, h, total * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        fprintf(stderr, "fortis: copying the MLP chain weights to the device failed\n");
+        fortis_dev_free(dev);
+        free(h);
+        return -1;
+    }
     free(h);
     d->nlayers = nlayers;
     d->wall = dev;

@@ -14,6 +14,13 @@
             fprintf(stderr, "fortis: %s failed: %s (%s:%d)\n", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
     } while (0)
 
+// Raw device memory for what the library keeps itself (weights, tables, staging planes): hipMalloc / hipFree
+// behind the same switchable allocator as the pool (fortis_pool_set_allocator), so that a test can make any of
+// these allocations fail.  fortis_dev_malloc returns 0, or -1 after printing what could not be allocated; a
+// caller that gets -1 must not launch anything on the pointer.
+int  fortis_dev_malloc(void** p, size_t nbytes, const char* what);
+void fortis_dev_free(void* p);
+
 extern "C" long fortis_step_generation(void);   // plan.hip: count of forward passes of the bound step
 static inline hipStream_t fortis_stream_get() { return (hipStream_t)mgpuStreamCreate(); }
 static inline long cdiv(long a, long b) { return (a + b - 1) / b; }
@@ -115,7 +122,7 @@ int fortis_launch_convt2d(const float* x, const float* w, float* y, long C, long
                           long ctot, hipStream_t s);
 int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long D, long H, long Wd, long F,
                          long KD, long KH, long KW, long Do, long Ho, long Wo, long pd, long ph, long pw,
-                         const ConvEpi& e, hipStream_t s);
+                         const ConvEpi& e, hipStream_t s, long sd = 1, long sh = 1, long sw = 1);
 // MFMA implicit-GEMM path (conv_mfma.hip).  kind 0: KD x KS x KS conv, pad KS/2, stride 1; kind 1: 2x2
 // stride-2 transposed conv.  wp: weights packed by fortis_conv_mfma_pack.  -1: shape not taken.
 float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats);

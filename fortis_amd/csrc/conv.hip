@@ -359,11 +359,12 @@ static int thin_cus()
 
 int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long D, long H, long Wd, long F, long KD,
                          long KH, long KW, long Do, long Ho, long Wo, long pd, long ph, long pw, const ConvEpi& e,
-                         hipStream_t s)
+                         hipStream_t s, long sd, long sh_, long sw_)
 {
-    if (!fits_int(C * D * H * Wd) || !fits_int(F * Do * Ho * Wo) || KD <= 0 || KH <= 0 || KW <= 0) return -1;
-    if (Do != D + 2 * pd - KD + 1 || Ho != H + 2 * ph - KH + 1 || Wo != Wd + 2 * pw - KW + 1) return -1;
-    if (KD == 3 && KH == 3 && KW == 3 && pd == 1 && ph == 1 && pw == 1 && F <= CT_F) {
+    if (!fits_int(C * D * H * Wd) || !fits_int(F * Do * Ho * Wo) || KD <= 0 || KH <= 0 || KW <= 0 || sd <= 0 || sh_ <= 0 || sw_ <= 0) return -1;
+    if (Do != (D + 2 * pd - KD) / sd + 1 || Ho != (H + 2 * ph - KH) / sh_ + 1 || Wo != (Wd + 2 * pw - KW) / sw_ + 1) return -1;
+    const bool unit = sd == 1 && sh_ == 1 && sw_ == 1;
+    if (unit && KD == 3 && KH == 3 && KW == 3 && pd == 1 && ph == 1 && pw == 1 && F <= CT_F) {
         const int P = (int)Wd + 1, plane = (int)H * P, tiles = (int)cdiv(plane, CT_MT), R = CT_MT + 2 * P + 2;
         const size_t shmem = (size_t)2 * CT_CC * 3 * R * sizeof(float);
         if (R <= CONV_THREADS * CT_NR && shmem <= 160 * 1024) {
@@ -398,8 +399,8 @@ int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long 
             return 0;
         }
     }
-    ConvShape sh = { (int)C, (int)D, (int)H, (int)Wd, (int)F, (int)KD, (int)KH, (int)KW, (int)Do, (int)Ho, (int)Wo, 1, 1, 1,
-                     (int)pd, (int)ph, (int)pw };
+    ConvShape sh = { (int)C, (int)D, (int)H, (int)Wd, (int)F, (int)KD, (int)KH, (int)KW, (int)Do, (int)Ho, (int)Wo, (int)sd,
+                     (int)sh_, (int)sw_, (int)pd, (int)ph, (int)pw };
     launch_direct(x, w, y, sh, e, Do * Ho * Wo, F, s);
     HIP_OK(hipGetLastError());
     return 0;

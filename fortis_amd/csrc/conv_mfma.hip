@@ -411,8 +411,14 @@ float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transpos
                             h[((fgi * nch + ch) * NCP + cp) * T * 2 * FT + ((long)t * 2 + hh) * FT + fl] = v;
                         }
     float* d = nullptr;
-    HIP_OK(hipMalloc((void**)&d, n * sizeof(float)));
-    HIP_OK(hipMemcpy(d, h, n * sizeof(float), hipMemcpyHostToDevice));
+    if (fortis_dev_malloc((void**)&d, n * sizeof(float), "packed conv weights") != 0) { free(h); return nullptr; }
+    if (hipMemcpy(d, h, n * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        fprintf(stderr, "fortis: copying packed conv weights to the device failed\n");
+        fortis_dev_free(d);
+        free(h);
+        return nullptr;
+    }
     free(h);
     if (nfloats) *nfloats = n;
     return d;
@@ -496,11 +502,12 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
         s.part = fortis_conv_split_scratch((size_t)s.ksplit * s.osize * sizeof(float));
         if (!s.part) return -1;
     }
+    // a shape is refused before anything is launched: -1 always means that nothing ran
+    const bool pooled = e.pool != nullptr;
+    if (pooled && (s.mode || s.D != 1 || (s.H & 1) || (s.W & 1) || (((uintptr_t)y | (uintptr_t)s.part) & 7))) return -1;   // the plan only asks for it on 2-D convs
     dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);
     hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
     HIP_OK(hipGetLastError());
-    const bool pooled = e.pool != nullptr;
-    if (pooled && (s.mode || s.D != 1 || (s.H & 1) || (s.W & 1) || (((uintptr_t)y | (uintptr_t)s.part) & 7))) return -1;   // the plan only asks for it on 2-D convs
     if (s.ksplit > 1 && pooled) {
         const long n = (long)s.F * (s.H / 2) * (s.W / 2);
         hipLaunchKernelGGL(conv_split_reduce_pool_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, st, s.part, y, e.pool, s.F, s.H, s.W,

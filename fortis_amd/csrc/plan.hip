@@ -52,7 +52,9 @@ struct fortis_plan {
     std::vector<Op> ops;
     std::vector<Exec> exec;
     std::vector<void*> owned;   // device allocations owned by the plan (weights, vectors)
+    std::vector<void*> bufs;    // distinct pool buffers behind the tensors (several tensors may share one)
     bool finalized = false;
+    bool upload_failed = false; // a weight / vector upload found no device memory
     int in_t = -1, out_t = -1;
     long rows0 = 0;             // rows at finalize (row-wise plans), for run-time extents
     int exec_skip = 0;          // ops folded into a neighbour at finalize
@@ -61,12 +63,19 @@ struct fortis_plan {
     size_t ev_used = 0;
 };
 
+// Host data -> a device allocation owned by the plan.  On failure (no memory, copy refused) returns null and
+// marks the plan: fortis_plan_finalize then fails, and a plan that is not finalized never launches.
 static void* upload(fortis_plan* p, const void* h, size_t nbytes)
 {
     void* d = nullptr;
-    HIP_OK(hipMalloc(&d, nbytes ? nbytes : 4));
-    if (nbytes) HIP_OK(hipMemcpy(d, h, nbytes, hipMemcpyHostToDevice));
+    if (fortis_dev_malloc(&d, nbytes, "plan weights") != 0) { p->upload_failed = true; return nullptr; }
     p->owned.push_back(d);
+    if (nbytes && hipMemcpy(d, h, nbytes, hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        fprintf(stderr, "fortis_plan: copying %zu bytes of weights to the device failed\n", nbytes);
+        p->upload_failed = true;
+        return nullptr;
+    }
     return d;
 }
 
@@ -82,8 +91,8 @@ fortis_plan* fortis_plan_create(void) { return new fortis_plan(); }
 void fortis_plan_destroy(fortis_plan* p)
 {
     if (!p) return;
-    for (void* d : p->owned) HIP_OK(hipFree(d));
-    for (size_t t = 0; t < p->tptr.size(); t++) if (p->view_of[t] < 0) fortis_free(p->tptr[t]);
+    for (void* d : p->owned) fortis_dev_free(d);
+    for (void* b : p->bufs) fortis_free(b);
     delete p;
 }
 int fortis_plan_tensor(fortis_plan* p, long nbytes)
@@ -323,6 +332,56 @@ static size_t try_chain(fortis_plan* p, size_t i, Exec* ex)
     return j - i;
 }
 
+// Gives every tensor its device buffer by walking the kernels in launch order the way the reference's generated
+// host code does at run time (compiler/FortisFuse.cpp:512-516: a temporary is taken from the pool in front of
+// the group that first writes it and handed back behind the group that last reads it), so that temporaries
+// whose lifetimes do not overlap share a pool buffer and a deep stack holds two or three activations instead of
+// all of them.  The walk happens once, here: the pointers are then fixed for the life of the plan (a captured
+// graph names them) and every buffer the walk touched stays marked in use in the pool until the plan is
+// destroyed.  The model's input and output, and tensors no kernel writes (filled by the caller), keep their
+// buffer throughout; a tensor no kernel touches (folded into a neighbour at fusion) gets none.
+void fortis_pool_hold(void* p);   // rt.hip: marks a pool buffer in use again
+static int assign_buffers(fortis_plan* p)
+{
+    const int nt = (int)p->tbytes.size(), ne = (int)p->exec.size();
+    const int never = ne + 1;
+    std::vector<int> first(nt, never), last(nt, -2);
+    auto base = [&](int t) { return p->view_of[t] >= 0 ? p->view_of[t] : t; };
+    auto reads = [&](int t, int i) { if (t < 0) return; t = base(t); if (first[t] == never) first[t] = -1; if (last[t] < i) last[t] = i; };
+    auto writes = [&](int t, int i) { if (t < 0) return; t = base(t); if (first[t] > i) first[t] = i; if (last[t] < i) last[t] = i; };
+    for (int i = 0; i < ne; i++) {
+        const Exec& e = p->exec[i];
+        reads(e.src, i); reads(e.res, i);
+        writes(e.dst, i); writes(e.pool_dst, i);
+    }
+    for (int t = 0; t < nt; t++) if (first[t] == -1) last[t] = ne;          // filled by the caller: never handed back
+    first[base(p->in_t)] = -1; last[base(p->in_t)] = ne;
+    if (first[base(p->out_t)] == never) first[base(p->out_t)] = -1;
+    last[base(p->out_t)] = ne;
+    for (void* b : p->bufs) fortis_free(b);
+    p->bufs.clear();
+    p->tptr.assign(nt, nullptr);
+    int rc = 0;
+    auto take = [&](int t) {
+        void* d = fortis_alloc(p->tbytes[t]);
+        if (!d) { rc = -1; return; }
+        p->tptr[t] = d;
+        bool seen = false;
+        for (void* b : p->bufs) if (b == d) seen = true;
+        if (!seen) p->bufs.push_back(d);
+    };
+    for (int t = 0; t < nt && rc == 0; t++) if (p->view_of[t] < 0 && first[t] == -1) take(t);
+    for (int i = 0; i < ne && rc == 0; i++) {
+        for (int t = 0; t < nt && rc == 0; t++) if (p->view_of[t] < 0 && first[t] == i) take(t);
+        for (int t = 0; t < nt; t++) if (p->view_of[t] < 0 && last[t] == i && p->tptr[t]) fortis_free(p->tptr[t]);
+    }
+    for (void* b : p->bufs) fortis_pool_hold(b);
+    if (rc != 0) return -1;
+    for (int t = 0; t < nt; t++)
+        if (p->view_of[t] >= 0 && p->tptr[p->view_of[t]]) p->tptr[t] = (char*)p->tptr[p->view_of[t]] + p->view_off[t];
+    return 0;
+}
+
 extern "C" {
 
 int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
@@ -331,13 +390,6 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
     if (in_t < 0 || in_t >= (int)p->tbytes.size() || out_t < 0 || out_t >= (int)p->tbytes.size()) return bad("finalize: bad input/output tensor");
     if (p->ops.empty()) return bad("finalize: empty plan");
     p->in_t = in_t; p->out_t = out_t;
-    (void)fortis_stream_get();
-    for (size_t t = 0; t < p->tbytes.size(); t++) {
-        if (p->view_of[t] >= 0) { p->tptr.push_back((char*)p->tptr[p->view_of[t]] + p->view_off[t]); continue; }
-        void* d = fortis_alloc(p->tbytes[t]);
-        if (!d) return bad("finalize: out of device memory");
-        p->tptr.push_back(d);
-    }
     const std::vector<Op>& ops = p->ops;
     int fuse_ups_src = -1;      // source tensor of an upsample folded into the convolution that follows
     for (size_t i = 0; i < ops.size();) {
@@ -416,7 +468,7 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                 else { ok = o.KH == 2 && o.KW == 2 && o.stride == 2 && o.pad == 0 && o.opad == 0; T = 1; tr = 1; }
                 if (ok && wide && !direct_only) {
                     float* wp = fortis_conv_mfma_pack(o.w.data(), o.F, o.C, T, tr, nullptr);
-                    p->owned.push_back(wp);
+                    if (!wp) p->upload_failed = true; else p->owned.push_back(wp);
                     ex.Wmfma = wp;
                 }
                 // A 2 x 2 max pool that directly follows and reads this conv's whole output is written by the conv's
@@ -462,6 +514,9 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
         if (rows < 0) rows = e.rows; else if (rows != e.rows) rowwise = false;
     }
     p->rows0 = rowwise ? rows : 0;
+    if (p->upload_failed) return bad("finalize: out of device memory for the weights");
+    if (assign_buffers(p) != 0) return bad("finalize: out of device memory for the activations");
+    (void)fortis_stream_get();
     p->finalized = true;
     HIP_OK(hipDeviceSynchronize());
     return 0;
@@ -578,10 +633,25 @@ int fortis_plan_as_chain(fortis_plan* p, ChainDesc* out)
     return 0;
 }
 
-// Run-time extents: row-wise plans can be re-run on fewer rows than they were sized for.
+// Run-time extents: a row-wise plan runs on any row count.  Up to the rows its buffers were sized for only
+// the launch extents change; beyond that every tensor grows in proportion and the buffers are assigned anew
+// (the weights do not depend on the row count).  Plans with tensor windows keep their size.
 static int plan_set_rows(fortis_plan* p, long rows)
 {
-    if (!p || !p->finalized || p->rows0 <= 0 || rows <= 0 || rows > p->rows0) return -1;
+    if (!p || !p->finalized || p->rows0 <= 0 || rows <= 0) return -1;
+    if (rows > p->rows0) {
+        for (int v : p->view_of) if (v >= 0) return -1;
+        std::vector<long> old(p->tbytes);
+        for (long& b : p->tbytes) b = (long)(((__int128)b * rows + p->rows0 - 1) / p->rows0);
+        HIP_OK(hipStreamSynchronize(fortis_stream_get()));      // nothing in flight may still use the old buffers
+        if (assign_buffers(p) != 0) {
+            p->tbytes = old;
+            if (assign_buffers(p) != 0) { fprintf(stderr, "fortis_plan: could not restore the plan's buffers\n"); p->finalized = false; }
+            return -1;
+        }
+        p->rows0 = rows;
+        for (Exec& e : p->exec) e.rows_cap = rows;
+    }
     for (Exec& e : p->exec) e.rows = rows;
     return 0;
 }
@@ -654,7 +724,16 @@ void mlp_forward_dev(void)
     g_forward_gen++;
     hipStream_t s = fortis_stream_get();
     if (g_step.gexec) { HIP_OK(hipGraphLaunch(g_step.gexec, s)); return; }
-    const int cap = (++g_step.ncalls == 2) && (g_step.h.graph || getenv("FORTIS_GRAPH") != 0);
+    // Replay pays on this runtime only for steps of several kernels: one graph launch costs about as much as
+    // five plain launches here (the opposite of the CUDA case FORTIS_GRAPH was built for), so a step of fewer
+    // than FORTIS_GRAPH_MIN_KERNELS kernels (default 6) keeps running eagerly.  The rule depends on the plan
+    // alone, never on timing, and no extra forward pass runs inside a caller's call.  FORTIS_GRAPH_KEEP in the
+    // environment captures whatever the step's length.
+    static int min_kernels = -1;
+    if (min_kernels < 0) { const char* e = getenv("FORTIS_GRAPH_MIN_KERNELS"); min_kernels = e ? atoi(e) : 6; }
+    const bool wanted = g_step.h.graph || getenv("FORTIS_GRAPH") != 0;
+    const bool pays = (int)g_step.plan->exec.size() >= min_kernels || getenv("FORTIS_GRAPH_KEEP") != 0;
+    const int cap = (++g_step.ncalls == 2) && wanted && pays;
     if (cap) {
         fortis_capturing = 1;
         if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) {
@@ -671,26 +750,6 @@ void mlp_forward_dev(void)
         fortis_capturing = 0;
         if (hipStreamEndCapture(s, &g) == hipSuccess && g && hipGraphInstantiate(&g_step.gexec, g, nullptr, nullptr, 0) == hipSuccess) {
             HIP_OK(hipGraphLaunch(g_step.gexec, s));
-            // Replay is kept only if it is measured to be no slower than launching the kernels one by one:
-            // on this runtime a graph launch costs more than a few plain launches, so short steps are
-            // faster eager.  The step is a pure function of the resident input, so the trial passes change
-            // nothing.  FORTIS_GRAPH_KEEP in the environment keeps the replay unconditionally.
-            if (!getenv("FORTIS_GRAPH_KEEP")) {
-                const int trials = 3;
-                hipEvent_t e0, e1, e2;
-                HIP_OK(hipEventCreate(&e0)); HIP_OK(hipEventCreate(&e1)); HIP_OK(hipEventCreate(&e2));
-                HIP_OK(hipEventRecord(e0, s));
-                for (int i = 0; i < trials; i++) HIP_OK(hipGraphLaunch(g_step.gexec, s));
-                HIP_OK(hipEventRecord(e1, s));
-                for (int i = 0; i < trials; i++) fortis_plan_run(g_step.plan);
-                HIP_OK(hipEventRecord(e2, s));
-                HIP_OK(hipEventSynchronize(e2));
-                float replay_ms = 0.f, eager_ms = 0.f;
-                HIP_OK(hipEventElapsedTime(&replay_ms, e0, e1));
-                HIP_OK(hipEventElapsedTime(&eager_ms, e1, e2));
-                HIP_OK(hipEventDestroy(e0)); HIP_OK(hipEventDestroy(e1)); HIP_OK(hipEventDestroy(e2));
-                if (replay_ms > eager_ms) { HIP_OK(hipGraphExecDestroy(g_step.gexec)); g_step.gexec = nullptr; }
-            }
         } else {
             fprintf(stderr, "fortis: graph capture failed, running eagerly\n");
             g_step.gexec = nullptr;
@@ -703,9 +762,14 @@ void mlp_forward_dev(void)
 
 static void setup_xy()
 {
-    // page-locked staging is allocated, never registered over existing host memory
-    HIP_OK(hipHostMalloc(&g_step.X, (size_t)g_step.h.n_in * g_step.h.in_esz, hipHostMallocDefault));
-    HIP_OK(hipHostMalloc(&g_step.Y, (size_t)g_step.h.n_out * g_step.h.out_esz, hipHostMallocDefault));
+    // page-locked staging is allocated, never registered over existing host memory; without it the entries that
+    // stage cannot run at all, which ends the program like the reference's failed specialisation does
+    if (hipHostMalloc(&g_step.X, (size_t)g_step.h.n_in * g_step.h.in_esz, hipHostMallocDefault) != hipSuccess ||
+        hipHostMalloc(&g_step.Y, (size_t)g_step.h.n_out * g_step.h.out_esz, hipHostMallocDefault) != hipSuccess) {
+        fprintf(stderr, "fortis: no page-locked host memory for the staging buffers (%ld + %ld bytes)\n",
+                g_step.h.n_in * g_step.h.in_esz, g_step.h.n_out * g_step.h.out_esz);
+        exit(1);
+    }
 }
 
 // ---- large host arrays: copies through page-locked staging, filled and drained by a few host threads --------
@@ -898,15 +962,26 @@ void fortis_begin(int count)
 {
     if (!bound("fortis_begin")) return;
     fortis_host_t& h = g_step.h;
-    if (h.verdict != FORTIS_VERDICT_BATCHED || count <= 0 || count > g_step.count0) {
-        fprintf(stderr, "fortis_begin: %d rows do not fit the bound step (at most %ld)\n", count, g_step.count0);
+    if (h.verdict != FORTIS_VERDICT_BATCHED || count <= 0) {
+        fprintf(stderr, "fortis_begin: %d rows cannot be specialised (the bound step is %s)\n", count,
+                h.verdict != FORTIS_VERDICT_BATCHED ? "not a batched build" : "batched");
         exit(1);   // the reference stub exits when it cannot specialise (driver/fortis_stub.c:23)
     }
     if (count == h.count) return;
-    const long per = g_step.plan->rows0 / g_step.count0;   // rows per cell (enclosing-loop distribution)
+    const long per = g_step.plan->rows0 / g_step.count0;   // model rows per cell (enclosing-loop distribution)
+    const long nin_row = h.n_in / g_step.count0, nout_row = h.n_out / g_step.count0;
     if (plan_set_rows(g_step.plan, (long)count * per) != 0) {
-        fprintf(stderr, "fortis_begin: the bound model is not row-wise, cannot change its extent\n");
+        fprintf(stderr, "fortis_begin: the bound model cannot be re-sized to %d rows (not row-wise, tensor windows, or out of memory)\n", count);
         exit(1);
+    }
+    if (count > g_step.count0) {
+        // the step grew: its buffers moved and the host-side staging is too small
+        g_step.count0 = count;
+        h.n_in = nin_row * count; h.n_out = nout_row * count;
+        g_step.din = g_step.plan->tptr[g_step.plan->in_t];
+        g_step.dout = g_step.plan->tptr[g_step.plan->out_t];
+        if (g_step.X) { HIP_OK(hipHostFree(g_step.X)); g_step.X = nullptr; }
+        if (g_step.Y) { HIP_OK(hipHostFree(g_step.Y)); g_step.Y = nullptr; }
     }
     h.count = count;
     drop_graph();

@@ -38,6 +38,24 @@ static fortis_raw_alloc_fn g_alloc = dev_alloc;
 static fortis_raw_free_fn g_free = dev_free;
 static struct { long n; void* p; int used; } g_pool[FORTIS_POOL];
 
+int fortis_dev_malloc(void** p, size_t nbytes, const char* what)
+{
+    *p = nullptr;
+    if (g_alloc(p, nbytes ? nbytes : 4) == 0 && *p) return 0;
+    if (g_alloc == dev_alloc) (void)hipGetLastError();
+    *p = nullptr;
+    fprintf(stderr, "fortis: device allocation of %zu bytes failed (%s)\n", nbytes, what);
+    return -1;
+}
+void fortis_dev_free(void* p) { if (p) g_free(p); }
+
+// A buffer the pool handed out earlier and has since taken back is claimed again by its address (the plan
+// fixes its buffers once and keeps them while it lives).  A pointer the pool does not hold is ignored.
+void fortis_pool_hold(void* p)
+{
+    for (int i = 0; i < FORTIS_POOL; i++) if (g_pool[i].p == p) { g_pool[i].used = 1; return; }
+}
+
 extern "C" {
 // Test hook: replaces the raw allocator (null restores hipMalloc/hipFree) and empties the pool table.
 void fortis_pool_set_allocator(fortis_raw_alloc_fn a, fortis_raw_free_fn f)
@@ -137,30 +155,42 @@ void fortis_conv2d(float* xa, float* x, long xo, long x0, long x1, long x2, long
     }
 }
 
-static void conv3d_any(const char* who, float* x, long xo, float* w, long wo, float* y, long yo, long N, long C,
+// fortis_conv3d takes what the reference's library path takes (runtime/fortis_rt.c:128-156): any batch, any
+// stride.  The direct and large-kernel entries keep the reference's own limits (N = 1, stride 1;
+// runtime/fortis_fft.cu:70, 135).
+static void conv3d_any(const char* who, bool general, float* x, long xo, float* w, long wo, float* y, long yo, long N, long C,
                        long Din, long Hin, long Win, long F, long KD, long KH, long KW, long Dout, long Hout,
                        long Wout, long sd, long sh, long sw, long pd, long ph, long pw)
 {
-    if (N != 1 || sd != 1 || sh != 1 || sw != 1) { fprintf(stderr, "%s: unsupported shape\n", who); return; }
-    if (KD == 3 && KH == 3 && KW == 3 && pd == 1 && ph == 1 && pw == 1 && Dout == Din && Hout == Hin && Wout == Win &&
-        conv_entry_mfma(x + xo, w + wo, y + yo, C, Din, Hin, Win, F, 3, 3) == 0)
-        return;
-    ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
-    if (fortis_launch_conv3d(x + xo, w + wo, y + yo, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, pd, ph, pw, e,
-                             fortis_stream_get()) != 0)
-        fprintf(stderr, "%s: unsupported shape\n", who);
+    const bool unit = sd == 1 && sh == 1 && sw == 1;
+    if (!general && (N != 1 || !unit)) { fprintf(stderr, "%s: unsupported shape\n", who); return; }
+    const long xn = C * Din * Hin * Win, yn = F * Dout * Hout * Wout;
+    for (long n = 0; n < N; n++) {
+        float* xb = x + xo + n * xn;
+        float* yb = y + yo + n * yn;
+        if (unit && KD == 3 && KH == 3 && KW == 3 && pd == 1 && ph == 1 && pw == 1 && Dout == Din && Hout == Hin && Wout == Win &&
+            conv_entry_mfma(xb, w + wo, yb, C, Din, Hin, Win, F, 3, 3) == 0)
+            continue;
+        ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
+        if (fortis_launch_conv3d(xb, w + wo, yb, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, pd, ph, pw, e,
+                                 fortis_stream_get(), sd, sh, sw) != 0) {
+            fprintf(stderr, "%s: unsupported shape\n", who);
+            return;
+        }
+    }
 }
 #define CONV3D_FWD(who)                                                                                             \
     (void)xa; (void)x0; (void)x1; (void)x2; (void)x3; (void)x4; (void)xt0; (void)xt1; (void)xt2; (void)xt3; (void)xt4; \
     (void)wa; (void)w0; (void)w1; (void)w2; (void)w3; (void)w4; (void)wt0; (void)wt1; (void)wt2; (void)wt3; (void)wt4; \
     (void)ya; (void)y0; (void)y1; (void)y2; (void)y3; (void)y4; (void)yt0; (void)yt1; (void)yt2; (void)yt3; (void)yt4; \
-    conv3d_any(who, x, xo, w, wo, y, yo, N, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, sd, sh, sw, pd, ph, pw)
+    conv3d_any(who, general, x, xo, w, wo, y, yo, N, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, sd, sh, sw, pd, ph, pw)
 
-void fortis_conv3d(FORTIS_CONV3D_ARGS) { CONV3D_FWD("fortis_conv3d"); }
-void fortis_conv3d_direct(FORTIS_CONV3D_ARGS) { CONV3D_FWD("fortis_conv3d_direct"); }
+void fortis_conv3d(FORTIS_CONV3D_ARGS) { const bool general = true; CONV3D_FWD("fortis_conv3d"); }
+void fortis_conv3d_direct(FORTIS_CONV3D_ARGS) { const bool general = false; CONV3D_FWD("fortis_conv3d_direct"); }
 void fortis_conv3d_fft(FORTIS_CONV3D_ARGS)
 {
     if (pd || ph || pw) { fprintf(stderr, "fortis_conv3d_fft: unsupported shape\n"); return; }
+    const bool general = false;
     CONV3D_FWD("fortis_conv3d_fft");
 }
 

@@ -12,6 +12,7 @@
 //            block of 256 x n floats (a row-per-thread store would touch n cache lines per lane).
 //   scatter: thread = cell; Y rows staged through LDS the same way in reverse; plane stores
 //            are coalesced along i.
+#include <vector>
 #include "stencil_dev.h"
 
 #define ST_THREADS 256
@@ -202,14 +203,62 @@ struct BoundStencil {
 };
 static BoundStencil g_gather, g_scatter;
 
-// Returns the table's route (see route_table) after copying its cell list to the device.
+// Device copies of cell lists, shared by content: the gather and the scatter table of one step name the same
+// cells, and with ONE device copy behind both the fused kernel sees equal list pointers and decodes a row once.
+struct CellList { unsigned long long hash; long count; int* d; int users; };
+static CellList g_lists[32];
+static unsigned long long cells_hash(const int* c, long n)
+{
+    unsigned long long h = 1469598103934665603ULL;
+    for (long i = 0; i < n; i++) { h ^= (unsigned)c[i]; h *= 1099511628211ULL; }
+    return h;
+}
+static int* cells_acquire(const int* host, long count)
+{
+    const unsigned long long h = cells_hash(host, count);
+    CellList* slot = nullptr;
+    std::vector<int> tmp;
+    for (CellList& l : g_lists) {
+        if (!l.d) { if (!slot) slot = &l; continue; }
+        if (l.hash != h || l.count != count) continue;
+        // same hash: compare the contents before sharing
+        if (tmp.empty()) tmp.resize((size_t)count);
+        if (hipMemcpy(tmp.data(), l.d, (size_t)count * sizeof(int), hipMemcpyDeviceToHost) == hipSuccess &&
+            !memcmp(tmp.data(), host, (size_t)count * sizeof(int))) { l.users++; return l.d; }
+        (void)hipGetLastError();
+    }
+    int* d = nullptr;
+    if (fortis_dev_malloc((void**)&d, (size_t)count * sizeof(int), "stencil cell list") != 0) return nullptr;
+    if (hipMemcpy(d, host, (size_t)count * sizeof(int), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError();
+        fprintf(stderr, "fortis: copying the stencil cell list to the device failed\n");
+        fortis_dev_free(d);
+        return nullptr;
+    }
+    if (slot) { slot->hash = h; slot->count = count; slot->d = d; slot->users = 1; }   // no free slot: an unshared copy
+    return d;
+}
+static void cells_release(int* d)
+{
+    if (!d) return;
+    for (CellList& l : g_lists)
+        if (l.d == d) {
+            if (--l.users > 0) return;
+            l.d = nullptr;
+            break;
+        }
+    fortis_dev_free(d);
+}
+
+// Returns the table's route (see route_table) after copying its cell list to the device; -1 also when the
+// list found no device memory (nothing may then be launched on the table).
 static int upload_table(const fortis_stencil_t* t, StencilDev* low, int** dcells)
 {
     const int route = route_table(t, low);
     if (route < 0) return -1;
     if (t->cells) {
-        HIP_OK(hipMalloc((void**)dcells, t->count * sizeof(int)));
-        HIP_OK(hipMemcpy(*dcells, t->cells, t->count * sizeof(int), hipMemcpyHostToDevice));
+        *dcells = cells_acquire(t->cells, t->count);
+        if (!*dcells) return -1;
         if (route == 0) low->cells = *dcells;
     }
     return route;
@@ -217,9 +266,9 @@ static int upload_table(const fortis_stencil_t* t, StencilDev* low, int** dcells
 
 static void release(BoundStencil& b)
 {
-    if (b.dcells) HIP_OK(hipFree(b.dcells));
+    cells_release(b.dcells);
     for (int a = 0; a < FORTIS_MAX_ARRAYS; a++)
-        if (b.darr[a]) { if (b.host_planes) HIP_OK(hipHostFree(b.darr[a])); else HIP_OK(hipFree(b.darr[a])); }
+        if (b.darr[a]) { if (b.host_planes) HIP_OK(hipHostFree(b.darr[a])); else fortis_dev_free(b.darr[a]); }
     for (int a = 0; a < FORTIS_MAX_ARRAYS; a++) if (b.sall[a]) HIP_OK(hipHostFree(b.sall[a]));
     b = BoundStencil();
 }
@@ -251,7 +300,9 @@ void fortis_stencil_reset_internal()
 }
 
 // cache of device tables for the device-resident API (keyed by table contents)
-struct CacheEnt { fortis_stencil_t key; const int* cells_key; int* dcells; StencilDev low; bool generic; };
+// A table with a cell list is matched by the list's contents too (a host copy is kept for the comparison, a few
+// microseconds for some thousand cells): a caller may free a list and build another at the same address.
+struct CacheEnt { fortis_stencil_t key; std::vector<int> cells_key; int* dcells; StencilDev low; bool generic; };
 static CacheEnt g_cache[16];
 static int g_ncache = 0;
 static CacheEnt* cached(const fortis_stencil_t* t)
@@ -259,7 +310,8 @@ static CacheEnt* cached(const fortis_stencil_t* t)
     for (int i = 0; i < g_ncache; i++) {
         fortis_stencil_t a = g_cache[i].key, b = *t;
         a.cells = b.cells = nullptr;
-        if (!memcmp(&a, &b, sizeof a) && g_cache[i].cells_key == t->cells) return &g_cache[i];
+        if (memcmp(&a, &b, sizeof a) || (t->cells != nullptr) != !g_cache[i].cells_key.empty()) continue;
+        if (!t->cells || !memcmp(g_cache[i].cells_key.data(), t->cells, (size_t)t->count * sizeof(int))) return &g_cache[i];
     }
     CacheEnt* e;
     const bool evict = g_ncache == 16;
@@ -269,7 +321,7 @@ static CacheEnt* cached(const fortis_stencil_t* t)
         e = &g_cache[victim];
         victim = (victim + 1) % 16;
         HIP_OK(hipStreamSynchronize(fortis_stream_get()));
-        if (e->dcells) HIP_OK(hipFree(e->dcells));
+        cells_release(e->dcells);
         e->key.narrays = -1;            // matches no table until it is filled again
     } else {
         e = &g_cache[g_ncache];
@@ -279,7 +331,8 @@ static CacheEnt* cached(const fortis_stencil_t* t)
     if (route < 0) return nullptr;
     e->generic = route == 1;
     e->key = *t;
-    e->cells_key = t->cells;
+    e->cells_key.clear();
+    if (t->cells) e->cells_key.assign(t->cells, t->cells + t->count);
     if (!evict) g_ncache++;
     return e;
 }
@@ -340,8 +393,8 @@ void fortis_gather_v(const int* a, const void* const* H)
     const fortis_stencil_t& t = b.host;
     const bool kdist = t.nk > 1;
     if (!b.init) {
-        for (int ai = 0; ai < t.narrays; ai++)
-            HIP_OK(hipMalloc(&b.darr[ai], (size_t)t.plane[ai] * t.nk * esz_of(t, ai)));   // gather.cu:8-11
+        for (int ai = 0; ai < t.narrays; ai++)   // gather.cu:8-11
+            if (!b.darr[ai] && fortis_dev_malloc(&b.darr[ai], (size_t)t.plane[ai] * t.nk * esz_of(t, ai), "gather planes") != 0) return;
         b.init = true;
     }
     const float* dptr[FORTIS_MAX_ARRAYS];
@@ -375,8 +428,14 @@ void fortis_scatter_v(const int* a, void* const* H)
     // per call (gather.cu:84-90); as copy commands from and to pageable memory those cost far more than the
     // kernel here (a pitched download is handled row by row).
     if (!b.init) {
-        for (int ai = 0; ai < t.narrays; ai++) HIP_OK(hipHostMalloc(&b.darr[ai], (size_t)t.plane[ai] * esz_of(t, ai), hipHostMallocDefault));
         b.host_planes = true;
+        for (int ai = 0; ai < t.narrays; ai++)
+            if (!b.darr[ai] && hipHostMalloc(&b.darr[ai], (size_t)t.plane[ai] * esz_of(t, ai), hipHostMallocDefault) != hipSuccess) {
+                (void)hipGetLastError();
+                b.darr[ai] = nullptr;
+                fprintf(stderr, "fortis_scatter: no page-locked memory for the staging planes\n");
+                return;
+            }
         b.init = true;
     }
     const int k1 = a ? a[0] : 1;   // 1-based enclosing-loop index
@@ -400,7 +459,12 @@ void fortis_scatter_v(const int* a, void* const* H)
         if (idx == 0) {
             float* sp[FORTIS_MAX_ARRAYS];
             for (int ai = 0; ai < t.narrays; ai++) {
-                if (!b.sall[ai]) HIP_OK(hipHostMalloc(&b.sall[ai], (size_t)planes(ai) * pelems(ai) * sizeof(float), hipHostMallocDefault));
+                if (!b.sall[ai] && hipHostMalloc(&b.sall[ai], (size_t)planes(ai) * pelems(ai) * sizeof(float), hipHostMallocDefault) != hipSuccess) {
+                    (void)hipGetLastError();
+                    b.sall[ai] = nullptr;
+                    fprintf(stderr, "fortis_scatter: no page-locked memory for the staging planes\n");
+                    return;
+                }
                 sp[ai] = (float*)b.sall[ai];
                 if (!b.written[ai]) {
                     const long off = t.total[ai] > t.plane[ai] ? (long)(t.klo - 1) * t.plane[ai] : 0;

@@ -174,7 +174,7 @@ __device__ __forceinline__ void sg_load_slots(const GenArgs& d, float* mine, int
 __global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args, float* __restrict__ X, unsigned rows)
 {
     __shared__ GenArgs d;
-    extern __shared__ double sg_dyn[];
+    extern __shared__ __attribute__((aligned(16))) double sg_dyn[];
     params_to_lds(&d, SG_THREADS);
     const int tid = threadIdx.x;
     const int n = st_u(d.nrefs), nins = st_u(d.nins);
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args
 __global__ __launch_bounds__(SG_THREADS) void scatter_generic_kernel(GenArgs args, const float* __restrict__ Y, int kk)
 {
     __shared__ GenArgs d;
-    extern __shared__ double sg_dyn[];
+    extern __shared__ __attribute__((aligned(16))) double sg_dyn[];
     params_to_lds(&d, SG_THREADS);
     double (*r)[SG_THREADS] = (double (*)[SG_THREADS])sg_dyn;
     const int tid = threadIdx.x;
@@ -258,6 +258,16 @@ int fortis_stencil_validate(const fortis_stencil_t* t)
     for (int r = 0; r < t->nrefs + t->nscal; r++) {
         const fortis_ref_t& f = r < t->nrefs ? t->refs[r] : t->scal[r - t->nrefs];
         if (f.array < 0 || f.array >= t->narrays) { fprintf(stderr, "fortis: stencil ref names array %d\n", f.array); return -1; }
+    }
+    // An array with a plane per enclosing-loop iteration must hold the nk planes starting at klo: the host-array
+    // entries copy exactly those, and the kernels index them.
+    for (int a = 0; a < t->narrays; a++) {
+        if (t->plane[a] < 1 || t->total[a] < t->plane[a]) { fprintf(stderr, "fortis: stencil array %d has %ld elements in planes of %ld\n", a, t->total[a], t->plane[a]); return -1; }
+        if (t->total[a] > t->plane[a] && ((long)(t->klo > 1 ? t->klo : 1) - 1 + t->nk) * t->plane[a] > t->total[a]) {
+            fprintf(stderr, "fortis: stencil array %d holds %ld elements, fewer than the %d planes of %ld from iteration %d on\n",
+                    a, t->total[a], t->nk, t->plane[a], t->klo > 1 ? t->klo : 1);
+            return -1;
+        }
     }
     // Every element a kernel will touch must lie inside its array's plane: base + i*si + j*sj in [0, plane) for
     // every visited cell (the plane index kk only adds whole planes).  A descriptor that fails this would make

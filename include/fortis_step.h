@@ -191,9 +191,8 @@ typedef struct {
     const int* cells;                  /* optional host list of `count` 0-based cell indices (i-1)+(j-1)*sx;
                                           NULL = the rectangle.  Copied to the device at config; the
                                           device-resident calls (fortis_stencil_*_dev, _step_fused) copy it the
-                                          first time they see a (table contents, list address) pair, so a list
-                                          must not be edited in place or another list put at its address while
-                                          the table is in use: give a changed list a new address. */
+                                          first time they see a table with these contents and this list (compared
+                                          by value on every call), and equal lists share one device copy. */
     int  elt[FORTIS_MAX_ARRAYS];       /* bytes per element of each host array: 4 (or 0) fp32, 8 fp64
                                           (the descriptor's "elt", driver/fortis_gather_emit.py:13) */
     int  cdouble[FORTIS_MAX_CONST];    /* constant n is a C double literal: its value is dconsts[n], not consts[n] */

@@ -91,6 +91,40 @@ def test_config3_climsim_full_size_row_sample(L, gpu):
     plan.close()
 
 
+def test_config3_climsim_full_size_with_boundary_kernels(L, gpu):
+    """Config 3 as the benchmark times it: the host's column-major A(24576, 556) in, column-major B(24576, 368)
+    out, the boundary transposes around the six GEMMs.  A seeded sample of 192 columns against
+    boundary_pre -> fp64-accumulated MLP -> boundary_post; non-trivial mean / range / scale vectors so that a
+    dropped or transposed vector shows."""
+    case = configs.climsim()
+    rng = np.random.default_rng(8)
+    case["mean"] = rng.standard_normal(556).astype(np.float32) * np.float32(0.1)
+    case["vmax"] = rng.uniform(1.5, 2.5, 556).astype(np.float32)
+    case["vmin"] = rng.uniform(0.0, 0.5, 556).astype(np.float32)
+    case["scale"] = rng.uniform(0.5, 2.0, 368).astype(np.float32)
+    plan = configs.climsim_plan(case, boundary=True)
+    assert plan.kernel_names() == ["boundary_pre"] + ["gemm_bias_act"] * 6 + ["boundary_post"]
+    B = plan.forward(case["A"].reshape(-1, order="F"), (368, 24576)).T          # column-major (24576, 368)
+    idx = np.sort(np.random.default_rng(5).choice(24576, 192, replace=False))
+    X = O.boundary_pre(np.asfortranarray(case["A"][idx]), case["mean"], case["vmax"], case["vmin"])
+    Yref = O.mlp_f64(case["Ws"], case["bs"], case["acts"], X, alphas=case["alphas"])
+    ref = O.boundary_post(Yref, case["scale"])
+    assert maxrel(B[idx], ref) < TOL
+    assert np.isfinite(B).all()
+    plan.close()
+    # the boundary kernels alone at this size are exact arithmetic: bit-equal to the oracle on the sampled columns
+    p = P.Plan()
+    t0, t1, t2 = p.tensor(24576 * 556), p.tensor(24576 * 556), p.tensor(24576 * 556)
+    p.boundary_pre(t0, t1, 24576, 556, case["mean"], case["vmax"], case["vmin"], np.float32)
+    sc = rng.uniform(0.5, 2.0, 556).astype(np.float32)
+    p.boundary_post(t1, t2, 24576, 556, sc, np.float32)
+    p.finalize(t0, t2)
+    Bt = p.forward(case["A"].reshape(-1, order="F"), (556, 24576)).T
+    assert np.array_equal(p.read(t1, (24576, 556))[idx].view(np.uint32), X.view(np.uint32))
+    assert np.array_equal(Bt[idx].view(np.uint32), O.boundary_post(X, sc).view(np.uint32))
+    p.close()
+
+
 def test_masked_relu_head_and_output_scale_fold_into_gemm(L, gpu):
     """124 -> 512 -> 128 with ReLU on the last 8 outputs (benchmarks/climsim/export_wide.py:24-28)."""
     rng = np.random.default_rng(1)

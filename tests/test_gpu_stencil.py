@@ -158,6 +158,53 @@ def test_fused_step_config2_network(L, gpu, golden, hidden):
     plan.close()
 
 
+@pytest.mark.parametrize("ncells", [4736, 2376])
+@pytest.mark.parametrize("lists", ["shared", "copies", "permuted"])
+def test_fused_step_masked_cell_list_config2(L, gpu, ncells, lists):
+    """Config 2 as BASELINE states it: 480 x 240 grid, 1-cell halo, seeded ~30 % land mask, the first 4736
+    (2376) ocean cells as the active list, 27 -> 64 -> 64 -> 3 between the gather and the scatter, all in the
+    one-launch kernel.  `shared`: both tables name one list object; `copies`: equal lists at two addresses (the
+    library still keeps one device copy and decodes a row once); `permuted`: the scatter visits the cells in
+    reverse order, so the kernel decodes gather and scatter cells separately."""
+    sx, sy, nz = 482, 242, 3
+    gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    A = configs.zb_arrays(sx, sy, nz, mask_land=0.3)
+    cells = configs.zb_cells_from_mask(A["mask"], sx, sy, ncells)
+    scells = cells if lists == "shared" else cells.copy() if lists == "copies" else np.ascontiguousarray(cells[::-1])
+    gt, st = S.build_table(gd, lp, kd, "gather", cells), S.build_table(sd, lp, kd, "scatter", scells)
+    net = configs.zb_mlp()
+    rows = ncells * nz
+    plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows)
+    garr = [A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"]]
+    n2, n3 = sx * sy, sx * sy * nz
+    host = [A["norm_h"], A["kappa_h"], np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+    out, Y = _fused(L, gt, st, plan, garr, host, rows)
+    X = O.stencil_gather(gd, garr, ncells, nz, cells=cells)
+    assert maxrel(Y, O.mlp_f64(net["Ws"], net["bs"], net["acts"], X)) < TOL
+    # the scatter of the kernel's own Y, and the unfused route (gather kernel -> X -> MLP -> Y -> scatter per layer)
+    ref = [a.copy() for a in host[:2]] + [np.zeros(n2, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+    txy = np.zeros((nz, n2), np.float32)
+    for kk in range(nz):
+        O.stencil_scatter(sd, ref, Y[kk * ncells:(kk + 1) * ncells], ncells, kk, cells=scells)
+        txy[kk] = ref[2]
+        ref[2][:] = 0
+    assert bits_equal(out[3], ref[3]) and bits_equal(out[4], ref[4]) and bits_equal(out[2].reshape(nz, n2), txy)
+    assert np.abs(ref[3]).max() > 0
+    gb, sb = [DevBuf(L, a) for a in garr], [DevBuf(L, a) for a in host]
+    dX, dY = plan.ptr(plan.in_tensor), plan.ptr(plan.out_tensor)
+    L.fortis_stencil_gather_dev(C.byref(gt), ptrs(gb), C.c_void_p(dX))
+    plan.run()
+    for kk in range(nz):
+        L.fortis_stencil_scatter_dev(C.byref(st), ptrs(sb), C.c_void_p(dY + kk * ncells * 3 * 4), kk)
+    L.fortis_sync()
+    assert bits_equal(plan.read(plan.out_tensor, (rows, 3)), Y)
+    for q in (3, 4):
+        assert bits_equal(sb[q].get((n3,)), out[q])
+    for b in gb + sb:
+        b.free()
+    plan.close()
+
+
 def test_bench_grid_fused_equals_unfused_and_layer_vs_oracle(L, gpu):
     """The benchmark grid, 1028 x 1028 x 15 (15.7 M columns), through properties that do not need the oracle at
     that size: the one-launch fused step and the reference's structure (gather kernel -> X -> MLP -> Y -> one

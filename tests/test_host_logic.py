@@ -83,6 +83,53 @@ def test_pool_unknown_pointer_is_really_freed(pool):
     assert dev.frees == 1
 
 
+# ---- allocations the library makes for itself fail cleanly ---------------------------------------------
+def test_finalize_fails_when_the_weights_find_no_device_memory(pool, capfd):
+    """Weights, vectors and packed blobs go through the same switchable allocator as the pool: when one of them
+    finds no memory, finalize returns -1 (the reference prints and returns NULL, runtime/fortis_rt.c:35), the
+    plan never launches, and destroying it hands everything back."""
+    L, dev = pool                                              # 1000 bytes of "device" memory
+    p = L.fortis_plan_create()
+    t0, t1 = L.fortis_plan_tensor(p, 2 * 4 * 4), L.fortis_plan_tensor(p, 2 * 300 * 4)
+    W = np.zeros((300, 4), np.float32)                         # 4800 bytes: does not fit
+    assert L.fortis_plan_linear(p, t0, t1, W.ctypes.data_as(C.c_void_p), None, 2, 4, 300, 0, 0.0) == 0
+    assert L.fortis_plan_finalize(p, t0, t1) == -1
+    err = capfd.readouterr().err
+    assert "device allocation of 4800 bytes failed (plan weights)" in err and "out of device memory" in err
+    assert L.fortis_plan_num_kernels(p) == -1                  # not finalized
+    L.fortis_plan_run(p)
+    assert "not finalized" in capfd.readouterr().err
+    L.fortis_plan_destroy(p)
+    assert not dev.live and stats(L)[1] == 0
+
+
+def test_stencil_config_fails_when_the_cell_list_finds_no_device_memory(pool, capfd, golden):
+    L, dev = pool
+    g, lp, kd = [json.load(open(os.path.join(golden, f"zb_{n}.json"))) for n in ("gather", "loop", "kdist")]
+    cells = (np.arange(300, dtype=np.int32) % 60) + 1 + 68 * (1 + np.arange(300, dtype=np.int32) // 60)   # 1200 bytes
+    t = S.build_table(g, lp, kd, "gather", cells=cells)
+    assert L.fortis_stencil_check(C.byref(t)) == 0
+    assert L.fortis_gather_config(C.byref(t)) == -1
+    assert "stencil cell list" in capfd.readouterr().err
+    L.fortis_gather_v(None, None)                              # nothing configured: prints, touches nothing
+    assert "no gather table configured" in capfd.readouterr().err
+    assert not dev.live
+
+
+def test_stencil_table_must_hold_the_planes_it_names(L, golden, capfd):
+    """nk planes from iteration klo on must fit the array: the host-array entries copy exactly those."""
+    g, lp, kd = [json.load(open(os.path.join(golden, f"zb_{n}.json"))) for n in ("gather", "loop", "kdist")]
+    t = S.build_table(g, lp, kd, "gather")
+    assert L.fortis_stencil_check(C.byref(t)) == 0
+    t.nk = 16                                                  # the arrays hold 15 planes
+    assert L.fortis_stencil_check(C.byref(t)) == -1
+    t.nk, t.klo = 15, 2
+    assert L.fortis_stencil_check(C.byref(t)) == -1
+    t.nk, t.klo = 14, 2
+    assert L.fortis_stencil_check(C.byref(t)) == 0
+    assert "fewer than the" in capfd.readouterr().err
+
+
 # ---- plan argument checks (no device work before finalize) ------------------------------------------
 def test_plan_rejects_bad_arguments(L):
     p = L.fortis_plan_create()

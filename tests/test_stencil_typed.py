@@ -57,6 +57,37 @@ def test_c_eval_closed_forms_and_promotion():
     assert O.c_eval("tv / 2.0f * 4.0f", {"tv": tv})[4] == np.float32(14.0)
 
 
+def test_c_eval_transcendentals_pinned_by_special_values_and_identities():
+    """expf / logf / tanhf of the evaluator against what the mathematics fixes, not against a retyped formula:
+    exact special values, published constants to two fp32 ulps, inverse and symmetry relations.  Swapping any two
+    of the three names, or mapping one to another function, fails at least one line."""
+    z, one = np.zeros(4, np.float32), np.ones(4, np.float32)
+    ev = lambda text, tv: O.c_eval(text, {"tv": np.asarray(tv, np.float32)})
+    for fn in ("expf(tv)", "logf(tv)", "tanhf(tv)"):
+        assert ev(fn, one).dtype == np.float32                  # float in, float out (the f-suffixed C functions)
+    assert np.array_equal(ev("expf(tv)", z), one)               # e^0 = 1
+    assert np.array_equal(ev("logf(tv)", one), z)               # ln 1 = 0
+    assert np.array_equal(ev("tanhf(tv)", z), z)                # tanh 0 = 0
+    ulp = lambda v: np.spacing(np.float32(abs(v)))
+    for text, x, want in (("expf(tv)", 1.0, 2.718281828459045), ("expf(tv)", -1.0, 0.36787944117144233),
+                          ("logf(tv)", 2.0, 0.6931471805599453), ("logf(tv)", 10.0, 2.302585092994046),
+                          ("tanhf(tv)", 0.5, 0.46211715726000974), ("tanhf(tv)", 1.0, 0.7615941559557649)):
+        got = float(ev(text, [x])[0])
+        assert abs(got - want) <= 2 * ulp(want), (text, x, got)
+    x = np.linspace(-8, 8, 161).astype(np.float32)
+    back = ev("logf(expf(tv))", x)                              # ln(e^x) = x
+    assert np.abs(back - x).max() <= 8 * 2.0 ** -23 * 8
+    t = ev("tanhf(tv)", x)
+    assert np.array_equal(ev("tanhf(-tv)", x), -t)              # odd
+    assert (np.abs(t) <= 1).all() and (np.diff(t) >= 0).all() and t[-1] > 0.999999
+    e = ev("expf(tv)", x)
+    assert (e > 0).all() and (np.diff(e) > 0).all()
+    # tanh x = (e^2x - 1) / (e^2x + 1), evaluated in binary64 from the pinned exponential's argument
+    ref = np.expm1(2 * x.astype(np.float64)) / (np.exp(2 * x.astype(np.float64)) + 1)
+    assert np.abs(t - ref).max() <= 2.0 ** -22
+    assert np.isnan(ev("logf(tv)", [-1.0])[0]) and ev("logf(tv)", [0.0])[0] == -np.inf
+
+
 def test_table_compiler_types_follow_c():
     F64 = S.INS_F64
     # all fp32: no flags, no conversions; the reference's own ZB expressions
