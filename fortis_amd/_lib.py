@@ -47,6 +47,7 @@ PROTOTYPES = {
     "fortis_gemm": (None, [vp, vp, l, l, l, l, l] * 3 + [l, l, l]),
     "fortis_conv2d": (None, [vp, vp] + [l] * 9 + [vp, vp] + [l] * 9 + [vp, vp] + [l] * 9 + [l] * 13),
     "fortis_conv3d": (None, ([vp, vp] + [l] * 11) * 3 + [l] * 18),
+    "fortis_conv3d_noalloc": (i, ([vp, vp] + [l] * 11) * 3 + [l] * 18),
     "fortis_conv3d_direct": (None, ([vp, vp] + [l] * 11) * 3 + [l] * 18),
     "fortis_conv3d_fft": (None, ([vp, vp] + [l] * 11) * 3 + [l] * 18),
     "fortis_h2d": (None, [vp, vp, l]), "fortis_d2h": (None, [vp, vp, l]), "fortis_d2d": (None, [vp, vp, l]),

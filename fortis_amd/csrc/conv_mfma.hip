@@ -361,16 +361,31 @@ static int conv_cus()
     return n;
 }
 
+// A caller-provided workspace replaces the two buffers this file otherwise grows with hipMalloc (the packed
+// weights of fortis_conv_mfma_pack_dev first, the partial sums of channel-split launches behind them) until it is
+// taken away again with (null, 0).  A request that does not fit returns null, which the launchers turn into -1
+// before anything is launched, and is remembered for fortis_conv_workspace_overflowed().
+static char* g_ws = nullptr;
+static size_t g_ws_bytes = 0, g_ws_pack = 0, g_ws_wanted = 0;
+void fortis_conv_workspace(void* base, size_t bytes) { g_ws = (char*)base; g_ws_bytes = bytes; g_ws_pack = 0; g_ws_wanted = 0; }
+size_t fortis_conv_workspace_overflowed() { return g_ws_wanted; }
+static float* ws_take(size_t offset, size_t need)
+{
+    if (offset + need > g_ws_bytes) { g_ws_wanted = offset + need; return nullptr; }
+    return (float*)(g_ws + offset);
+}
+
 // Partial sums of channel-split launches: one buffer for every shape (launches on the library's stream run
 // one after the other).  It grows on the first, eager run of a plan; replays and captured runs find it in
 // place.  An outgrown buffer stays allocated: a graph captured earlier may still name it.
 float* fortis_conv_split_scratch(size_t need)
 {
+    if (g_ws) return ws_take(g_ws_pack, need);
     static float* scratch = nullptr;
     static size_t cap = 0;
     if (need > cap) {
         float* p = nullptr;
-        if (hipMalloc((void**)&p, need) != hipSuccess) { fprintf(stderr, "fortis: no memory for %zu bytes of conv partial sums\n", need); return nullptr; }
+        if (hipMalloc((void**)&p, need) != hipSuccess) { (void)hipGetLastError(); fprintf(stderr, "fortis: no memory for %zu bytes of conv partial sums\n", need); return nullptr; }
         scratch = p;
         cap = need;
     }
@@ -449,6 +464,14 @@ const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, h
     static size_t cap = 0;
     const long FT = conv_ft(F), CC = cm_cc(T);
     const long nch = cdiv(C, CC), n = cdiv(F, FT) * nch * (CC / 2) * T * 2 * FT;
+    if (g_ws) {
+        float* w = ws_take(0, (size_t)n * sizeof(float));
+        if (!w) return nullptr;
+        g_ws_pack = ((size_t)n * sizeof(float) + 255) & ~(size_t)255;
+        hipLaunchKernelGGL(conv_pack_kernel, dim3((unsigned)cdiv(n, 256)), dim3(256), 0, st, dW, w, F, C, T, (int)FT, (int)CC, nch, n);
+        HIP_OK(hipGetLastError());
+        return w;
+    }
     if ((size_t)n * sizeof(float) > cap) {
         float* p = nullptr;
         if (hipMalloc((void**)&p, (size_t)n * sizeof(float)) != hipSuccess) { (void)hipGetLastError(); return nullptr; }

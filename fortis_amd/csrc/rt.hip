@@ -6,6 +6,30 @@
 
 // ---- stream (runtime/fortis_rt.c:5-12) ---------------------------------------------------
 static hipStream_t g_stream = nullptr;
+
+// ---- fixed scratch of the entry that allocates nothing (fortis_conv3d_noalloc) -----------------------------
+// The array's name is a host-side handle, not a device address: host code uses the address that
+// hipGetSymbolAddress returns for the current device, looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[FORTIS_NOALLOC_SCRATCH_BYTES];
+#define FORTIS_MAX_DEVICES 64
+static void* g_scratch_ptr[FORTIS_MAX_DEVICES];
+static void* noalloc_scratch()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= FORTIS_MAX_DEVICES) { (void)hipGetLastError(); return nullptr; }
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            fprintf(stderr, "fortis: the fixed scratch array has no address on device %d: %s\n", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+
 extern "C" {
 int fortis_capturing = 0;
 
@@ -18,6 +42,7 @@ void* mgpuStreamCreate(void)
             abort();
         }
         HIP_OK(hipStreamCreate(&g_stream));   // default priority, blocking flag like cudaStreamCreate
+        (void)noalloc_scratch();              // set-up: the fixed scratch's address on this device
     }
     return (void*)g_stream;
 }
@@ -158,12 +183,12 @@ void fortis_conv2d(float* xa, float* x, long xo, long x0, long x1, long x2, long
 // fortis_conv3d takes what the reference's library path takes (runtime/fortis_rt.c:128-156): any batch, any
 // stride.  The direct and large-kernel entries keep the reference's own limits (N = 1, stride 1;
 // runtime/fortis_fft.cu:70, 135).
-static void conv3d_any(const char* who, bool general, float* x, long xo, float* w, long wo, float* y, long yo, long N, long C,
-                       long Din, long Hin, long Win, long F, long KD, long KH, long KW, long Dout, long Hout,
-                       long Wout, long sd, long sh, long sw, long pd, long ph, long pw)
+static int conv3d_any(const char* who, bool general, float* x, long xo, float* w, long wo, float* y, long yo, long N, long C,
+                      long Din, long Hin, long Win, long F, long KD, long KH, long KW, long Dout, long Hout,
+                      long Wout, long sd, long sh, long sw, long pd, long ph, long pw)
 {
     const bool unit = sd == 1 && sh == 1 && sw == 1;
-    if (!general && (N != 1 || !unit)) { fprintf(stderr, "%s: unsupported shape\n", who); return; }
+    if (!general && (N != 1 || !unit)) { fprintf(stderr, "%s: unsupported shape\n", who); return -1; }
     const long xn = C * Din * Hin * Win, yn = F * Dout * Hout * Wout;
     for (long n = 0; n < N; n++) {
         float* xb = x + xo + n * xn;
@@ -172,26 +197,50 @@ static void conv3d_any(const char* who, bool general, float* x, long xo, float* 
             conv_entry_mfma(xb, w + wo, yb, C, Din, Hin, Win, F, 3, 3) == 0)
             continue;
         ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
-        if (fortis_launch_conv3d(xb, w + wo, yb, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, pd, ph, pw, e,
-                                 fortis_stream_get(), sd, sh, sw) != 0) {
-            fprintf(stderr, "%s: unsupported shape\n", who);
-            return;
+        int rc = -1;
+        // a caller's fixed workspace that was too small is an error of its own: the shape is not handed on to
+        // a slower kernel behind the caller's back
+        if (!fortis_conv_workspace_overflowed())
+            rc = fortis_launch_conv3d(xb, w + wo, yb, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, pd, ph, pw, e,
+                                      fortis_stream_get(), sd, sh, sw);
+        if (fortis_conv_workspace_overflowed()) {
+            fprintf(stderr, "%s: this shape needs %zu bytes of scratch, more than the fixed %ld; nothing computed\n", who,
+                    fortis_conv_workspace_overflowed(), (long)FORTIS_NOALLOC_SCRATCH_BYTES);
+            return -1;
         }
+        if (rc != 0) { fprintf(stderr, "%s: unsupported shape\n", who); return -1; }
     }
+    return 0;
 }
-#define CONV3D_FWD(who)                                                                                             \
+#define CONV3D_UNUSED                                                                                               \
     (void)xa; (void)x0; (void)x1; (void)x2; (void)x3; (void)x4; (void)xt0; (void)xt1; (void)xt2; (void)xt3; (void)xt4; \
     (void)wa; (void)w0; (void)w1; (void)w2; (void)w3; (void)w4; (void)wt0; (void)wt1; (void)wt2; (void)wt3; (void)wt4; \
-    (void)ya; (void)y0; (void)y1; (void)y2; (void)y3; (void)y4; (void)yt0; (void)yt1; (void)yt2; (void)yt3; (void)yt4; \
+    (void)ya; (void)y0; (void)y1; (void)y2; (void)y3; (void)y4; (void)yt0; (void)yt1; (void)yt2; (void)yt3; (void)yt4
+#define CONV3D_FWD(who, general)                                                                                    \
     conv3d_any(who, general, x, xo, w, wo, y, yo, N, C, Din, Hin, Win, F, KD, KH, KW, Dout, Hout, Wout, sd, sh, sw, pd, ph, pw)
 
-void fortis_conv3d(FORTIS_CONV3D_ARGS) { const bool general = true; CONV3D_FWD("fortis_conv3d"); }
-void fortis_conv3d_direct(FORTIS_CONV3D_ARGS) { const bool general = false; CONV3D_FWD("fortis_conv3d_direct"); }
+void fortis_conv3d(FORTIS_CONV3D_ARGS) { CONV3D_UNUSED; (void)CONV3D_FWD("fortis_conv3d", true); }
+// The same call for callers that cannot allocate device memory: the packed weights and the partial sums of
+// channel-split launches live in the fixed scratch array instead of buffers grown with hipMalloc.  Every call
+// on a GPU uses that GPU's one array (both regions are written in full before they are read, so nothing needs
+// clearing): calls that overlap in time on one GPU race.
+int fortis_conv3d_noalloc(FORTIS_CONV3D_ARGS)
+{
+    CONV3D_UNUSED;
+    (void)fortis_stream_get();
+    void* ws = noalloc_scratch();
+    if (!ws) return -1;
+    fortis_conv_workspace(ws, FORTIS_NOALLOC_SCRATCH_BYTES);
+    const int rc = CONV3D_FWD("fortis_conv3d_noalloc", true);
+    fortis_conv_workspace(nullptr, 0);
+    return rc;
+}
+void fortis_conv3d_direct(FORTIS_CONV3D_ARGS) { CONV3D_UNUSED; (void)CONV3D_FWD("fortis_conv3d_direct", false); }
 void fortis_conv3d_fft(FORTIS_CONV3D_ARGS)
 {
+    CONV3D_UNUSED;
     if (pd || ph || pw) { fprintf(stderr, "fortis_conv3d_fft: unsupported shape\n"); return; }
-    const bool general = false;
-    CONV3D_FWD("fortis_conv3d_fft");
+    (void)CONV3D_FWD("fortis_conv3d_fft", false);
 }
 
 // ---- host utilities ----------------------------------------------------------------------------

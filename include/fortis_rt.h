@@ -72,6 +72,16 @@ void fortis_conv2d(float* xa, float* x, long xo, long x0, long x1, long x2, long
  * kernel with FORTIS_DIRECT; here every shape runs the library-free direct path.
  *                                                                   runtime/fortis_rt.c:128-156 */
 void fortis_conv3d(FORTIS_CONV3D_ARGS);
+/* No counterpart in the reference.  fortis_conv3d for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments and result, but the
+ * packed weights and the partial sums of channel-split launches live in a fixed device array of
+ * FORTIS_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs on, and the call makes no hipMalloc,
+ * hipFree or other allocating call.  Returns 0, or -1 with a message on stderr when the shape is unsupported or
+ * needs more scratch than that (nothing is computed then).  All calls on one GPU share the array: calls that
+ * overlap in time on one GPU race.  The library must have been used once before (any entry; mgpuStreamCreate
+ * does) when the caller is capturing. */
+#define FORTIS_NOALLOC_SCRATCH_BYTES (32L << 20)
+int  fortis_conv3d_noalloc(FORTIS_CONV3D_ARGS);
 /* Direct tiled conv3d; N = 1 and stride 1 only, otherwise prints "unsupported shape" and
  * returns without computing.                                        runtime/fortis_fft.cu:131-146 */
 void fortis_conv3d_direct(FORTIS_CONV3D_ARGS);
