@@ -74,7 +74,7 @@ PROTOTYPES = {
     "fortis_plan_tensor_ptr": (vp, [vp, i]), "fortis_plan_num_kernels": (i, [vp]),
     # step + entries
     "fortis_step_bind": (i, [vp, C.POINTER(HostFacts)]), "fortis_step_reset": (None, []),
-    "fortis_step_graph_active": (i, []),
+    "fortis_step_graph_active": (i, []), "fortis_step_on_first_use": (None, [vp]),
     "mlp_upload": (None, [vp]), "mlp_forward_dev": (None, []), "mlp_download": (None, [vp]),
     "mlp_forward": (None, [vp, vp]), "mlp_forward_batched": (None, [vp, vp]),
     "fortis_pack": (None, [vp, i]), "fortis_unpack": (None, [vp, i]),

@@ -123,10 +123,11 @@ def climsim(rows=24576, n_in=556, hidden=768, nhidden=5, n_out=368, alpha=0.15):
                 rows=rows, widths=widths, flops=flops, bytes=nbytes)
 
 
-def climsim_plan(case, boundary=True):
-    """gather (boundary pre) -> GEMM chain -> scatter (boundary post), or the bare chain."""
+def climsim_plan(case, boundary=True, plan_cls=None):
+    """gather (boundary pre) -> GEMM chain -> scatter (boundary post), or the bare chain.  plan_cls: a class with
+    Plan's interface to fill instead (the op-list recorder of fortis_amd.shim_hip)."""
     rows, widths = case["rows"], case["widths"]
-    p = P.Plan()
+    p = (plan_cls or P.Plan)()
     if boundary:
         t_in = p.tensor(rows * widths[0])
         cur = p.tensor(rows * widths[0])
@@ -186,9 +187,9 @@ def unet(H=256, cin=4, chans=(32, 64, 128, 256), cout=4):
                 flops=2 * macs, voxels=H * H)
 
 
-def unet_plan(case):
+def unet_plan(case, plan_cls=None):
     H, chans = case["H"], case["chans"]
-    p = P.Plan()
+    p = (plan_cls or P.Plan)()
     t_in = p.tensor(case["cin"] * H * H)
     # one buffer per decoder level holds [skip | up]; the encoder's last conv of the level writes the
     # first window, the transposed conv writes the second: the concatenation costs no copy
@@ -245,11 +246,11 @@ def tsrgan(D=33, cin=3, ch=64, nblocks=8, cout=3, alpha=0.2):
                 alpha=alpha, flops=2 * macs, voxels=v2)
 
 
-def tsrgan_plan(case):
+def tsrgan_plan(case, plan_cls=None):
     D, ch, cin, cout, a = case["D"], case["ch"], case["cin"], case["cout"], case["alpha"]
     v1, D2 = D ** 3, 2 * D
     v2 = D2 ** 3
-    p = P.Plan()
+    p = (plan_cls or P.Plan)()
     t_in = p.tensor(v1 * cin)
     t = p.tensor(v1 * cin)
     p.permute(t_in, t, cin, v1, True)

@@ -707,15 +707,29 @@ void fortis_step_reset(void)
 }
 int fortis_step_graph_active(void) { return g_step.gexec != nullptr; }
 
+// A step file registers its binder instead of binding at load time: the binder runs at the first use of an
+// entry point, like setup() in the reference's shim (driver/fortis_shim.py:64-73, `if (!din) setup();`), when
+// the host's global vectors that the plan copies (boundary and lifted normalisation vectors) hold their values.
+static void (*g_bind_on_use)(void) = nullptr;
+void fortis_step_on_first_use(void (*bind)(void)) { g_bind_on_use = bind; }
+static void bind_if_pending()
+{
+    if (g_step.plan || !g_bind_on_use) return;
+    void (*f)(void) = g_bind_on_use;
+    g_bind_on_use = nullptr;
+    f();
+}
+
 static bool bound(const char* who)
 {
+    bind_if_pending();
     if (!g_step.plan) { fprintf(stderr, "%s: no step bound (fortis_step_bind was not called)\n", who); return false; }
     return true;
 }
 
 static long g_forward_gen = 0;   // bumped by every forward pass of the bound step
-void* fortis_model_input(void) { return g_step.din; }
-void* fortis_model_output(void) { return g_step.dout; }
+void* fortis_model_input(void) { bind_if_pending(); return g_step.din; }
+void* fortis_model_output(void) { bind_if_pending(); return g_step.dout; }
 long fortis_step_generation(void) { return g_forward_gen; }   // internal: lets the scatter entry notice a new forward pass
 
 void mlp_forward_dev(void)

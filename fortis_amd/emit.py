@@ -1,84 +1,94 @@
-"""Emitter of the per-build step file: what driver/fortis_shim.py writes as shim.c (and
-fortis_outline.py as weights.o) for the reference's CUDA build, written instead as one C file that
-builds the plan through the library's C ABI in a constructor and binds it as the process's step.  A host
-object that calls mlp_forward / mlp_upload / mlp_forward_dev / ... by bind(c) name links against this
-file's object and libfortis_rt.so and runs unchanged.
-
-Weights travel as a raw fp32 blob next to the C file, pulled into the object with .incbin (the role of
-the `extern float w0[], w1[], ...` blobs of weights.o)."""
+"""Per-build generated files of a FORTIS_BACKEND=hip build, written from Python arguments: the module-side
+inputs of fortis_amd/shim_hip.py (m4.mlir's attribute line, outline.json, ops.json, a weights.o stand-in) for
+models given as numpy arrays, and the C file that replaces the generated gather.cu
+(driver/fortis_gather_emit.py).  The step file itself always comes out of shim_hip.generate, the one
+generator: nothing here writes plan calls."""
+import json
 import os
 
 import numpy as np
 
-ACT = {None: 0, "none": 0, "relu": 1, "leaky": 2}
-VERDICT = {"whole": "FORTIS_VERDICT_WHOLE", "batched": "FORTIS_VERDICT_BATCHED", "boundary": "FORTIS_VERDICT_BOUNDARY"}
+from . import shim_hip
 
 
-def _preamble(bin_path):
-    """Head of the generated file up to the creation of the plan; `w` points at the weight blob."""
-    return [
-        "/* generated by fortis_amd/emit.py: plan of the step + host facts, bound at load time */",
-        "#include <stdio.h>", "#include <stdlib.h>", '#include "fortis_step.h"',
-        '__asm__(".section .rodata\\n .balign 16\\n .globl fortis_step_blob\\n fortis_step_blob:\\n .incbin \\"%s\\"\\n .previous\\n");' % bin_path,
-        "extern const float fortis_step_blob[];",
-        '#define OK(call) do { if ((call) < 0) { fprintf(stderr, "fortis step: %s failed\\n", #call); exit(1); } } while (0)',
-        "__attribute__((constructor)) static void fortis_bind_step(void)", "{",
-        "    const float* w = fortis_step_blob;",
-        "    fortis_plan* p = fortis_plan_create();",
-    ]
+def host_attr(verdict="whole", shape=(1,), batch=1, repeat=0, graph=False, loop=None, expand=None, lift=None, boundary=None):
+    """The attribute dictionary driver/fortis_hostattr.py:11-28 attaches to the model entry, as MLIR text.
+    loop: dict(lo, step, count, minc, in, out, post_download); expand: dict(in, out, count, nin, nout);
+    lift: dict(globals=[...], in=...); boundary: dict(in, in_elt, out, out_elt, pre=[...], post=[...])."""
+    q = lambda v: '"%s"' % v
+    i64 = lambda v: "%d : i64" % int(v)
+    parts = ["version = 1 : i64", "shape = [%s]" % ", ".join(str(x) for x in shape), "batch = " + i64(batch),
+             "repeat = " + i64(repeat), "verdict = " + q(verdict),
+             'provenance = {shape = "proven", repeat = "proven", dependence = "proven", lift = "proven", layout = "proven", '
+             'scope = "proven", aliasing = "checked", purity = "checked", fp_order = "assumed"}']
+    if loop:
+        parts.append("loop = {lo = %s, step = %s, count = %s, minc = %s, in = %s, out = %s, post_download = %s}" % (
+            i64(loop["lo"]), i64(loop["step"]), i64(loop["count"]), i64(loop["minc"]), q(loop.get("in", "x")), q(loop.get("out", "y")),
+            "true" if loop.get("post_download") else "false"))
+    if expand:
+        parts.append("expand = {in = %s, out = %s, count = %s, nin = %s, nout = %s}" % (
+            q(expand.get("in", "x")), q(expand.get("out", "y")), i64(expand["count"]), i64(expand["nin"]), i64(expand["nout"])))
+    if lift:
+        parts.append("lift = {globals = [%s], in = %s}" % (", ".join(q(g) for g in lift["globals"]), q(lift.get("in", "x"))))
+    if boundary:
+        parts.append("boundary = {in = %s, in_elt = %s, out = %s, out_elt = %s, pre = [%s], post = [%s]}" % (
+            q(boundary["in"]), q(boundary["in_elt"]), q(boundary["out"]), q(boundary["out_elt"]),
+            ", ".join(q(g) for g in boundary["pre"]), ", ".join(q(g) for g in boundary["post"])))
+    attrs = "fortis.host = {" + ", ".join(parts) + "}"
+    if graph:
+        attrs += ", fortis.graph = true"
+    return attrs
 
 
-def emit_mlp_step(prefix, Ws, bs, acts, rows, alphas=None, in_norms=None, out_norms=None, verdict="whole",
-                  graph=False, expanded=False, count=0, lo=1, step=1, minc=1, in_esz=4, out_esz=4,
-                  gather=False, scatter=False):
-    """Writes <prefix>.c and <prefix>.bin for a Linear(+activation) stack over `rows` rows with optional
-    input division / output multiplication vectors (mom6_zb/export_zb.py:10-16).  Returns the two paths."""
-    n = len(Ws)
-    widths = [int(Ws[0].shape[1])] + [int(w.shape[0]) for w in Ws]
-    alphas = alphas or [0.0] * n
-    blob, offs = [], {}
+def module_stub(attr_text, outline):
+    """The one line of m4.mlir the shim generators read: the signature of @mlp_kernel with its attributes."""
+    args = ", ".join("%%arg%d: %s" % (i, t) for i, t in enumerate(outline["inputs"] + outline["weights"] + [outline["output"]]))
+    return "module {\n  func.func @mlp_kernel(%s) attributes {%s} {\n    return\n  }\n}\n" % (args, attr_text)
 
-    def add(name, a):
-        a = np.ascontiguousarray(a, dtype=np.float32).reshape(-1)
-        pad = (-sum(x.size for x in blob)) % 4            # keep every vector 16-byte aligned
-        if pad:
-            blob.append(np.zeros(pad, np.float32))
-        offs[name] = sum(x.size for x in blob)
-        blob.append(a)
 
-    for l in range(n):
-        add(f"w{l}", Ws[l])
-        add(f"b{l}", bs[l] if bs[l] is not None else np.zeros(widths[l + 1], np.float32))
-    if in_norms is not None:
-        add("in_norms", in_norms)
-    if out_norms is not None:
-        add("out_norms", out_norms)
-    bin_path, c_path = os.path.abspath(prefix + ".bin"), os.path.abspath(prefix + ".c")
-    np.concatenate(blob).tofile(bin_path)
+def step_files(outdir, oplist, attr_text, in_type, out_type, extra_inputs=(), env=None):
+    """Writes, under outdir, what a FORTIS_BACKEND=hip build holds for one model: m4.mlir (attribute line only),
+    outline.json, ops.json, then runs the generator (-> step_tables.c, link_hip.txt) and writes the weights
+    stand-in (weights.c + w<i>.bin).  Returns [step_tables.c, weights.c]."""
+    os.makedirs(outdir, exist_ok=True)
+    outline = oplist.outline(in_type, out_type, extra_inputs)
+    with open(os.path.join(outdir, "m4.mlir"), "w") as f:
+        f.write(module_stub(attr_text, outline))
+    json.dump(outline, open(os.path.join(outdir, "outline.json"), "w"))
+    json.dump(oplist.as_json(), open(os.path.join(outdir, "ops.json"), "w"))
+    c = shim_hip.generate(os.path.join(outdir, "m4.mlir"), os.path.join(outdir, "outline.json"), outdir, env=env)
+    return [c, shim_hip.write_weights_c(outdir, oplist.weights)]
 
-    L = _preamble(bin_path)
-    L.append(f"    const long rows = {rows};")
-    L.append("    int cur, nxt, in_t;")
-    L.append(f"    OK(in_t = cur = fortis_plan_tensor(p, rows * {widths[0]} * 4));")
-    if in_norms is not None:
-        L.append(f"    OK(nxt = fortis_plan_tensor(p, rows * {widths[0]} * 4));")
-        L.append(f"    OK(fortis_plan_scale(p, cur, nxt, w + {offs['in_norms']}, rows, {widths[0]}, 1)); cur = nxt;")
-    for l in range(n):
-        L.append(f"    OK(nxt = fortis_plan_tensor(p, rows * {widths[l + 1]} * 4));")
-        L.append(f"    OK(fortis_plan_linear(p, cur, nxt, w + {offs[f'w{l}']}, w + {offs[f'b{l}']}, rows, {widths[l]}, {widths[l + 1]}, "
-                 f"{ACT[acts[l]]}, {float(alphas[l])!r}f)); cur = nxt;")
-    if out_norms is not None:
-        L.append(f"    OK(nxt = fortis_plan_tensor(p, rows * {widths[-1]} * 4));")
-        L.append(f"    OK(fortis_plan_scale(p, cur, nxt, w + {offs['out_norms']}, rows, {widths[-1]}, 0)); cur = nxt;")
-    L.append("    OK(fortis_plan_finalize(p, in_t, cur));")
-    L.append("    fortis_host_t host = { .n_in = rows * %d, .n_out = rows * %d, .in_esz = %d, .out_esz = %d, .verdict = %s,"
-             % (widths[0], widths[-1], in_esz, out_esz, VERDICT[verdict]))
-    L.append("                           .expanded = %d, .count = %d, .lo = %d, .step = %d, .minc = %d, .graph = %d, .gather = %d, .scatter = %d };"
-             % (1 if expanded else 0, count, lo, step, minc, 1 if graph else 0, 1 if gather else 0, 1 if scatter else 0))
-    L.append("    OK(fortis_step_bind(p, &host));\n}")
-    with open(c_path, "w") as f:
-        f.write("\n".join(L) + "\n")
-    return c_path, bin_path
+
+def emit_mlp_step(outdir, Ws, bs, acts, rows, alphas=None, in_norms=None, out_norms=None, verdict="whole",
+                  graph=False, expanded=False, count=0, lo=1, step=1, minc=1, gather=False, scatter=False):
+    """Step files for a Linear(+activation) stack over `rows` rows with optional input division / output
+    multiplication vectors (mom6_zb/export_zb.py:10-16)."""
+    from . import plan as P
+    ol = P.mlp_plan(Ws, bs, acts, rows, alphas=alphas, in_norms=in_norms, out_norms=out_norms, plan_cls=shim_hip.OpList)
+    nin, nout = int(Ws[0].shape[1]), int(Ws[-1].shape[0])
+    kw = {}
+    if verdict == "batched":
+        kw["loop"] = dict(lo=lo, step=step, count=count, minc=minc)
+        if expanded:
+            kw["expand"] = dict(count=count, nin=rows * nin // count, nout=rows * nout // count)
+    env = dict(FORTIS_GATHER="1" if gather else "", FORTIS_SCATTER="1" if scatter else "")
+    attr = host_attr(verdict, shape=(nin,), batch=count or rows, graph=graph, **kw)
+    return step_files(outdir, ol, attr, "tensor<%dx%dxf32>" % (rows, nin), "tensor<%dx%dxf32>" % (rows, nout), env=env)
+
+
+def emit_conv3d_step(outdir, W, b, shape, pad=1, act=None, alpha=0.0, graph=False):
+    """Step files for one conv3d (+ activation) on an NCDHW tensor of `shape` = (C, D, H, W), stride 1
+    (frontend/export_conv.py:4)."""
+    C_, D, H, Wd = (int(v) for v in shape)
+    F, K = int(W.shape[0]), int(W.shape[2])
+    Do, Ho, Wo = D + 2 * pad - K + 1, H + 2 * pad - K + 1, Wd + 2 * pad - K + 1
+    ol = shim_hip.OpList()
+    t0, t1 = ol.tensor(C_ * D * H * Wd), ol.tensor(F * Do * Ho * Wo)
+    ol.conv3d(t0, t1, W, b, C_, D, H, Wd, pad, act, alpha)
+    ol.finalize(t0, t1)
+    attr = host_attr("whole", shape=(1, C_, D, H, Wd), graph=graph)
+    return step_files(outdir, ol, attr, "tensor<1x%dx%dx%dx%dxf32>" % (C_, D, H, Wd), "tensor<1x%dx%dx%dx%dxf32>" % (F, Do, Ho, Wo))
 
 
 def _table_c(name, t):
@@ -147,30 +157,3 @@ def emit_stencil_tables(path, gather_desc, scatter_desc, loop, kdist=None):
     with open(path, "w") as f:
         f.write("\n".join(L) + "\n")
     return path
-
-
-def emit_conv3d_step(prefix, W, b, shape, pad=1, act=None, alpha=0.0, graph=False):
-    """Writes <prefix>.c / <prefix>.bin for one conv3d (+ activation) on an NCDHW tensor of `shape` =
-    (C, D, H, W), stride 1 (frontend/export_conv.py:4).  Returns the two paths."""
-    C_, D, H, Wd = (int(v) for v in shape)
-    F, K = int(W.shape[0]), int(W.shape[2])
-    Do, Ho, Wo = D + 2 * pad - K + 1, H + 2 * pad - K + 1, Wd + 2 * pad - K + 1
-    wflat = np.ascontiguousarray(W, dtype=np.float32).reshape(-1)
-    padn = (-wflat.size) % 4
-    boff = wflat.size + padn
-    bin_path, c_path = os.path.abspath(prefix + ".bin"), os.path.abspath(prefix + ".c")
-    np.concatenate([wflat, np.zeros(padn, np.float32), np.ascontiguousarray(b, dtype=np.float32).reshape(-1)]).tofile(bin_path)
-    n_in, n_out = C_ * D * H * Wd, F * Do * Ho * Wo
-    L = _preamble(bin_path)
-    L.append("    int in_t, out_t;")
-    L.append(f"    OK(in_t = fortis_plan_tensor(p, {n_in}L * 4));")
-    L.append(f"    OK(out_t = fortis_plan_tensor(p, {n_out}L * 4));")
-    L.append(f"    OK(fortis_plan_conv3d(p, in_t, out_t, -1, w, w + {boff}, {C_}, {D}, {H}, {Wd}, {F}, {K}, {pad}, {ACT[act]}, {float(alpha)!r}f));")
-    L.append("    OK(fortis_plan_finalize(p, in_t, out_t));")
-    L.append("    fortis_host_t host = { .n_in = %d, .n_out = %d, .in_esz = 4, .out_esz = 4, .verdict = FORTIS_VERDICT_WHOLE, .graph = %d };"
-             % (n_in, n_out, 1 if graph else 0))
-    L.append("    OK(fortis_step_bind(p, &host));")
-    L.append("}")
-    with open(c_path, "w") as f:
-        f.write("\n".join(L) + "\n")
-    return c_path, bin_path

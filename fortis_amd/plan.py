@@ -165,10 +165,11 @@ class Plan:
         return self._L.fortis_plan_time_ms(self._p, iters, 1 if graph else 0)
 
 
-def mlp_plan(Ws, bs, acts, rows, alphas=None, in_norms=None, out_norms=None, mask_tail=0):
+def mlp_plan(Ws, bs, acts, rows, alphas=None, in_norms=None, out_norms=None, mask_tail=0, plan_cls=None):
     """Linear stack as a plan: optional x/in_norms, Linear+act layers, optional *out_norms, optional
-    masked-ReLU head (benchmarks/climsim/export_wide.py:27-28; mom6_zb/export_zb.py:10-16)."""
-    p = Plan()
+    masked-ReLU head (benchmarks/climsim/export_wide.py:27-28; mom6_zb/export_zb.py:10-16).  plan_cls: a class
+    with Plan's interface to fill instead (the op-list recorder of fortis_amd.shim_hip)."""
+    p = (plan_cls or Plan)()
     widths = [Ws[0].shape[1]] + [w.shape[0] for w in Ws]
     t_in = p.tensor(rows * widths[0])
     cur = t_in

@@ -118,6 +118,10 @@ typedef struct {
 } fortis_host_t;
 
 int  fortis_step_bind(fortis_plan* p, const fortis_host_t* host);
+/* Registers a function that builds and binds the step; it runs once, at the first use of any entry point
+ * below while no step is bound: the role of `if (!din) setup();` in the generated shim
+ * (driver/fortis_shim.py:64-73), which copies weights and host globals at the first call, not at load time. */
+void fortis_step_on_first_use(void (*bind)(void));
 /* Forgets the bound step, the stencil tables and the graph (tests; a host never calls it). */
 void fortis_step_reset(void);
 int  fortis_step_graph_active(void);    /* 1 once a captured graph is being replayed */

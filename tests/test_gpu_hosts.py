@@ -1,6 +1,7 @@
-"""The reference's own Fortran host programs, compiled from its sources and linked against this library
-(oracle/build_hosts.py): they call the entry points by bind(c) name exactly as they do in a FORTIS
-build, and their printed checksums and written fields are compared with the reference-held numbers."""
+"""Host programs linked against this library with step files from the FORTIS_BACKEND=hip generator
+(fortis_amd/hosts/build_hosts.py): the reference's own Fortran hosts compiled from its sources, which call the
+entry points by bind(c) name exactly as they do in a FORTIS build (their printed checksums and written fields are
+compared with the reference-held numbers), and plain C hosts for every verdict the generator handles."""
 import os
 import re
 import subprocess
@@ -9,16 +10,19 @@ import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
-REFBIN = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref")
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+REFBIN = os.path.join(ROOT, "build", "hosts")
 
 
-def run_host(name, cwd, env=None):
+def run_host(name, cwd, env=None, args=()):
     exe = os.path.join(REFBIN, name)
     if not os.path.exists(exe):
-        pytest.skip(f"{exe} not built (needs the reference sources and flang at build time)")
+        if name.endswith("_hip"):
+            pytest.skip(f"{exe} not built (needs the reference sources and flang at build time)")
+        raise AssertionError(f"{exe} is not built: run __graft_entry__.build()")
     e = dict(os.environ)
     e.update(env or {})
-    r = subprocess.run([exe], cwd=cwd, capture_output=True, text=True, timeout=120, env=e)
+    r = subprocess.run([exe] + [str(a) for a in args], cwd=cwd, capture_output=True, text=True, timeout=120, env=e)
     assert r.returncode == 0, r.stdout + r.stderr
     return r.stdout
 
@@ -76,7 +80,7 @@ import numpy as np
 root, golden = sys.argv[1], sys.argv[2]
 sys.path.insert(0, root)
 from oracle import oracle as O          # checker: field synthesis of the reference host only
-so = C.CDLL(os.path.join(root, "oracle", "_ref", "zb_lifted_step.so"))   # constructors: plan bound, tables configured
+so = C.CDLL(os.path.join(root, "build", "hosts", "zb_lifted_step.so"))   # constructors: plan bound, tables configured
 G = np.load(os.path.join(golden, "zb_native_golden.npz"))
 F = O.zb_fields(); P = O.zb_prep(F)
 p = lambda a: a.ctypes.data_as(C.c_void_p)
@@ -101,12 +105,92 @@ print("lifted step ok")
 
 
 def test_emitted_step_and_tables_drive_the_lifted_zb_step(gpu, golden, tmp_path):
-    """The files fortis_amd/emit.py writes for the lifted ZB host -- the step (plan + host facts) and the stencil
+    """The files the generator writes for the lifted ZB host -- the step (plan + host facts) and the stencil
     tables with their generated fortis_gather / fortis_scatter entries -- built into one shared object at build
     time and driven in the lifted host's call order (mom6_zb/host_fissioned.fir:732-740), in a process of its
     own because loading the object binds the step; results against the reference's native CPU build."""
-    root = os.path.dirname(REFBIN.rstrip("/")).rsplit("/oracle", 1)[0]
-    if not os.path.exists(os.path.join(REFBIN, "zb_lifted_step.so")):
-        pytest.skip("zb_lifted_step.so not built")
-    r = subprocess.run([os.sys.executable, "-c", _LIFTED_CHILD, root, golden], capture_output=True, text=True, timeout=180)
+    assert os.path.exists(os.path.join(REFBIN, "zb_lifted_step.so")), "zb_lifted_step.so is not built: run __graft_entry__.build()"
+    r = subprocess.run([os.sys.executable, "-c", _LIFTED_CHILD, ROOT, golden], capture_output=True, text=True, timeout=180)
     assert r.returncode == 0 and "lifted step ok" in r.stdout, r.stdout + r.stderr
+
+
+# ---- C hosts on generated step files: one per verdict of the fortis.host attribute ------------------------
+def _io(tmp_path, x):
+    fin, fout = os.path.join(tmp_path, "in.bin"), os.path.join(tmp_path, "out.bin")
+    np.ascontiguousarray(x).tofile(fin)
+    return fin, fout
+
+
+@pytest.mark.parametrize("mode", ["call", "dev"])
+def test_generated_unet_step_from_a_c_host(gpu, tmp_path, mode):
+    """Config 4 through the whole generator chain: fortis.host attribute text + outline.json + op list ->
+    step_tables.c -> C host calling mlp_forward (and the resident triple, whose graph is captured on call 2:
+    fortis.graph is set and the step has more kernels than the replay threshold)."""
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from fortis_amd import configs
+    from refmodels import unet_ref
+    from util import TOL, maxrel
+    case = configs.unet()
+    fin, fout = _io(tmp_path, case["x"])
+    out = run_host("unet_host", tmp_path, args=[mode, fin, fout, case["x"].nbytes, 4 * 256 * 256 * 4, 3])
+    y = np.fromfile(fout, np.float32).reshape(4, 256, 256)
+    assert maxrel(y, unet_ref(case)) < TOL, out
+
+
+def test_generated_tsrgan_step_from_a_c_host(gpu, tmp_path):
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from fortis_amd import configs
+    from refmodels import tsrgan_ref
+    from util import TOL, maxrel
+    case = configs.tsrgan()
+    fin, fout = _io(tmp_path, case["x"])
+    run_host("tsrgan_host", tmp_path, args=["call", fin, fout, case["x"].nbytes, 66 ** 3 * 3 * 4, 2])
+    y = np.fromfile(fout, np.float32).reshape(66, 66, 66, 3)
+    assert maxrel(y, tsrgan_ref(case)) < TOL
+
+
+def test_generated_batched_steps_from_a_c_host(gpu, tmp_path):
+    """Batched verdict in both forms: expanded (fortis_pack / mlp_forward_batched() / fortis_unpack) and the slice
+    form with a strided loop (step 2 from column 3: rows 2, 4, ... of the host's arrays, the others untouched)."""
+    from fortis_amd import configs
+    from oracle import oracle as O
+    from util import TOL, maxrel
+    case = configs.toy_mlp(200)
+    ref = O.mlp_f64(case["Ws"], case["bs"], case["acts"], case["X"])
+    fin, fout = _io(tmp_path, case["X"])
+    run_host("packed_host", tmp_path, args=["packed", fin, fout, case["X"].nbytes, 200 * 32 * 4, 2, 200])
+    assert maxrel(np.fromfile(fout, np.float32).reshape(200, 32), ref) < TOL
+    big = np.random.default_rng(9).uniform(-1, 1, (210, 64)).astype(np.float32)
+    fin, fout = _io(tmp_path, big)
+    run_host("strided_host", tmp_path, args=["slice", fin, fout, big.nbytes, 210 * 32 * 4])
+    out = np.fromfile(fout, np.float32).reshape(210, 32)
+    rows = np.arange(100) * 2 + 2
+    c100 = configs.toy_mlp(100)
+    assert maxrel(out[rows], O.mlp_f64(c100["Ws"], c100["bs"], c100["acts"], big[rows])) < TOL
+    assert not out[np.setdiff1d(np.arange(210), rows)].any()
+
+
+def test_generated_boundary_step_reads_host_globals_at_first_use(gpu, tmp_path):
+    """Boundary verdict: the host passes its own f64 column-major arrays, and the normalisation vectors are
+    arrays of the host object that it fills at run time -- the step binds at the first mlp_forward, as the
+    reference's setup() does, so it sees the filled values (zeros at load time would divide by zero)."""
+    from oracle import oracle as O
+    from util import TOL, maxrel
+    NI, NIN, NH, NOUT = 384, 124, 128, 128
+    rng = np.random.default_rng(4)                                  # the seeds of build_hosts.py
+    Ws = [(rng.standard_normal((NH, NIN)) / 11).astype(np.float32), (rng.standard_normal((NOUT, NH)) / 11).astype(np.float32)]
+    bs = [rng.standard_normal(NH).astype(np.float32), rng.standard_normal(NOUT).astype(np.float32)]
+    r2 = np.random.default_rng(14)
+    A = np.asfortranarray(r2.standard_normal((NI, NIN)))
+    mean, vmax, vmin, scale = r2.standard_normal(NIN), r2.uniform(2, 3, NIN), r2.uniform(0, 1, NIN), r2.uniform(0.5, 2, NOUT)
+    fin, fvec, fout = [os.path.join(tmp_path, n) for n in ("in.bin", "vec.bin", "out.bin")]
+    A.reshape(-1, order="F").tofile(fin)
+    np.concatenate([mean, vmax, vmin, scale]).tofile(fvec)
+    out = run_host("boundary_host", tmp_path, args=[fin, fvec, fout])
+    assert "boundary host ok" in out
+    B = np.fromfile(fout, np.float64).reshape(NOUT, NI).T
+    X = O.boundary_pre(A, mean, vmax, vmin)
+    ref = O.boundary_post(O.mlp_f64(Ws, bs, ["leaky", "none"], X, alphas=[0.15, 0]), scale, np.float64)
+    assert maxrel(B, ref) < TOL
