@@ -243,6 +243,65 @@ __device__ __forceinline__ void layer_group(const v4f (&a)[KGMAX], v4f* o, const
     for (int u = 0; u < NTG; u++) o[u] = acc[u];
 }
 
+// One layer of a narrow network (at most four 16-wide k groups and n-tiles) as straight-line code: NT and KG are
+// compile-time, so every weight and bias read is a per-lane base (set once per layer) plus a literal offset, no
+// branch separates the reads from the MFMAs and the compiler is free to issue the reads ahead.  The activation is
+// applied in place: a[0 .. NT) leave as the next layer's operand.
+template <int NT, int KG, bool WLDS>
+__device__ __forceinline__ void layer_fixed(v4f (&a)[4], const float* sWts, const gfloat* wall, int woff4, int boff, int lane,
+                                            int lq, int act, float alpha)
+{
+    v4f acc[NT];
+    const v4f* wl = (const v4f*)sWts + woff4 + lane;
+    const v4f* bl = (const v4f*)sWts + boff / 4 + lq;
+    const gv4f* wg = (const gv4f*)wall + woff4 + lane;
+    const gv4f* bg = (const gv4f*)wall + boff / 4 + lq;
+#pragma unroll
+    for (int u = 0; u < NT; u++) { if (WLDS) acc[u] = bl[u * 4]; else acc[u] = bg[u * 4]; }
+#pragma unroll
+    for (int kg = 0; kg < KG; kg++) {
+        v4f w[NT];
+#pragma unroll
+        for (int u = 0; u < NT; u++) { if (WLDS) w[u] = wl[(u * KG + kg) * 64]; else w[u] = wg[(u * KG + kg) * 64]; }
+#pragma unroll
+        for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].x, a[kg].x, acc[u], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].y, a[kg].y, acc[u], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].z, a[kg].z, acc[u], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].w, a[kg].w, acc[u], 0, 0, 0);
+    }
+    if (act == FORTIS_ACT_RELU) {
+#pragma unroll
+        for (int u = 0; u < NT; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) a[u][r] = fmaxf(acc[u][r], 0.f);
+    } else if (act == FORTIS_ACT_NONE) {
+#pragma unroll
+        for (int u = 0; u < NT; u++) a[u] = acc[u];
+    } else {
+#pragma unroll
+        for (int u = 0; u < NT; u++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) a[u][r] = apply_act(acc[u][r], act, alpha);
+    }
+}
+// The layer's shape picks its code once per layer (wave-uniform).
+template <bool WLDS>
+__device__ __forceinline__ void layer_narrow(v4f (&a)[4], const LayerRegs& R, const float* sWts, const gfloat* wall, int lane, int lq)
+{
+#define FORTIS_LF(NT_, KG_) case (NT_) * 4 + (KG_): layer_fixed<NT_, KG_, WLDS>(a, sWts, wall, R.woff / 4, R.boff, lane, lq, R.act, R.alpha); break;
+    switch (R.NT * 4 + R.KG) {
+        FORTIS_LF(1, 1) FORTIS_LF(1, 2) FORTIS_LF(1, 3) FORTIS_LF(1, 4)
+        FORTIS_LF(2, 1) FORTIS_LF(2, 2) FORTIS_LF(2, 3) FORTIS_LF(2, 4)
+        FORTIS_LF(3, 1) FORTIS_LF(3, 2) FORTIS_LF(3, 3) FORTIS_LF(3, 4)
+        FORTIS_LF(4, 1) FORTIS_LF(4, 2) FORTIS_LF(4, 3) FORTIS_LF(4, 4)
+        default: break;
+    }
+#undef FORTIS_LF
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Wave-independent, register-resident variant: ONE WAVE owns 16 rows from the gather (or the X load)
 // to the scatter (or the Y store), and the activations never leave its registers (see layer_group).
@@ -390,6 +449,10 @@ void chain_wave_kernel(ChainParams params)
         for (int l = 0; l < nlayers; l++) {
             asm volatile("" ::: "memory");
             const LayerRegs R = layer_regs(d, l);
+            if constexpr (NTMAX == 4 && !STENCIL) {       // (the general stencil form has no registers to spare for it)
+                layer_narrow<WLDS>(a, R, sWts, wall, lane, lq);
+                continue;
+            }
             // n-tiles in groups of four independent accumulators; the size of the last group is
             // dispatched once per layer
 #pragma unroll
@@ -465,7 +528,7 @@ void chain_wave_kernel(ChainParams params)
 
     const unsigned long long ntile = ((unsigned long long)rows + 15) / 16;
     const unsigned long long stride = (unsigned long long)gridDim.x * 4;
-    unsigned long long t = (unsigned long long)blockIdx.x * 4 + wave;
+    unsigned long long t = (unsigned long long)(STENCIL ? st_xcd_band_block() : blockIdx.x) * 4 + wave;
     TileIn cur, nxt;
     if (t < ntile) issue(cur, (unsigned)(t * 16));      // in flight while the weights are staged
     if (WLDS) {
@@ -493,6 +556,165 @@ void chain_wave_kernel(ChainParams params)
             process(cur);
             if (more) issue(cur, (unsigned)((t + stride) * 16));
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The stencil form for the tables that lifted column physics usually gives (the ZB step is one): every gather
+// slot has the same strides, the scatter's stores share theirs, gather and scatter visit the same cells, each
+// table has at most two same-cell scalars and two per-cell instructions, the network is narrow (every width at
+// most 64) with at most four outputs, and every array spans less than 4 GiB.  Same arithmetic and same
+// wave-per-16-rows layout as chain_wave_kernel<true>, with what those conditions allow taken out of the tile
+// loop: the lane's eight slot pointers stay in registers for the life of the (persistent) wave, scalar and store
+// pointers and all strides are wave-uniform scalar registers, a cell is decoded once and its element offsets are
+// 32-bit, and the expression interpreter looks at two scalars and two per-cell results instead of four and six.
+template <bool WLDS>
+__global__ __launch_bounds__(CH_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void chain_stencil_fast_kernel(ChainParams params)
+{
+    constexpr int NS = 2, NC = 2;
+    __shared__ ChainParams P;
+    extern __shared__ float4 smem4[];
+    params_to_lds(&P, CH_THREADS);
+    const ChainDesc& d = P.d;
+    const GatherArgs& g = P.g;
+    const ScatterArgs& sc = P.sc;
+    float* sWts = (float*)smem4;
+    const int wfloats = st_u(d.wfloats), nlayers = st_u(d.nlayers);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K0 = st_u(d.L[0].K), NO = st_u(d.L[nlayers - 1].N);
+    const unsigned rows = (unsigned)st_u((int)P.rows);
+    const int lrow = lane & 15, lq = lane >> 4;
+    const gfloat* wall = st_g(d.wall);
+    const gfloat* in_div = st_g(d.in_div);
+    const gfloat* out_mul = st_g(d.out_mul);
+    // ---- hoisted table values -------------------------------------------------------------------------------
+    const gfloat* gp[8];                                   // this lane's slots q = 16 (t / 4) + 4 lq + t % 4
+#pragma unroll
+    for (int t = 0; t < 8; t++) gp[t] = st_g(g.refs[16 * (t >> 2) + 4 * lq + (t & 3)].p);
+    const unsigned g_si = (unsigned)st_u(g.refs[0].si), g_sj = (unsigned)st_u(g.refs[0].sj), g_pl = (unsigned)st_u((int)g.refs[0].plane);
+    const unsigned o_si = (unsigned)st_u(sc.refs[0].si), o_sj = (unsigned)st_u(sc.refs[0].sj), o_pl = (unsigned)st_u((int)sc.refs[0].plane);
+    const bool o_as_g = g_si == o_si && g_sj == o_sj && g_pl == o_pl;
+    const gfloat* gsp[NS];
+    const gfloat* ssp[NS];
+    unsigned s_si[NS], s_sj[NS], s_pl[NS];
+    bool s_as_o[NS];
+#pragma unroll
+    for (int q = 0; q < NS; q++) {
+        gsp[q] = st_uptr(st_g(g.scal[q].p));
+        ssp[q] = st_uptr(st_g(sc.scal[q].p));
+        s_si[q] = (unsigned)st_u(sc.scal[q].si); s_sj[q] = (unsigned)st_u(sc.scal[q].sj); s_pl[q] = (unsigned)st_u((int)sc.scal[q].plane);
+        s_as_o[q] = s_si[q] == o_si && s_sj[q] == o_sj && s_pl[q] == o_pl;
+    }
+    gfloat* op[4];
+#pragma unroll
+    for (int n = 0; n < 4; n++) op[n] = st_uptr(st_g(sc.refs[n].p));       // entries past the outputs repeat store 0
+
+    struct TileIn { float x[8], gS[NS], sS[NS]; unsigned soff, row0; };
+    auto issue = [&](TileIn& in, unsigned row0) __attribute__((always_inline)) {
+        in.row0 = row0;
+        const unsigned row = row0 + lrow;
+        int i, j, kk;
+        st_row(g, row < rows ? row : 0, i, j, kk);
+        const unsigned goff = (unsigned)i * g_si + (unsigned)j * g_sj + (unsigned)kk * g_pl;
+        in.soff = o_as_g ? goff : (unsigned)i * o_si + (unsigned)j * o_sj + (unsigned)kk * o_pl;
+#pragma unroll
+        for (int t = 0; t < 8; t++) in.x[t] = gp[t][goff];
+#pragma unroll
+        for (int q = 0; q < NS; q++) in.gS[q] = gsp[q][goff];
+#pragma unroll
+        for (int q = 0; q < NS; q++) {
+            const unsigned off = s_as_o[q] ? in.soff : (unsigned)i * s_si[q] + (unsigned)j * s_sj[q] + (unsigned)kk * s_pl[q];
+            in.sS[q] = ssp[q][off];
+        }
+    };
+    auto process = [&](TileIn& in) __attribute__((always_inline)) {
+        const unsigned row = in.row0 + lrow;
+        const bool valid = row < rows;
+        v4f a[4];
+        {
+            StCellT<NS, NC> cell;
+#pragma unroll
+            for (int q = 0; q < NS; q++) cell.S[q] = in.gS[q];
+            st_cell_program(g, cell);
+            float tv[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) tv[t] = in.x[t];
+            st_chain_apply(g, cell, tv);
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const int q = 16 * (t >> 2) + 4 * lq + (t & 3);
+                float v = (valid && q < K0) ? tv[t] : 0.f;
+                if (in_div && q < K0) v = __fdiv_rn(v, in_div[q]);
+                a[t >> 2][t & 3] = v;
+            }
+            a[2] = a[3] = (v4f)(0.f);
+        }
+        // the matrix phase outranks the other waves' vector phases at the issue port: a wave that has its operands
+        // streams its MFMAs while the others decode and divide in the gaps (2.5 % on the 15.7 M-column grid)
+        __builtin_amdgcn_s_setprio(3);
+        for (int l = 0; l < nlayers; l++) {
+            asm volatile("" ::: "memory");
+            const LayerRegs R = layer_regs(d, l);
+            layer_narrow<WLDS>(a, R, sWts, wall, lane, lq);
+        }
+        __builtin_amdgcn_s_setprio(0);
+        asm volatile("" ::: "memory");
+        // outputs 0..3 of the row are in the lanes of the first quarter
+        float ov[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            ov[r] = a[0][r];
+            if (out_mul && r < NO) ov[r] = __fmul_rn(ov[r], out_mul[r]);
+        }
+        gfloat* Yraw = st_g(P.Yraw);
+        if (Yraw && valid && lq == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) if (r < NO) Yraw[(size_t)row * NO + r] = ov[r];
+        }
+        StCellT<NS, NC> cell;
+#pragma unroll
+        for (int q = 0; q < NS; q++) cell.S[q] = in.sS[q];
+        st_cell_program(sc, cell);
+        st_chain_apply(sc, cell, ov);
+        if (valid && lq == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) if (r < NO) op[r][in.soff] = ov[r];
+        }
+    };
+
+    const unsigned long long ntile = ((unsigned long long)rows + 15) / 16;
+    // Each XCD (workgroups b % 8 == x run on XCD x) walks its own contiguous eighth of the tiles, its workgroups
+    // side by side: a cell's 3 x 3 neighbourhood is read through one L2, and the halo rows of one round are the
+    // interior rows of that XCD's next.  Grids that are not a multiple of eight workgroups walk all tiles together.
+    unsigned long long t, tend, stride;
+    if (gridDim.x % 8 == 0) {
+        const unsigned long long per = (ntile + 7) / 8, x = blockIdx.x % 8;
+        t = x * per + (unsigned long long)(blockIdx.x / 8) * 4 + wave;
+        tend = (x + 1) * per < ntile ? (x + 1) * per : ntile;
+        stride = (unsigned long long)(gridDim.x / 8) * 4;
+    } else {
+        t = (unsigned long long)blockIdx.x * 4 + wave; tend = ntile; stride = (unsigned long long)gridDim.x * 4;
+    }
+    TileIn cur, nxt;
+    if (t < tend) issue(cur, (unsigned)(t * 16));       // in flight while the weights are staged
+    if (WLDS) {
+        const int n4 = wfloats / 4;
+        for (int i0 = tid; i0 < n4; i0 += 8 * CH_THREADS) {
+            v4f r[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) { const int i = i0 + u * CH_THREADS; r[u] = ((const gv4f*)wall)[i < n4 ? i : n4 - 1]; }
+#pragma unroll
+            for (int u = 0; u < 8; u++) { const int i = i0 + u * CH_THREADS; if (i < n4) ((v4f*)sWts)[i] = r[u]; }
+        }
+        __syncthreads();
+    }
+    for (; t < tend; t += stride) {
+        asm volatile("" ::: "memory");
+        const bool more = t + stride < tend;
+        if (more) issue(nxt, (unsigned)((t + stride) * 16));
+        process(cur);
+        if (more) cur = nxt;
     }
 }
 
@@ -674,6 +896,46 @@ void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows
     }
 }
 
+// Whether the tables and the network meet the conditions of chain_stencil_fast_kernel (see there).
+static bool stencil_fast_ok(const ChainParams& P, const StencilDev& g, const StencilDev& sc)
+{
+    static int off = -1;
+    if (off < 0) off = getenv("FORTIS_STENCIL_GENERIC") != nullptr;
+    if (off || chain_ntmax(P.d) > 4 || P.d.L[P.d.nlayers - 1].N > 4 || P.d.mask_tail) return false;
+    if (!P.g.uniform || !P.sc.refs_uniform) return false;
+    if (g.nscal > 2 || sc.nscal > 2 || g.ncell > 2 || sc.ncell > 2) return false;
+    if (P.g.count != P.sc.count || P.g.ni != P.sc.ni || P.g.ilo != P.sc.ilo || P.g.jlo != P.sc.jlo || P.g.sx != P.sc.sx || P.g.cells != P.sc.cells) return false;
+    // 32-bit element offsets: every array the kernel indexes spans less than 2^30 elements, strides are not negative
+    auto fits = [](const StencilDev& t) {
+        for (int a = 0; a < t.narrays; a++) if (t.plane[a] * (long)t.nk >= (1L << 30)) return false;
+        for (int r = 0; r < t.nrefs + t.nscal; r++) {
+            const fortis_ref_t& f = r < t.nrefs ? t.refs[r] : t.scal[r - t.nrefs];
+            if (f.si < 0 || f.sj < 0) return false;
+        }
+        return true;
+    };
+    return fits(g) && fits(sc);
+}
+
+template <bool WLDS>
+static void launch_stencil_fast(ChainParams& P, hipStream_t s)
+{
+    const size_t shmem = (size_t)(WLDS ? P.d.wfloats : 0) * sizeof(float);
+    static size_t attr = 0;
+    static long slots = 0;
+    if (shmem > attr || !slots) {
+        HIP_OK(hipFuncSetAttribute((const void*)chain_stencil_fast_kernel<WLDS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        attr = shmem;
+        int occ = 0;
+        HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void*)chain_stencil_fast_kernel<WLDS>, CH_THREADS, shmem));
+        slots = (long)(occ < 1 ? 1 : occ) * num_cus();
+    }
+    long grid = cdiv(P.rows, 64);
+    if (grid > slots) grid = slots;
+    hipLaunchKernelGGL((chain_stencil_fast_kernel<WLDS>), dim3((unsigned)grid), dim3(CH_THREADS), shmem, s, P);
+    HIP_OK(hipGetLastError());
+}
+
 void fortis_launch_chain_stencil(const ChainDesc& d, const StencilDev& g, const StencilDev& sc, long rows,
                                  const float* const* dG, float* const* dS, float* dY, hipStream_t s)
 {
@@ -682,5 +944,9 @@ void fortis_launch_chain_stencil(const ChainDesc& d, const StencilDev& g, const 
     fill_params(&P, d, nullptr, nullptr, rows, dY);
     st_make_args<const float*>(g, g.cells, dG, &P.g);
     st_make_args<float*>(sc, sc.cells, dS, &P.sc);
+    if (stencil_fast_ok(P, g, sc)) {
+        if (chain_wave_wlds(P.d)) launch_stencil_fast<true>(P, s); else launch_stencil_fast<false>(P, s);
+        return;
+    }
     launch_wave<true>(P, s);
 }

@@ -106,31 +106,35 @@ __device__ __forceinline__ float st_arith(int op, float a, float b)
         default: return __fdiv_rn(a, b);
     }
 }
-// operand of per-cell code: 1..8 scalar, 16+ constant (value inlined as cv), 32+ earlier result
-__device__ __forceinline__ float st_operand(int code, float cv, const float (&S)[ST_SCAL_MAX],
-                                            const float (&c)[ST_CELL_MAX])
+// operand of per-cell code: 1..8 scalar, 16+ constant (value inlined as cv), 32+ earlier result.
+// NS / NC: how many scalars / per-cell results the caller's tables can hold (the full table sizes by default; the
+// kernels for small tables pass less and save a select per slot they do not have).
+template <int NS, int NC>
+__device__ __forceinline__ float st_operand(int code, float cv, const float (&S)[NS], const float (&c)[NC])
 {
     float v = cv;
 #pragma unroll
-    for (int m = 0; m < ST_CELL_MAX; m++) v = (code == 32 + m) ? c[m] : v;
+    for (int m = 0; m < NC; m++) v = (code == 32 + m) ? c[m] : v;
 #pragma unroll
-    for (int s = 0; s < ST_SCAL_MAX; s++) v = (code == 1 + s) ? S[s] : v;
+    for (int s = 0; s < NS; s++) v = (code == 1 + s) ? S[s] : v;
     return v;
 }
 // Same-cell scalars and per-cell instruction results of one cell.
-struct StCell { float S[ST_SCAL_MAX]; float c[ST_CELL_MAX]; };
+template <int NS = ST_SCAL_MAX, int NC = ST_CELL_MAX>
+struct StCellT { float S[NS]; float c[NC]; };
+typedef StCellT<> StCell;
 
 // Evaluates the per-cell instructions on scalars already in cell.S.
-template <typename A>
-__device__ __forceinline__ void st_cell_program(const A& d, StCell& cell)
+template <typename A, int NS, int NC>
+__device__ __forceinline__ void st_cell_program(const A& d, StCellT<NS, NC>& cell)
 {
     const int ncell = st_u(d.ncell);
 #pragma unroll
-    for (int n = 0; n < ST_CELL_MAX; n++) {
+    for (int n = 0; n < NC; n++) {
         cell.c[n] = 0.f;
         if (n < ncell) {
             const StIns ci = d.cell[n];
-            cell.c[n] = st_arith(st_u(ci.op), st_operand(st_u(ci.a), ci.ca, cell.S, cell.c), st_operand(st_u(ci.b), ci.cb, cell.S, cell.c));
+            cell.c[n] = st_arith(st_u(ci.op), st_operand<NS, NC>(st_u(ci.a), ci.ca, cell.S, cell.c), st_operand<NS, NC>(st_u(ci.b), ci.cb, cell.S, cell.c));
         }
     }
 }
@@ -150,13 +154,13 @@ __device__ __forceinline__ void st_prepare(const A& d, int i, int j, int kk, StC
 // Runs the tv chain on N slot values at once: the loop over chain steps is a real loop (one table
 // read and one wave-uniform switch per step), each arm handles all N values, so the generated code
 // holds each operation once per arm instead of once per slot and step.
-template <int N, typename A>
-__device__ __forceinline__ void st_chain_apply(const A& d, const StCell& cell, float (&tv)[N])
+template <int N, typename A, int NS, int NC>
+__device__ __forceinline__ void st_chain_apply(const A& d, const StCellT<NS, NC>& cell, float (&tv)[N])
 {
     const int nchain = st_u(d.nchain);
     for (int n = 0; n < nchain; n++) {
         const StStep st = d.chain[n];
-        const float o = st_operand(st_u(st.code), st.cv, cell.S, cell.c);
+        const float o = st_operand<NS, NC>(st_u(st.code), st.cv, cell.S, cell.c);
         switch (st_u(st.op * 2 + (st.tv_left ? 1 : 0))) {
             case 0: case 1:
 #pragma unroll
@@ -184,6 +188,15 @@ __device__ __forceinline__ void st_chain_apply(const A& d, const StCell& cell, f
                 break;
         }
     }
+}
+// A wave-uniform pointer, told to the compiler: it then lives in scalar registers and a load through it takes its
+// per-lane part as a 32-bit offset.
+template <typename T>
+__device__ __forceinline__ T* st_uptr(T* p)
+{
+    const unsigned long long v = (unsigned long long)p;
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)v), hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(v >> 32));
+    return (T*)(((unsigned long long)hi << 32) | lo);
 }
 
 // Host: lowered table + device array pointers -> kernel arguments.
