@@ -18,6 +18,9 @@
 #define ST_THREADS 256
 typedef float st_v4f __attribute__((ext_vector_type(4)));
 
+// NQ: slots a thread loads and evaluates (the table's slot count rounded up to a size that is compiled; entries
+// past the table's own repeat slot 0 and are not stored).
+template <int NQ>
 __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, float* __restrict__ X, unsigned rows)
 {
     __shared__ GatherArgs d;
@@ -32,20 +35,20 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
         int i, j, kk;
         st_row(d, row, i, j, kk);
         // all slot loads are issued before any of them is consumed
-        float tv[FORTIS_MAX_REFS];
+        float tv[NQ];
         StCell cell;
         if (st_u(d.uniform)) {
             // every slot and scalar has the same strides: one element offset per cell, and a slot is its
             // pointer plus that offset (unused table entries repeat slot 0)
             const long off = st_off(d.refs[0], i, j, kk);
 #pragma unroll
-            for (int q = 0; q < FORTIS_MAX_REFS; q++) tv[q] = st_g(d.refs[q].p)[off];
+            for (int q = 0; q < NQ; q++) tv[q] = st_g(d.refs[q].p)[off];
 #pragma unroll
             for (int sI = 0; sI < ST_SCAL_MAX; sI++) cell.S[sI] = st_g(d.scal[sI].p)[off];
             st_cell_program(d, cell);
         } else {
 #pragma unroll
-            for (int q = 0; q < FORTIS_MAX_REFS; q++) {
+            for (int q = 0; q < NQ; q++) {
                 const StSlotT<const float*> sl = d.refs[q < n ? q : 0];
                 tv[q] = st_g(sl.p)[st_off(sl, i, j, kk)];
             }
@@ -53,17 +56,18 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
         }
         st_chain_apply(d, cell, tv);
 #pragma unroll
-        for (int q = 0; q < FORTIS_MAX_REFS; q++)
+        for (int q = 0; q < NQ; q++)
             if (q < n) lds[tid * n + q] = tv[q];
     }
     __syncthreads();
     const unsigned lim = (rows - row0 < ST_THREADS ? rows - row0 : ST_THREADS) * n;
     float* out = X + (size_t)row0 * n;
     // the block's rows are one contiguous run of X, which starts on a 16-byte boundary when X does (256 rows
-    // of n floats each): written as 16-byte vectors, the last few floats of a ragged block one by one
+    // of n floats each): written as 16-byte vectors, the last few floats of a ragged block one by one.  X is
+    // written once and read by another kernel: the stores are marked non-temporal.
     if (((uintptr_t)X & 15) == 0) {
         const unsigned lim4 = lim / 4;
-        for (unsigned idx = tid; idx < lim4; idx += ST_THREADS) ((st_v4f*)out)[idx] = ((const st_v4f*)lds)[idx];
+        for (unsigned idx = tid; idx < lim4; idx += ST_THREADS) __builtin_nontemporal_store(((const st_v4f*)lds)[idx], (st_v4f*)out + idx);
         for (unsigned idx = lim4 * 4 + tid; idx < lim; idx += ST_THREADS) out[idx] = lds[idx];
     } else {
         for (unsigned idx = tid; idx < lim; idx += ST_THREADS) out[idx] = lds[idx];
@@ -83,7 +87,7 @@ __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, c
     const float* in = Y + ((size_t)blockIdx.y * d.count + col0) * n;
     if (((uintptr_t)in & 15) == 0) {
         const unsigned lim4 = lim / 4;
-        for (unsigned idx = tid; idx < lim4; idx += ST_THREADS) ((st_v4f*)lds)[idx] = ((const st_v4f*)in)[idx];
+        for (unsigned idx = tid; idx < lim4; idx += ST_THREADS) ((st_v4f*)lds)[idx] = __builtin_nontemporal_load((const st_v4f*)in + idx);   // Y is read once
         for (unsigned idx = lim4 * 4 + tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
     } else {
         for (unsigned idx = tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
@@ -342,8 +346,13 @@ static void launch_gather(const StencilDev& low, const float* const* dA, float* 
     GatherArgs a;
     st_make_args<const float*>(low, low.cells, dA, &a);
     const unsigned rows = (unsigned)(low.count * low.nk);
-    hipLaunchKernelGGL(gather_kernel, dim3((unsigned)cdiv(rows, ST_THREADS)), dim3(ST_THREADS),
-                       (size_t)ST_THREADS * low.nrefs * sizeof(float), s, a, dX, rows);
+    const dim3 grid((unsigned)cdiv(rows, ST_THREADS)), block(ST_THREADS);
+    const size_t shmem = (size_t)ST_THREADS * low.nrefs * sizeof(float);
+    if (low.nrefs <= 8) hipLaunchKernelGGL(gather_kernel<8>, grid, block, shmem, s, a, dX, rows);
+    else if (low.nrefs <= 16) hipLaunchKernelGGL(gather_kernel<16>, grid, block, shmem, s, a, dX, rows);
+    else if (low.nrefs <= 24) hipLaunchKernelGGL(gather_kernel<24>, grid, block, shmem, s, a, dX, rows);
+    else if (low.nrefs <= 28) hipLaunchKernelGGL(gather_kernel<28>, grid, block, shmem, s, a, dX, rows);
+    else hipLaunchKernelGGL(gather_kernel<32>, grid, block, shmem, s, a, dX, rows);
     HIP_OK(hipGetLastError());
 }
 static void launch_scatter(const StencilDev& low, float* const* dA, const float* dY, int kk, hipStream_t s, int layers = 1)

@@ -211,7 +211,9 @@ __global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args
     float* dst = X + (size_t)row0 * n;
     if (((uintptr_t)dst & 15) == 0) {
         const unsigned t4 = total / 4;
-        for (unsigned v = tid; v < t4; v += SG_THREADS) ((float4*)dst)[v] = ((const float4*)tile)[v];
+        typedef float sg_v4f __attribute__((ext_vector_type(4)));
+        // X is written once and read by another kernel: non-temporal stores
+        for (unsigned v = tid; v < t4; v += SG_THREADS) __builtin_nontemporal_store(((const sg_v4f*)tile)[v], (sg_v4f*)dst + v);
         for (unsigned e = t4 * 4 + tid; e < total; e += SG_THREADS) dst[e] = tile[e];
     } else {
         for (unsigned e = tid; e < total; e += SG_THREADS) dst[e] = tile[e];
