@@ -302,6 +302,17 @@ __device__ __forceinline__ void layer_narrow(v4f (&a)[4], const LayerRegs& R, co
 #undef FORTIS_LF
 }
 
+// All layers of a narrow network on the operand in a[]; the result is left in a[].
+template <bool WLDS>
+__device__ __forceinline__ void layers_narrow(v4f (&a)[4], const ChainDesc& d, int nlayers, const float* sWts, const gfloat* wall, int lane, int lq)
+{
+    for (int l = 0; l < nlayers; l++) {
+        asm volatile("" ::: "memory");
+        const LayerRegs R = layer_regs(d, l);
+        layer_narrow<WLDS>(a, R, sWts, wall, lane, lq);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Wave-independent, register-resident variant: ONE WAVE owns 16 rows from the gather (or the X load)
 // to the scatter (or the Y store), and the activations never leave its registers (see layer_group).
@@ -446,13 +457,12 @@ void chain_wave_kernel(ChainParams params)
                     a[kg][s4] = v;
                 }
         }
+        if constexpr (NTMAX == 4 && !STENCIL) {           // (the general stencil form has no registers to spare for it)
+            layers_narrow<WLDS>(a, d, nlayers, sWts, wall, lane, lq);
+        } else
         for (int l = 0; l < nlayers; l++) {
             asm volatile("" ::: "memory");
             const LayerRegs R = layer_regs(d, l);
-            if constexpr (NTMAX == 4 && !STENCIL) {       // (the general stencil form has no registers to spare for it)
-                layer_narrow<WLDS>(a, R, sWts, wall, lane, lq);
-                continue;
-            }
             // n-tiles in groups of four independent accumulators; the size of the last group is
             // dispatched once per layer
 #pragma unroll
@@ -653,11 +663,7 @@ void chain_stencil_fast_kernel(ChainParams params)
         // the matrix phase outranks the other waves' vector phases at the issue port: a wave that has its operands
         // streams its MFMAs while the others decode and divide in the gaps (2.5 % on the 15.7 M-column grid)
         __builtin_amdgcn_s_setprio(3);
-        for (int l = 0; l < nlayers; l++) {
-            asm volatile("" ::: "memory");
-            const LayerRegs R = layer_regs(d, l);
-            layer_narrow<WLDS>(a, R, sWts, wall, lane, lq);
-        }
+        layers_narrow<WLDS>(a, d, nlayers, sWts, wall, lane, lq);
         __builtin_amdgcn_s_setprio(0);
         asm volatile("" ::: "memory");
         // outputs 0..3 of the row are in the lanes of the first quarter
@@ -715,6 +721,163 @@ void chain_stencil_fast_kernel(ChainParams params)
         if (more) issue(nxt, (unsigned)((t + stride) * 16));
         process(cur);
         if (more) cur = nxt;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Same conditions and same arithmetic as chain_stencil_fast_kernel, other division of labour: a wave takes 64
+// rows at a time and LANE = ROW for everything that is per row -- decoding the cell, loading its NQ slots and
+// scalars, the lifted expressions (the divisions), and at the end the scatter expressions and stores -- so each
+// of those instructions serves 64 rows instead of 16.  The evaluated slot values go through a per-wave LDS tile
+// ([64 rows][36 floats]: the pitch keeps the 16-byte reads of an m-tile conflict free) into the MFMA operand
+// layout; the four 16-row m-tiles then run the layers in registers as before and leave their outputs in a
+// second small LDS tile from which every lane picks up its own row.  The next 64 rows' loads are issued as soon
+// as the slot registers are free, i.e. before the four m-tiles are multiplied.
+#define CSR_PITCH 36
+#define CSR_THREADS 512      // eight waves share one LDS copy of the weights: four waves per SIMD stay resident
+template <bool WLDS, int NQ>
+__global__ __launch_bounds__(CSR_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void chain_stencil_rows_kernel(ChainParams params)
+{
+    constexpr int NS = 2, NC = 2;
+    __shared__ ChainParams P;
+    extern __shared__ float4 smem4[];
+    params_to_lds(&P, CSR_THREADS);
+    const ChainDesc& d = P.d;
+    const GatherArgs& g = P.g;
+    const ScatterArgs& sc = P.sc;
+    const int wfloats = st_u(d.wfloats), nlayers = st_u(d.nlayers);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float* sWts = (float*)smem4;
+    float* sOp = sWts + (WLDS ? wfloats : 0) + wave * (32 * CSR_PITCH + 64 * 4);   // this wave's operand tile (32 rows at a time)
+    float* sOut = sOp + 32 * CSR_PITCH;                                            // and its output tile [64][4]
+    const int K0 = st_u(d.L[0].K), NO = st_u(d.L[nlayers - 1].N);
+    const unsigned rows = (unsigned)st_u((int)P.rows);
+    const int lrow = lane & 15, lq = lane >> 4;
+    const gfloat* wall = st_g(d.wall);
+    const gfloat* in_div = st_g(d.in_div);
+    const gfloat* out_mul = st_g(d.out_mul);
+    const unsigned g_si = (unsigned)st_u(g.refs[0].si), g_sj = (unsigned)st_u(g.refs[0].sj), g_pl = (unsigned)st_u((int)g.refs[0].plane);
+    const unsigned o_si = (unsigned)st_u(sc.refs[0].si), o_sj = (unsigned)st_u(sc.refs[0].sj), o_pl = (unsigned)st_u((int)sc.refs[0].plane);
+    const bool o_as_g = g_si == o_si && g_sj == o_sj && g_pl == o_pl;
+
+    struct RowIn { float x[NQ], gS[NS], sS[NS]; unsigned soff, row; };
+    // ---- every global load of the 64 rows at row0; lane = row ----------------------------------------------
+    auto issue = [&](RowIn& in, unsigned row0) __attribute__((always_inline)) {
+        in.row = row0 + lane;
+        int i, j, kk;
+        st_row(g, in.row < rows ? in.row : 0, i, j, kk);
+        const unsigned goff = (unsigned)i * g_si + (unsigned)j * g_sj + (unsigned)kk * g_pl;
+        in.soff = o_as_g ? goff : (unsigned)i * o_si + (unsigned)j * o_sj + (unsigned)kk * o_pl;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) in.x[q] = st_uptr(st_g(g.refs[q].p))[goff];          // entries past the table's repeat slot 0
+#pragma unroll
+        for (int q = 0; q < NS; q++) in.gS[q] = st_uptr(st_g(g.scal[q].p))[goff];
+#pragma unroll
+        for (int q = 0; q < NS; q++) {
+            const unsigned ssi = (unsigned)st_u(sc.scal[q].si), ssj = (unsigned)st_u(sc.scal[q].sj), spl = (unsigned)st_u((int)sc.scal[q].plane);
+            const unsigned off = (ssi == o_si && ssj == o_sj && spl == o_pl) ? in.soff : (unsigned)i * ssi + (unsigned)j * ssj + (unsigned)kk * spl;
+            in.sS[q] = st_uptr(st_g(sc.scal[q].p))[off];
+        }
+    };
+
+    // per-XCD contiguous ranges of 64-row groups (see chain_stencil_fast_kernel)
+    const unsigned long long ngroup = ((unsigned long long)rows + 63) / 64;
+    unsigned long long t, tend, stride;
+    if (gridDim.x % 8 == 0) {
+        const unsigned long long per = (ngroup + 7) / 8, x = blockIdx.x % 8;
+        t = x * per + (unsigned long long)(blockIdx.x / 8) * 8 + wave;
+        tend = (x + 1) * per < ngroup ? (x + 1) * per : ngroup;
+        stride = (unsigned long long)(gridDim.x / 8) * 8;
+    } else {
+        t = (unsigned long long)blockIdx.x * 8 + wave; tend = ngroup; stride = (unsigned long long)gridDim.x * 8;
+    }
+    RowIn in;
+    if (t < tend) issue(in, (unsigned)(t * 64));        // in flight while the weights are staged
+    if (WLDS) {
+        const int n4 = wfloats / 4;
+        for (int i0 = tid; i0 < n4; i0 += 4 * CSR_THREADS) {
+            v4f r[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) { const int i = i0 + u * CSR_THREADS; r[u] = ((const gv4f*)wall)[i < n4 ? i : n4 - 1]; }
+#pragma unroll
+            for (int u = 0; u < 4; u++) { const int i = i0 + u * CSR_THREADS; if (i < n4) ((v4f*)sWts)[i] = r[u]; }
+        }
+        __syncthreads();
+    }
+    for (; t < tend; t += stride) {
+        asm volatile("" ::: "memory");
+        // ---- lane = row: expressions, then the row's operands into the wave's LDS tile -----------------------
+        const unsigned row = in.row, soff = in.soff;
+        const bool valid = row < rows;
+        float sS[NS];
+#pragma unroll
+        for (int q = 0; q < NS; q++) sS[q] = in.sS[q];
+        {
+            StCellT<NS, NC> cell;
+#pragma unroll
+            for (int q = 0; q < NS; q++) cell.S[q] = in.gS[q];
+            st_cell_program(g, cell);
+            st_chain_apply(g, cell, in.x);
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                float v = (valid && q < K0) ? in.x[q] : 0.f;
+                if (in_div && q < K0) v = __fdiv_rn(v, in_div[q]);
+                in.x[q] = v;
+            }
+        }
+        // ---- two halves of 32 rows: their operands through the LDS tile, two m-tiles through the layers ------
+        __builtin_amdgcn_s_setprio(3);
+#pragma unroll 1
+        for (int half = 0; half < 2; half++) {
+            if ((lane >> 5) == half) {
+                v4f* dst = (v4f*)(sOp + (lane & 31) * CSR_PITCH);
+#pragma unroll
+                for (int q4 = 0; q4 < 8; q4++) {
+                    v4f v;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) v[r] = 4 * q4 + r < NQ ? in.x[4 * q4 + r] : 0.f;
+                    dst[q4] = v;
+                }
+            }
+            asm volatile("" ::: "memory");
+            // the slot registers are free once the second half is written: the next 64 rows' loads go out here
+            if (half == 1 && t + stride < tend) issue(in, (unsigned)((t + stride) * 64));
+#pragma unroll 1
+            for (int T = 0; T < 2; T++) {
+                v4f a[4];
+                const v4f* src = (const v4f*)(sOp + (16 * T + lrow) * CSR_PITCH) + lq;
+                a[0] = src[0]; a[1] = src[4];
+                a[2] = a[3] = (v4f)(0.f);
+                layers_narrow<WLDS>(a, d, nlayers, sWts, wall, lane, lq);
+                if (lq == 0) ((v4f*)sOut)[32 * half + 16 * T + lrow] = a[0];
+            }
+            asm volatile("" ::: "memory");
+        }
+        __builtin_amdgcn_s_setprio(0);
+        asm volatile("" ::: "memory");
+        // ---- lane = row again: the row's outputs, scatter expressions, stores --------------------------------
+        const v4f o4 = ((const v4f*)sOut)[lane];
+        float ov[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            ov[r] = o4[r];
+            if (out_mul && r < NO) ov[r] = __fmul_rn(ov[r], out_mul[r]);
+        }
+        gfloat* Yraw = st_g(P.Yraw);
+        if (Yraw && valid) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) if (r < NO) Yraw[(size_t)row * NO + r] = ov[r];
+        }
+        StCellT<NS, NC> cell;
+#pragma unroll
+        for (int q = 0; q < NS; q++) cell.S[q] = sS[q];
+        st_cell_program(sc, cell);
+        st_chain_apply(sc, cell, ov);
+        if (valid) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) if (r < NO) st_uptr(st_g(sc.refs[r].p))[soff] = ov[r];
+        }
     }
 }
 
@@ -936,6 +1099,25 @@ static void launch_stencil_fast(ChainParams& P, hipStream_t s)
     HIP_OK(hipGetLastError());
 }
 
+template <bool WLDS, int NQ>
+static void launch_stencil_rows(ChainParams& P, hipStream_t s)
+{
+    const size_t shmem = ((size_t)(WLDS ? P.d.wfloats : 0) + (CSR_THREADS / 64) * (32 * CSR_PITCH + 64 * 4)) * sizeof(float);
+    static size_t attr = 0;
+    static long slots = 0;
+    if (shmem > attr || !slots) {
+        HIP_OK(hipFuncSetAttribute((const void*)chain_stencil_rows_kernel<WLDS, NQ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        attr = shmem;
+        int occ = 0;
+        HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void*)chain_stencil_rows_kernel<WLDS, NQ>, CSR_THREADS, shmem));
+        slots = (long)(occ < 1 ? 1 : occ) * num_cus();
+    }
+    long grid = cdiv(P.rows, CSR_THREADS);
+    if (grid > slots) grid = slots;
+    hipLaunchKernelGGL((chain_stencil_rows_kernel<WLDS, NQ>), dim3((unsigned)grid), dim3(CSR_THREADS), shmem, s, P);
+    HIP_OK(hipGetLastError());
+}
+
 void fortis_launch_chain_stencil(const ChainDesc& d, const StencilDev& g, const StencilDev& sc, long rows,
                                  const float* const* dG, float* const* dS, float* dY, hipStream_t s)
 {
@@ -945,7 +1127,17 @@ void fortis_launch_chain_stencil(const ChainDesc& d, const StencilDev& g, const 
     st_make_args<const float*>(g, g.cells, dG, &P.g);
     st_make_args<float*>(sc, sc.cells, dS, &P.sc);
     if (stencil_fast_ok(P, g, sc)) {
-        if (chain_wave_wlds(P.d)) launch_stencil_fast<true>(P, s); else launch_stencil_fast<false>(P, s);
+        // lane-per-row form from three of its rounds of the chip on (64 rows x 16 waves x CUs); below that the
+        // wave-per-16-rows form spreads the rows over more waves and finishes a partial round sooner.
+        // FORTIS_STENCIL_FORM=16|64 forces one of them.
+        static int form = -1;
+        if (form < 0) { const char* e = getenv("FORTIS_STENCIL_FORM"); form = e ? atoi(e) : 0; }
+        const bool v1 = form == 16 || (form != 64 && rows < 3L * 64 * 16 * num_cus());
+        const bool wlds = chain_wave_wlds(P.d);
+        if (v1) { if (wlds) launch_stencil_fast<true>(P, s); else launch_stencil_fast<false>(P, s); return; }
+        const int k0 = P.d.L[0].K;
+        if (wlds) { if (k0 <= 16) launch_stencil_rows<true, 16>(P, s); else if (k0 <= 28) launch_stencil_rows<true, 28>(P, s); else launch_stencil_rows<true, 32>(P, s); }
+        else { if (k0 <= 16) launch_stencil_rows<false, 16>(P, s); else if (k0 <= 28) launch_stencil_rows<false, 28>(P, s); else launch_stencil_rows<false, 32>(P, s); }
         return;
     }
     launch_wave<true>(P, s);

@@ -256,6 +256,55 @@ def test_bench_grid_fused_equals_unfused_and_layer_vs_oracle(L, gpu):
     plan.close()
 
 
+@pytest.mark.parametrize("form", ["16", "64"])
+@pytest.mark.parametrize("sx,sy,nz,hidden", [(68, 78, 15, (64, 64)), (37, 29, 3, (20,)), (133, 70, 2, (48, 16, 8))])
+def test_fused_step_both_fast_forms(L, gpu, form, sx, sy, nz, hidden):
+    """The two kernels behind the fused step for uniform-stride tables -- a wave per 16 rows, and a lane per row
+    with 64 rows per wave -- are chosen by the row count; both are forced here on grids of either size class
+    (ragged counts, a partial last group) in a process of their own, since the choice is read from the
+    environment once.  Y against the oracle's gather + fp64-accumulated network, fields bit-equal to the
+    oracle's scatter of the kernel's own Y."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = f"""
+import sys, ctypes as C, numpy as np
+sys.path.insert(0, {root!r}); sys.path.insert(0, {os.path.join(root, 'tests')!r})
+import fortis_amd
+from fortis_amd import configs, plan as P, stencil as S
+from oracle import oracle as O
+from util import TOL, DevBuf, bits_equal, maxrel, ptrs
+L = fortis_amd.load()
+sx, sy, nz, hidden = {sx}, {sy}, {nz}, {hidden!r}
+gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+gt, st = S.build_table(gd, lp, kd, "gather"), S.build_table(sd, lp, kd, "scatter")
+A = configs.zb_arrays(sx, sy, nz)
+count, n2, n3 = (sx - 4) * (sy - 4), sx * sy, sx * sy * nz
+rows = count * nz
+net = configs.zb_mlp(hidden)
+plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows)
+garr = [A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"]]
+host = [A["norm_h"], A["kappa_h"], np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+gb, sb = [DevBuf(L, a) for a in garr], [DevBuf(L, a) for a in host]
+dY = DevBuf(L, nbytes=rows * 3 * 4)
+assert L.fortis_stencil_step_fused(C.byref(gt), C.byref(st), plan.handle, ptrs(gb), ptrs(sb), dY.ptr) == 0
+L.fortis_sync()
+Y = dY.get((rows, 3))
+X = O.stencil_gather(gd, garr, count, nz, 3, 3, sx - 4)
+assert maxrel(Y, O.mlp_f64(net["Ws"], net["bs"], net["acts"], X)) < TOL
+ref = [a.copy() for a in host[:2]] + [np.zeros(n2, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+txy = np.zeros((nz, n2), np.float32)
+for kk in range(nz):
+    O.stencil_scatter(sd, ref, Y[kk * count:(kk + 1) * count], count, kk, 3, 3, sx - 4)
+    txy[kk] = ref[2]
+assert bits_equal(sb[3].get((n3,)), ref[3]) and bits_equal(sb[4].get((n3,)), ref[4]) and bits_equal(sb[2].get((nz, n2)), txy)
+print("forms ok")
+"""
+    env = dict(os.environ, FORTIS_STENCIL_FORM=form)
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110, env=env)
+    assert r.returncode == 0 and "forms ok" in r.stdout, r.stdout + r.stderr
+
+
 def test_fused_step_rejects_mismatched_tables(L, gpu, golden, capfd):
     gt, st, gd, sd, lp, kd = golden_tables(golden)
     net = configs.toy_mlp(64)
