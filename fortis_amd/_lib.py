@@ -9,7 +9,7 @@ class FortisLibraryMissing(RuntimeError):
     pass
 
 
-MAX_ARRAYS, MAX_REFS, MAX_SCAL, MAX_INS, MAX_CONST = 8, 32, 8, 12, 8
+MAX_ARRAYS, MAX_REFS, MAX_SCAL, MAX_INS, MAX_CONST = 8, 128, 8, 32, 16
 
 
 class Ref(C.Structure):

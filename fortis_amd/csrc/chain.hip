@@ -324,9 +324,9 @@ template <bool STENCIL, bool WLDS, int NTMAX>
 __global__ __launch_bounds__(CH_THREADS) __attribute__((amdgpu_waves_per_eu(NTMAX <= 4 ? 4 : 2, NTMAX <= 4 ? 4 : 2)))
 void chain_wave_kernel(ChainParams params)
 {
-    constexpr int KG0 = STENCIL ? FORTIS_MAX_REFS / 16 : NTMAX;   // k groups the first layer can read
+    constexpr int KG0 = STENCIL ? ST_KREFS / 16 : NTMAX;   // k groups the first layer can read
     constexpr bool PREFETCH = KG0 <= 4;                           // wide inputs: no second register set
-    constexpr int NTO = STENCIL ? FORTIS_MAX_REFS / 16 : NTMAX;   // n-tiles the output stage can write
+    constexpr int NTO = STENCIL ? ST_KREFS / 16 : NTMAX;   // n-tiles the output stage can write
     __shared__ ChainParams P;
     extern __shared__ float4 smem4[];
     params_to_lds(&P, CH_THREADS);

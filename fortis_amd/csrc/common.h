@@ -57,6 +57,7 @@ int fortis_chain_build(ChainDesc* d, int nlayers, const float* const* W, const f
                        const int* N, float** blob_out);
 void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows, hipStream_t s);
 // ---- stencil tables as the kernels see them (stencil.hip) --------------------------------
+#define ST_KREFS 32     // slots a kernel launch handles: the fused-form kernels take tables up to this, the general ones chunk
 struct CellStep { int op, code, tv_left; };
 struct StencilDev {
     int narrays;

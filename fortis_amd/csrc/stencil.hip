@@ -119,10 +119,10 @@ static bool g_lower_quiet = false;     // set while a table is only being tried 
 int fortis_stencil_lower(const fortis_stencil_t* in, StencilDev* out)
 {
     memset(out, 0, sizeof *out);
-    if (in->narrays < 1 || in->narrays > FORTIS_MAX_ARRAYS || in->nrefs < 1 || in->nrefs > FORTIS_MAX_REFS ||
+    if (in->narrays < 1 || in->narrays > FORTIS_MAX_ARRAYS || in->nrefs < 1 || in->nrefs > ST_KREFS ||
         in->nscal < 0 || in->nscal > ST_SCAL_MAX || in->nins < 0 || in->nins > FORTIS_MAX_INS ||
         in->nconst < 0 || in->nconst > FORTIS_MAX_CONST || in->count < 1 || in->nk < 1 ||
-        in->count * in->nk >= 4294967295L / FORTIS_MAX_REFS) {
+        in->count * in->nk >= 4294967295L / ST_KREFS) {
         LOWER_ERR("fortis: stencil table out of range\n");
         return -1;
     }

@@ -60,7 +60,7 @@ __device__ __forceinline__ void st_divmod(unsigned n, const StMagic& m, unsigned
 template <typename P>
 struct alignas(16) StencilArgsT {
     int nrefs, nscal, ncell, nchain;
-    StSlotT<P> refs[FORTIS_MAX_REFS];
+    StSlotT<P> refs[ST_KREFS];
     StSlotT<P> scal[ST_SCAL_MAX];
     StIns cell[ST_CELL_MAX];
     StStep chain[ST_CHAIN_MAX];
@@ -222,7 +222,7 @@ static inline void st_make_args(const StencilDev& low, const int* dcells, P cons
         a->chain[n] = s;
     }
     // unused table entries repeat slot 0, so that a kernel may load through any of them without a clamp
-    for (int r = low.nrefs; r < FORTIS_MAX_REFS; r++) a->refs[r] = a->refs[0];
+    for (int r = low.nrefs; r < ST_KREFS; r++) a->refs[r] = a->refs[0];
     for (int r = low.nscal; r < ST_SCAL_MAX; r++) a->scal[r] = a->refs[0];
     a->count = (unsigned)low.count;
     a->ilo = low.ilo; a->jlo = low.jlo; a->ni = low.ni; a->sx = low.sx;

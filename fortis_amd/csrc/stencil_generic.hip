@@ -16,7 +16,7 @@
 struct GenSlot { const void* p; long si, sj, plane; int f64, pad_; };   // p: array base with the element offset folded in
 struct alignas(16) GenArgs {
     int nrefs, nscal, nins, cellmask;      // cellmask: bit n set = instruction n does not depend on the slot value
-    GenSlot refs[FORTIS_MAX_REFS];
+    GenSlot refs[ST_KREFS];                // the slots of this launch (a larger table goes in several launches)
     GenSlot scal[FORTIS_MAX_SCAL];
     int op[FORTIS_MAX_INS], a[FORTIS_MAX_INS], b[FORTIS_MAX_INS];
     double consts[FORTIS_MAX_CONST];
@@ -171,7 +171,10 @@ __device__ __forceinline__ void sg_load_slots(const GenArgs& d, float* mine, int
 // evaluated in place in the workgroup's tile of X in LDS; the tile -- SG_THREADS consecutive rows, contiguous
 // in X -- is written out with coalesced 16-byte stores (a thread storing its own row strides by the row length).
 // Dynamic LDS: [nins + nscal][SG_THREADS] doubles (expression results, then the row's scalars), then the tile [SG_THREADS][nrefs] floats.
-__global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args, float* __restrict__ X, unsigned rows)
+// A table of more than ST_KREFS slots is gathered in several launches: a launch holds slots q0 .. q0 + nrefs - 1 of the
+// table and writes those columns of X, whose rows are `pitch` floats long.
+__global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args, float* __restrict__ X, unsigned rows, unsigned pitch,
+                                                                    unsigned q0)
 {
     __shared__ GenArgs d;
     extern __shared__ __attribute__((aligned(16))) double sg_dyn[];
@@ -209,7 +212,10 @@ __global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args
     __syncthreads();
     const unsigned nr = rows - row0 < SG_THREADS ? rows - row0 : SG_THREADS, total = nr * n;
     float* dst = X + (size_t)row0 * n;
-    if (((uintptr_t)dst & 15) == 0) {
+    if (pitch != (unsigned)n) {
+        // a column band of X: element e of the tile is slot e % n of row e / n
+        for (unsigned e = tid; e < total; e += SG_THREADS) X[(size_t)(row0 + e / n) * pitch + q0 + e % n] = tile[e];
+    } else if (((uintptr_t)dst & 15) == 0) {
         const unsigned t4 = total / 4;
         typedef float sg_v4f __attribute__((ext_vector_type(4)));
         // X is written once and read by another kernel: non-temporal stores
@@ -221,7 +227,8 @@ __global__ __launch_bounds__(SG_THREADS) void gather_generic_kernel(GenArgs args
 }
 
 // One thread per cell of layer kk.  Dynamic LDS: [nins + nscal][SG_THREADS] doubles (expression results, scalars).
-__global__ __launch_bounds__(SG_THREADS) void scatter_generic_kernel(GenArgs args, const float* __restrict__ Y, int kk)
+__global__ __launch_bounds__(SG_THREADS) void scatter_generic_kernel(GenArgs args, const float* __restrict__ Y, int kk, unsigned pitch,
+                                                                     unsigned q0)
 {
     __shared__ GenArgs d;
     extern __shared__ __attribute__((aligned(16))) double sg_dyn[];
@@ -235,7 +242,7 @@ __global__ __launch_bounds__(SG_THREADS) void scatter_generic_kernel(GenArgs arg
     sg_scalars(d, r, tid, i, j, kk);
     const long off0 = (long)i * d.refs[0].si + (long)j * d.refs[0].sj + (long)kk * d.refs[0].plane;
     const int n = st_u(d.nrefs);
-    const float* in = Y + (size_t)col * n;
+    const float* in = Y + (size_t)col * pitch + q0;          // this launch's outputs of the cell's row
     sg_eval(d, 0.f, r, tid, 1);
     for (int q = 0; q < n; q++) {
         const GenSlot& sl = d.refs[q];
@@ -251,7 +258,7 @@ int fortis_stencil_validate(const fortis_stencil_t* t)
 {
     if (t->narrays < 1 || t->narrays > FORTIS_MAX_ARRAYS || t->nrefs < 1 || t->nrefs > FORTIS_MAX_REFS || t->nscal < 0 ||
         t->nscal > FORTIS_MAX_SCAL || t->nins < 0 || t->nins > FORTIS_MAX_INS || t->nconst < 0 ||
-        t->nconst > FORTIS_MAX_CONST || t->count < 1 || t->nk < 1 || t->count * t->nk >= 4294967295L / FORTIS_MAX_REFS) {
+        t->nconst > FORTIS_MAX_CONST || t->count < 1 || t->nk < 1 || t->count * t->nk >= 4294967295L / t->nrefs) {
         fprintf(stderr, "fortis: stencil table out of range\n");
         return -1;
     }
@@ -319,13 +326,14 @@ bool fortis_stencil_typed(const fortis_stencil_t* t)
     return t->nscal > ST_SCAL_MAX;
 }
 
-static void sg_make_args(const fortis_stencil_t& t, const int* dcells, const void* const* arrays, GenArgs* g)
+// Kernel arguments for slots q0 .. q0 + nq - 1 of the table.
+static void sg_make_args(const fortis_stencil_t& t, const int* dcells, const void* const* arrays, GenArgs* g, int q0, int nq)
 {
     memset(g, 0, sizeof *g);
-    g->nrefs = t.nrefs; g->nscal = t.nscal; g->nins = t.nins;
-    for (int r = 0; r < t.nrefs + t.nscal; r++) {
-        const fortis_ref_t& f = r < t.nrefs ? t.refs[r] : t.scal[r - t.nrefs];
-        GenSlot& s = r < t.nrefs ? g->refs[r] : g->scal[r - t.nrefs];
+    g->nrefs = nq; g->nscal = t.nscal; g->nins = t.nins;
+    for (int r = 0; r < nq + t.nscal; r++) {
+        const fortis_ref_t& f = r < nq ? t.refs[q0 + r] : t.scal[r - nq];
+        GenSlot& s = r < nq ? g->refs[r] : g->scal[r - nq];
         s.p = (const char*)arrays[f.array] + f.base * sg_esz(t, f.array);
         s.si = f.si; s.sj = f.sj;
         s.plane = f.planar ? t.plane[f.array] : 0;
@@ -336,7 +344,7 @@ static void sg_make_args(const fortis_stencil_t& t, const int* dcells, const voi
         // depends on the slot value: reads it, or reads the result of an instruction that does
         auto dep = [&](int code) { return code == 0 || (code >= 32 && !((g->cellmask >> (code - 32)) & 1)); };
         const bool binary = (t.ins[n].op & 0xff) <= FORTIS_OP_MIN;
-        if (!dep(t.ins[n].a) && !(binary && dep(t.ins[n].b))) g->cellmask |= 1 << n;
+        if (!dep(t.ins[n].a) && !(binary && dep(t.ins[n].b))) g->cellmask |= 1u << n;
     }
     for (int c = 0; c < t.nconst; c++) g->consts[c] = t.cdouble[c] ? t.dconsts[c] : (double)t.consts[c];
     // Chain form: every slot-dependent instruction combines the previous one's result (the slot value for the
@@ -363,9 +371,9 @@ static void sg_make_args(const fortis_stencil_t& t, const int* dcells, const voi
         g->nchain = ok ? nch : -1;
     }
     g->slotkind = g->refs[0].f64;
-    for (int r = 1; r < t.nrefs; r++) if (g->refs[r].f64 != g->refs[0].f64) g->slotkind = 2;
+    for (int r = 1; r < nq; r++) if (g->refs[r].f64 != g->refs[0].f64) g->slotkind = 2;
     g->uniform = 1;
-    for (int r = 1; r < t.nrefs; r++)
+    for (int r = 1; r < nq; r++)
         if (g->refs[r].si != g->refs[0].si || g->refs[r].sj != g->refs[0].sj || g->refs[r].plane != g->refs[0].plane) g->uniform = 0;
     g->count = (unsigned)t.count;
     g->ilo = t.ilo; g->jlo = t.jlo; g->ni = t.ni > 0 ? t.ni : 1; g->sx = t.sx > 0 ? t.sx : 1;
@@ -377,24 +385,39 @@ static void sg_make_args(const fortis_stencil_t& t, const int* dcells, const voi
 
 void fortis_launch_gather_generic(const fortis_stencil_t& t, const int* dcells, const void* const* dA, float* dX, hipStream_t s)
 {
-    GenArgs g;
-    sg_make_args(t, dcells, dA, &g);
     const unsigned rows = (unsigned)(t.count * t.nk);
-    const size_t shmem = (size_t)SG_THREADS * ((t.nins + t.nscal) * sizeof(double) + t.nrefs * sizeof(float));   // at most 72 KB
     static bool sized = false;
     if (!sized) {
         HIP_OK(hipFuncSetAttribute((const void*)gather_generic_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   SG_THREADS * (int)((FORTIS_MAX_INS + FORTIS_MAX_SCAL) * sizeof(double) + FORTIS_MAX_REFS * sizeof(float))));
+                                   SG_THREADS * (int)((FORTIS_MAX_INS + FORTIS_MAX_SCAL) * sizeof(double) + ST_KREFS * sizeof(float))));   // 112 KB
+        HIP_OK(hipFuncSetAttribute((const void*)scatter_generic_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   SG_THREADS * (int)((FORTIS_MAX_INS + FORTIS_MAX_SCAL) * sizeof(double))));
         sized = true;
     }
-    hipLaunchKernelGGL(gather_generic_kernel, dim3((unsigned)cdiv(rows, SG_THREADS)), dim3(SG_THREADS), shmem, s, g, dX, rows);
-    HIP_OK(hipGetLastError());
+    for (int q0 = 0; q0 < t.nrefs; q0 += ST_KREFS) {
+        const int nq = t.nrefs - q0 < ST_KREFS ? t.nrefs - q0 : ST_KREFS;
+        GenArgs g;
+        sg_make_args(t, dcells, dA, &g, q0, nq);
+        const size_t shmem = (size_t)SG_THREADS * ((t.nins + t.nscal) * sizeof(double) + nq * sizeof(float));
+        hipLaunchKernelGGL(gather_generic_kernel, dim3((unsigned)cdiv(rows, SG_THREADS)), dim3(SG_THREADS), shmem, s, g, dX, rows,
+                           (unsigned)t.nrefs, (unsigned)q0);
+        HIP_OK(hipGetLastError());
+    }
 }
 void fortis_launch_scatter_generic(const fortis_stencil_t& t, const int* dcells, void* const* dA, const float* dY, int kk, hipStream_t s)
 {
-    GenArgs g;
-    sg_make_args(t, dcells, (const void* const*)dA, &g);
-    hipLaunchKernelGGL(scatter_generic_kernel, dim3((unsigned)cdiv(t.count, SG_THREADS)), dim3(SG_THREADS),
-                       (size_t)SG_THREADS * (t.nins + t.nscal) * sizeof(double), s, g, dY, kk);
-    HIP_OK(hipGetLastError());
+    static bool sized = false;
+    if (!sized) {
+        HIP_OK(hipFuncSetAttribute((const void*)scatter_generic_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   SG_THREADS * (int)((FORTIS_MAX_INS + FORTIS_MAX_SCAL) * sizeof(double))));
+        sized = true;
+    }
+    for (int q0 = 0; q0 < t.nrefs; q0 += ST_KREFS) {
+        const int nq = t.nrefs - q0 < ST_KREFS ? t.nrefs - q0 : ST_KREFS;
+        GenArgs g;
+        sg_make_args(t, dcells, (const void* const*)dA, &g, q0, nq);
+        hipLaunchKernelGGL(scatter_generic_kernel, dim3((unsigned)cdiv(t.count, SG_THREADS)), dim3(SG_THREADS),
+                           (size_t)SG_THREADS * (t.nins + t.nscal) * sizeof(double), s, g, dY, kk, (unsigned)t.nrefs, (unsigned)q0);
+        HIP_OK(hipGetLastError());
+    }
 }

@@ -43,7 +43,12 @@ def compile_exprs(exprs, scalar_f64=None):
         return code
 
     def const(value, f64):
-        consts.append((float(value) if f64 else float(np.float32(value)), f64))
+        entry = (float(value) if f64 else float(np.float32(value)), f64)
+        if entry in consts and not (entry[0] == 0 and np.signbit(entry[0]) != np.signbit(consts[consts.index(entry)][0])):
+            code = 16 + consts.index(entry)        # a literal seen before (same value, same type) is one constant
+            typ[code] = f64
+            return code
+        consts.append(entry)
         code = 16 + len(consts) - 1
         typ[code] = f64
         return code

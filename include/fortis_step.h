@@ -162,18 +162,19 @@ typedef struct { int array; int planar; long base, si, sj; } fortis_ref_t;
  * table builder marks with FORTIS_INS_F64 in op; the assignment back to tv at the end of an
  * expression is an explicit conversion (op 11) where the expression's type is double; the
  * f-suffixed functions convert their operands to float first.
- * Tables whose expressions are one chain of + - * / on the slot value over fp32 arrays (tv op c,
- * c op tv) run in the fused kernels; anything else takes the general kernels. */
+ * Tables of at most 32 slots whose expressions are one chain of + - * / on the slot value over fp32 arrays
+ * (tv op c, c op tv; at most 6 chained and 6 per-cell operations) run in the fused kernels; anything else takes
+ * the general kernels, which take a table's slots 32 at a time. */
 typedef struct { int op, a, b; } fortis_ins_t;
 #define FORTIS_INS_F64 0x100
 enum { FORTIS_OP_ADD = 0, FORTIS_OP_SUB, FORTIS_OP_MUL, FORTIS_OP_DIV, FORTIS_OP_MAX, FORTIS_OP_MIN,
        FORTIS_OP_NEG, FORTIS_OP_SQRT, FORTIS_OP_EXP, FORTIS_OP_LOG, FORTIS_OP_TANH, FORTIS_OP_F32 };
 
 #define FORTIS_MAX_ARRAYS 8
-#define FORTIS_MAX_REFS 32
+#define FORTIS_MAX_REFS 128   /* e.g. a 5 x 5 neighbourhood of five arrays */
 #define FORTIS_MAX_SCAL 8
-#define FORTIS_MAX_INS 12
-#define FORTIS_MAX_CONST 8
+#define FORTIS_MAX_INS 32
+#define FORTIS_MAX_CONST 16
 
 typedef struct {
     int  narrays;

@@ -50,9 +50,10 @@ def _gather(L, gd, lp, kd, garr):
     gt = S.build_table(gd, lp, kd, "gather")
     assert L.fortis_stencil_route(C.byref(gt)) == 1
     bufs = [DevBuf(L, a) for a in garr]
-    dX = DevBuf(L, nbytes=COUNT * NZ * 27 * 4)
+    n = len(gd["slots"])
+    dX = DevBuf(L, nbytes=COUNT * NZ * n * 4)
     L.fortis_stencil_gather_dev(C.byref(gt), ptrs(bufs), dX.ptr)
-    X = dX.get((COUNT * NZ, 27))
+    X = dX.get((COUNT * NZ, n))
     for b in bufs + [dX]:
         b.free()
     return X
@@ -87,6 +88,47 @@ def test_general_gather_bit_exact(L, gpu, exprs, g64):
             a["elt"] = "f32"
         ref32 = O.stencil_gather_typed(gd32, [np.asarray(a, np.float32) for a in garr], COUNT, NZ, 3, 3, SX - 4)
         assert not bits_equal(ref32, ref)
+
+
+@pytest.mark.parametrize("g64", [(), (1, 3)])
+def test_wide_stencil_and_long_expression(L, gpu, g64):
+    """A 5 x 5 neighbourhood of three arrays (75 slots) with a 21-operation expression: more slots than one
+    launch of the kernels holds (they go 32 at a time, the last launch 11) and more operations than the fused
+    form chains; an fp32 chain-form table of 75 slots takes the general kernels too.  Gather bit-exact; the
+    scatter of 40 outputs per cell onto five arrays' worth of stores likewise."""
+    gd, sd, lp, kd, garr, sarr = _case(g64=g64)
+    gd["slots"] = [dict(array=a, idx=[["i", di], ["j", dj], ["v", 0]]) for a in range(3) for dj in (-2, -1, 0, 1, 2) for di in (-2, -1, 0, 1, 2)]
+    gd["n"] = 75
+    gt = S.build_table(gd, lp, kd, "gather")
+    assert gt.nrefs == 75 and L.fortis_stencil_route(C.byref(gt)) == 1       # chain form, but wider than the fused kernels
+    X = _gather(L, gd, lp, kd, garr)
+    assert bits_equal(X, O.stencil_gather_typed(gd, garr, COUNT, NZ, 3, 3, SX - 4))
+    gd["exprs"] = ["((((((((((tv + 1.0f) * 2.0f) - 3.0f) * 0.5f) + S0) * S0) - 1.0f) * 2.0f) + 0.25f) / (S0 + 2.0f))",
+                   "(((((((((tv * 0.5f) + 0.125f) * S0) - tv) + ((S0 * S0) + 1.0f)) * 0.75f) - 2.0f) + (tv * tv)) * 1.5f)"]
+    assert S.build_table(gd, lp, kd, "gather").nins >= 21
+    X = _gather(L, gd, lp, kd, garr)
+    assert bits_equal(X, O.stencil_gather_typed(gd, garr, COUNT, NZ, 3, 3, SX - 4))
+    # scatter: 40 outputs per cell, store q to array 2 + q % 3 of the ZB scatter descriptor at (i + q / 3 - 6, j)
+    sd = copy.deepcopy(sd)
+    sd["n"] = 40
+    sd["stores"] = [dict(slot=q, array=2 + q % 3, idx=([["i", q // 3 - 6], ["j", 0]] if q % 3 == 0 else [["i", q // 3 - 6], ["j", 0], ["v", 0]])) for q in range(40)]
+    # a cell list 16 apart along i, so that no two cells' 14 shifted stores into one array meet
+    cells = np.array([(i - 1) + (j - 1) * SX for j in range(3, SY - 1) for i in (9, 25)], np.int32)
+    cnt = len(cells)
+    st = S.build_table(sd, lp, kd, "scatter", cells=cells)
+    assert st.nrefs == 40 and L.fortis_stencil_route(C.byref(st)) == 1
+    Y = np.random.default_rng(5).standard_normal((cnt * NZ, 40)).astype(np.float32)
+    ref = [a.copy() for a in sarr]
+    sb = [DevBuf(L, a) for a in sarr]
+    dY = DevBuf(L, Y)
+    for kk in range(NZ):
+        L.fortis_stencil_scatter_dev(C.byref(st), ptrs(sb), C.c_void_p(dY.ptr + kk * cnt * 40 * 4), kk)
+        O.stencil_scatter_typed(sd, ref, Y[kk * cnt:(kk + 1) * cnt], cnt, kk, cells=cells)
+    for b, r in zip(sb[2:], ref[2:]):
+        got = b.get(r.shape, r.dtype)
+        assert np.array_equal(got.view(np.uint8), r.view(np.uint8)) and np.abs(r).max() > 0
+    for b in sb + [dY]:
+        b.free()
 
 
 def test_general_gather_libm_functions(L, gpu):
