@@ -456,9 +456,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20, help="untimed steps first; the clocks need about ten steps of this size to settle")
-    ap.add_argument("--workload", default="climsim", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan"])
+    ap.add_argument("--workload", default=None, help="default: climsim, followed by short runs of the other configurations (others)", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-others", action="store_true", help="default workload only: skip the short runs of the other configurations")
+    ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other configurations that follow the default workload")
     ap.add_argument("--f64", action="store_true", help="zb_unfused only: double-precision host arrays (the general stencil kernels)")
     ap.add_argument("--grid", default=None, help="zb / zb_ref / zb_unfused only: SXxSYxNZ grid instead of the reference's 68x78x15 (zb_unfused: 1028x1028x15)")
     args = ap.parse_args()
@@ -472,6 +472,8 @@ def main():
     if L.fortis_device_info(name, 64, None) != 0:
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
+    with_others = args.workload is None and not args.no_others
+    args.workload = args.workload or "climsim"
     r = run_workload(L, args, args.workload)
     ms_per_step = r["dt"] / args.steps * 1e3
     unit = r.get("unit", "columns/s")
@@ -481,7 +483,7 @@ def main():
             "config": r["config"], "roofline": r["roofline"]}
     if "cpu_baseline" in r:
         line["cpu_baseline"] = r["cpu_baseline"]
-    if args.workload == "climsim" and not args.no_others:
+    if with_others:
         line["others"] = run_others(L, args)
     print(json.dumps(line))
 
