@@ -26,10 +26,10 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # same command (see profiles/), or None where no counter run has been made for the workload.
-MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((2482.4 * 2 + 936.6) * 1024),
-                    "zb_ref": int((2396.6 * 2 + 936.6) * 1024), "zb_1028x1028x15": int((331322.2 * 2 + 207387.3) * 1024), "toy": None,
-                    "zb_unfused_1028x1028x15": int((242224.0 * 2 + 1658880.0) * 1024),
-                    "zb_unfused_1028x1028x15_f64": int((248700.0 * 2 + 1658880.0) * 1024),
+MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((1114.1 * 2 + 885.2) * 1024),
+                    "zb_ref": None, "zb_1028x1028x15": int((200550.7 * 2 + 193387.2) * 1024), "toy": None,
+                    "zb_unfused_1028x1028x15": int((242212.5 * 2 + 1658926.8) * 1024),
+                    "zb_unfused_1028x1028x15_f64": int((247386.7 * 2 + 1658898.9) * 1024),
                     # conv workloads: every conv, split-reduce and thin-head dispatch of a step summed, divided by the
                     # step's conv operations (18 and 19), like flop_per_launch
                     "unet": int((1163560.2 * 2 + 727552.0) * 1024 / 7 / 18), "tsrgan": int((3255367.7 * 2 + 5167927.1) * 1024 / 7 / 19)}
@@ -209,16 +209,26 @@ def run_zb_unfused(L, args):
         for kk in range(nz):
             L.fortis_stencil_scatter_dev(C.byref(st), dS, C.c_void_p(dY + kk * count * 3 * 4), kk)
     scatter_cb = CB(scatter_all)
-    for cb in (gather_cb, scatter_cb):
-        L.fortis_time_ms(cb, None, max(1, args.warmup))
-    plan.time_ms(max(1, args.warmup))
+    mlp_cb = CB(lambda _: plan.run())
+    parts = (CB * 3)(gather_cb, mlp_cb, scatter_cb)
+
+    def step():
+        gather_cb(None)
+        plan.run()
+        scatter_all(None)
+    for _ in range(max(1, args.warmup)):
+        step()
     L.fortis_sync()
+    # clocked pass: the step's own launches only, in the step's order; then the same steps with an event
+    # between the parts (gather / MLP / the scatter launches), each part right behind the one before it
     t0 = time.perf_counter()
-    g_ms = L.fortis_time_ms(gather_cb, None, args.steps) / args.steps
-    m_ms = plan.time_ms(args.steps) / args.steps
-    s_ms = L.fortis_time_ms(scatter_cb, None, args.steps) / args.steps
+    for _ in range(args.steps):
+        step()
     L.fortis_sync()
     dt = time.perf_counter() - t0
+    ms = (C.c_float * 3)()
+    assert L.fortis_time_parts_ms(3, parts, None, args.steps, ms) == 0
+    g_ms, m_ms, s_ms = (v / args.steps for v in ms)
     g_bytes = esz * 4 * n3 + 4 * 27 * rows                 # 4 planes read once, X written
     s_bytes = 4 * 3 * rows + esz * (n3 + nz * sx * sy + 3 * rows)  # Y read, norm + kappa read per layer, 3 outputs written
     gbs = g_bytes / (g_ms * 1e-3) / 1e9
@@ -227,7 +237,7 @@ def run_zb_unfused(L, args):
                 unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(g_ms, 5), bytes_per_launch=g_bytes,
                 scatter_GBs=round(s_bytes / (s_ms * 1e-3) / 1e9, 1), scatter_ms_all_layers=round(s_ms, 5), mlp_ms=round(m_ms, 5),
                 traffic=MEASURED_TRAFFIC.get("zb_unfused_%dx%dx%d%s" % (sx, sy, nz, "_f64" if args.f64 else "")))
-    out = dict(rows=rows, dt=(g_ms + m_ms + s_ms) * 1e-3 * args.steps, wall_dt=dt, dtype="f32",
+    out = dict(rows=rows, dt=dt, dtype="f32",
                config={"workload": "zb_unfused_gather_mlp_scatter_27_64_64_3_%dx%dx%d%s" % (sx, sy, nz, "_f64_arrays" if args.f64 else ""), "columns": rows,
                        "cells_per_layer": count, "layers": nz, "launches_per_step": 1 + nz + plan.num_kernels},
                roofline=roof)

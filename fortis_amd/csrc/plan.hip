@@ -1016,6 +1016,33 @@ float fortis_time_ms(void (*fn)(void*), void* arg, int iters)
     HIP_OK(hipEventDestroy(e0)); HIP_OK(hipEventDestroy(e1));
     return ms;
 }
+// A step made of several enqueues, clocked part by part: events between the parts, no host wait inside a
+// pass, so every part runs right behind the one before it as it does in the step itself.
+int fortis_time_parts_ms(int nparts, void (*const* fns)(void*), void* const* args, int iters, float* ms_out)
+{
+    if (nparts <= 0 || nparts > 16 || iters <= 0 || iters > 4096 || !fns || !ms_out) return -1;
+    hipStream_t s = fortis_stream_get();
+    std::vector<hipEvent_t> ev((size_t)iters * (nparts + 1));
+    for (auto& e : ev) HIP_OK(hipEventCreate(&e));
+    for (int it = 0; it < iters; it++) {
+        hipEvent_t* e = &ev[(size_t)it * (nparts + 1)];
+        HIP_OK(hipEventRecord(e[0], s));
+        for (int k = 0; k < nparts; k++) {
+            fns[k](args ? args[k] : nullptr);
+            HIP_OK(hipEventRecord(e[k + 1], s));
+        }
+    }
+    HIP_OK(hipEventSynchronize(ev.back()));
+    for (int k = 0; k < nparts; k++) ms_out[k] = 0.f;
+    for (int it = 0; it < iters; it++)
+        for (int k = 0; k < nparts; k++) {
+            float ms = 0.f;
+            HIP_OK(hipEventElapsedTime(&ms, ev[(size_t)it * (nparts + 1) + k], ev[(size_t)it * (nparts + 1) + k + 1]));
+            ms_out[k] += ms;
+        }
+    for (auto& e : ev) HIP_OK(hipEventDestroy(e));
+    return 0;
+}
 static void run_plan_cb(void* p) { fortis_plan_run((fortis_plan*)p); }
 float fortis_plan_time_ms(fortis_plan* p, int iters, int use_graph)
 {

@@ -238,6 +238,10 @@ int  fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t
 /* Runs fn(arg) `iters` times on the persistent stream between two HIP events on that stream and
  * returns the elapsed milliseconds (the benchmark's per-kernel clock). */
 float fortis_time_ms(void (*fn)(void*), void* arg, int iters);
+/* A step made of `nparts` (at most 16) enqueues fns[k](args[k]), run `iters` (at most 4096) times with a
+ * HIP event between the parts and no host wait inside: ms_out[k] receives the elapsed milliseconds of
+ * part k summed over the iterations.  Returns -1 on bad arguments. */
+int   fortis_time_parts_ms(int nparts, void (*const* fns)(void*), void* const* args, int iters, float* ms_out);
 /* Same clock around `iters` enqueues of a plan (use_graph: captured once, then replayed) and of
  * the fused stencil step. */
 float fortis_plan_time_ms(fortis_plan* p, int iters, int use_graph);
