@@ -37,7 +37,7 @@ struct ConvMShape {
     int tiles_x;               // TILE2D: tiles along x
     int mode;                  // 0: convolution, 1: 2x2 stride-2 transposed conv scatter
     int ksplit;                // channel chunks are split over blockIdx.z; > 1: raw partial sums go to `part`
-    int cb[17];                // slice k takes chunks cb[k] .. cb[k+1]-1 (larger slices first: they are dispatched first)
+    int cbase, cextra;         // slice k takes cbase chunks, the first cextra slices one more (larger slices first: they are dispatched first)
     float* part;               // [ksplit][output elements]
     int ups;                   // 1: the input tensor is (D/2, H/2, W/2) and is read through a nearest x2 upsample
     long osize;                // output elements
@@ -54,18 +54,24 @@ __device__ __forceinline__ void cm_lds_barrier()
 }
 
 #define CM_TP 34       // TILE2D: pitch of a staged row (32 columns + border)
-template <int KD, int KS, int MT, int FT, int NX, bool TILE2D>
+// KG > 1: the workgroup's waves also divide the input channels of every chunk among KG groups; each group
+// accumulates the same output tile over its channels and the groups' sums are added through LDS at the end, in
+// group order.  This is how a launch with few output tiles (deep, small images) still puts four waves on every
+// CU without partial sums in HBM and a second kernel: the tile shrinks to 32 x 32 and KG = 4.
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1>
 __global__ __launch_bounds__(CM_THREADS) __attribute__((amdgpu_waves_per_eu(KD == 3 && MT == 128 && FT == 64 && NX <= 8 ? 4 : 1)))
 void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
 {
     constexpr int T = KD * KS * KS;
-    constexpr int CC = cm_cc(T), NCP = CC / 2;       // NX: staging rounds of the input run (8 or 16)
+    constexpr int CC = cm_cc(T) * KG, NCP = CC / 2;  // NX: staging rounds of the input run (8 or 16)
+    constexpr int NCPW = NCP / KG;                               // channel pairs of a chunk per channel group
     constexpr int WCH = NCP * T * 2 * FT;                        // floats of packed weights per chunk
     constexpr int NW = (WCH / 4 + CM_THREADS - 1) / CM_THREADS;  // float4 per thread
     constexpr int FW = FT / 32;                                  // waves along the channels
-    constexpr int NMT = MT / 32 / (4 / FW);                      // m-tiles per wave
+    constexpr int NMT = MT / 32 / (4 / (FW * KG));               // m-tiles per wave
     static_assert(NMT >= 1, "tile too small for the wave layout");
+    static_assert(KG == 1 || NMT == 1, "channel groups: one m-tile per wave");
     constexpr int PADK = KS / 2;
     constexpr int TH = MT / 32, R2 = (TH + 2) * CM_TP;           // TILE2D: rows per tile, staged elements per channel
     static_assert(!TILE2D || (KD == 1 && KS == 3), "the 2-D tiling is for 3 x 3 convs");
@@ -159,23 +165,25 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
             if (i * CM_THREADS + el0 < XCHP) xdst[i * CM_THREADS] = gchk[i] < lim ? r.rx[i] : 0.f;
     };
 
-    const int ft = wave % FW, mt0 = (wave / FW) * NMT;
-    const int wbase = (lane >> 5) * FT + ft * 32 + (lane & 31);
+    const int kgi = wave % KG, wtile = wave / KG;                 // channel group; the wave's tile among the workgroup's
+    const int ft = wtile % FW, mt0 = (wtile / FW) * NMT;
+    const int wbase = (lane >> 5) * FT + ft * 32 + (lane & 31) + kgi * NCPW * T * 2 * FT;
     // lane's element for tap (0, 0) of its first m-tile; an m-tile is 32 consecutive positions of the run, or
     // (TILE2D) one row of the tile
-    const int xbase = (lane >> 5) * KD * RR + mt0 * (TILE2D ? CM_TP : 32) + (lane & 31);
+    const int xbase = (lane >> 5) * KD * RR + mt0 * (TILE2D ? CM_TP : 32) + (lane & 31) + 2 * kgi * NCPW * KD * RR;
     v16f acc[NMT];
 #pragma unroll
     for (int j = 0; j < NMT; j++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
-    const int ch0 = s.cb[blockIdx.z], ch1 = s.cb[blockIdx.z + 1];
+    const int kz = blockIdx.z;
+    const int ch0 = kz * s.cbase + (kz < s.cextra ? kz : s.cextra), ch1 = ch0 + s.cbase + (kz < s.cextra ? 1 : 0);
     auto multiply = [&](int buf) {
         const float* w = sW + buf * WCH + wbase;
         const float* xs = sX + buf * XCHP + xbase;
 #pragma unroll
-        for (int cp = 0; cp < NCP; cp++)
+        for (int cp = 0; cp < NCPW; cp++)
 #pragma unroll
             for (int kd = 0; kd < KD; kd++)
 #pragma unroll
@@ -226,36 +234,52 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 
     // epilogue: a lane holds one position and 16 output channels per m-tile
     const long ospatial = s.mode ? 4 * chan : chan;
-#pragma unroll
-    for (int j = 0; j < NMT; j++) {
+    auto finish = [&](const int j, const int r, float v) __attribute__((always_inline)) {
         unsigned yy, xx;
         if (TILE2D) {
             yy = (unsigned)(y0 + mt0 + j); xx = (unsigned)(x0 + (lane & 31));
-            if ((int)yy >= s.H) continue;
+            if ((int)yy >= s.H) return;
         } else {
             const int m = m0 + (mt0 + j) * 32 + (lane & 31);
-            if (m >= s.plane) continue;
+            if (m >= s.plane) return;
             st_divmod((unsigned)m, s.mP, yy, xx);
         }
-        if ((int)xx >= s.W) continue;
+        if ((int)xx >= s.W) return;
+        const int f = fg * FT + ft * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (f >= s.F) return;
+        int fo = f;
+        long opos = ((long)z * s.H + yy) * s.W + xx;
+        if (s.mode) {
+            fo = f >> 2;
+            opos = (long)(2 * yy + ((f >> 1) & 1)) * (2 * s.W) + 2 * xx + (f & 1);
+        }
+        if (s.ksplit > 1) { s.part[blockIdx.z * s.osize + fo * ospatial + opos] = v; return; }
+        if (e.scale) v = v * e.scale[fo];
+        if (e.shift) v = v + e.shift[fo];
+        if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
+        else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
+        if (e.res) v = v + e.res[fo * ospatial + opos];
+        y[fo * ospatial + opos] = v;
+    };
+    if constexpr (KG == 1) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int f = fg * FT + ft * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (f >= s.F) continue;
-            int fo = f;
-            long opos = ((long)z * s.H + yy) * s.W + xx;
-            if (s.mode) {
-                fo = f >> 2;
-                opos = (long)(2 * yy + ((f >> 1) & 1)) * (2 * s.W) + 2 * xx + (f & 1);
-            }
-            float v = acc[j][r];
-            if (s.ksplit > 1) { s.part[blockIdx.z * s.osize + fo * ospatial + opos] = v; continue; }
-            if (e.scale) v = v * e.scale[fo];
-            if (e.shift) v = v + e.shift[fo];
-            if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
-            else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
-            if (e.res) v = v + e.res[fo * ospatial + opos];
-            y[fo * ospatial + opos] = v;
+        for (int j = 0; j < NMT; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) finish(j, r, acc[j][r]);
+    } else {
+        // the loop above ended on a barrier: the staging buffers are free.  red[tile][group][register][lane]
+        float* red = (float*)smem4 + wtile * (KG * 16 * 64);
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[(kgi * 16 + r) * 64 + lane] = acc[0][r];
+        cm_lds_barrier();
+        // group g finishes registers g * 16 / KG ...: the groups' sums are added in group order
+#pragma unroll
+        for (int q = 0; q < 16 / KG; q++) {
+            const int r = kgi * (16 / KG) + q;
+            float v = red[r * 64 + lane];
+#pragma unroll
+            for (int g = 1; g < KG; g++) v += red[(g * 16 + r) * 64 + lane];
+            finish(0, r, v);
         }
     }
 }
@@ -400,16 +424,30 @@ int fortis_launch_conv_split_reduce(const float* part, float* y, long osize, lon
     return 0;
 }
 
+// Channel groups inside a workgroup (the kernel's KG) for a conv on images: 4 when tiles of 64 positions x 64
+// channels would leave CUs without a workgroup (the launch would otherwise be split over the input channels into
+// partial sums and a reduce kernel), 1 otherwise.  Fg: output channels of the GEMM (4 F for the transposed conv).
+// Weights are packed for the answer, so packing and launching ask with the same arguments.
+int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, int KS)
+{
+    static const int off = getenv("FORTIS_CONV_KGROUPS") != nullptr && atoi(getenv("FORTIS_CONV_KGROUPS")) == 0;
+    if (off || KD != 1 || D != 1 || C < 32) return 1;
+    if (KS == 3 && !(Wd >= 32 && cdiv(Wd, 32) * 32 * 4 <= 5L * Wd)) return 1;     // 3 x 3: the 32-column tiling only
+    if (KS != 1 && KS != 3) return 1;
+    const long pos = KS == 3 ? H * (Wd + 1) : H * Wd;
+    return cdiv(pos, 64) * cdiv(Fg, 64) < conv_cus() ? 4 : 1;
+}
+
 // Packs conv weights W[F][C][T] (T taps, row-major) into the kernel's order
-//   [F/FT][ceil(C/CC)][channel pair CC/2][tap T][half 2][FT channels], zero padded; CC = cm_cc(T)
-//   channels per chunk; FT = 32 when the GEMM has at most 32 output channels, else 64 (the launcher
-//   applies the same rules).
+//   [F/FT][ceil(C/CC)][channel pair CC/2][tap T][half 2][FT channels], zero padded; CC = cm_cc(T) * kg
+//   channels per chunk; FT = 32 when the GEMM has at most 32 output channels or kg > 1, else 64 (the launcher
+//   applies the same rules; kg = fortis_conv_mfma_kgroups of the shape).
 // Transposed 2x2 conv: W is [C][F][2][2]; GEMM channel f' = f*4 + a*2 + b.
-float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats)
+float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats, int kg)
 {
     const long Fg = transposed ? 4 * F : F;
-    const long FT = conv_ft(Fg);
-    const long CC = cm_cc(T), NCP = CC / 2;
+    const long FT = kg == 4 ? 32 : conv_ft(Fg);
+    const long CC = cm_cc(T) * kg, NCP = CC / 2;
     const long nfg = cdiv(Fg, FT), nch = cdiv(C, CC);
     const long wch = NCP * T * 2 * FT;
     const long n = nfg * nch * wch;
@@ -458,11 +496,11 @@ __global__ void conv_pack_kernel(const float* __restrict__ W, float* __restrict_
     P[idx] = (f < F && c < C) ? W[(f * C + c) * T + t] : 0.f;
 }
 
-const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, hipStream_t st)
+const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, hipStream_t st, int kg)
 {
     static float* buf = nullptr;
     static size_t cap = 0;
-    const long FT = conv_ft(F), CC = cm_cc(T);
+    const long FT = kg == 4 ? 32 : conv_ft(F), CC = cm_cc(T) * kg;
     const long nch = cdiv(C, CC), n = cdiv(F, FT) * nch * (CC / 2) * T * 2 * FT;
     if (g_ws) {
         float* w = ws_take(0, (size_t)n * sizeof(float));
@@ -483,11 +521,11 @@ const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, h
     return buf;
 }
 
-template <int KD, int KS, int MT, int FT, int NX, bool TILE2D>
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1>
 static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {
     constexpr int T = KD * KS * KS;
-    constexpr int CC = cm_cc(T);
+    constexpr int CC = cm_cc(T) * KG;
     s.tiles = (int)cdiv(s.plane, MT);
     s.R = MT + (KS == 3 ? 2 * s.P + 2 : 0);
     if (TILE2D) {
@@ -496,28 +534,28 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
         s.R = (MT / 32 + 2) * CM_TP;
     }
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
-    const size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, 64) * 64) * sizeof(float);
+    size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, 64) * 64) * sizeof(float);
+    if (KG > 1 && shmem < 4 * 16 * 64 * sizeof(float)) shmem = 4 * 16 * 64 * sizeof(float);   // the groups' sums meet in LDS
     if (shmem > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
-        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         attr = shmem;
     }
     // A launch that leaves most CUs idle (deep, small images) is split over the input channels: each
     // split writes raw partial sums, a second kernel adds them in order and applies the epilogue.
     const long wgs = (long)s.D * s.tiles * cdiv(s.F, FT);
     s.ksplit = 1;
-    s.cb[0] = 0; s.cb[1] = s.nchunks;
-    if (2 * wgs < 3 * conv_cus() && s.C >= 32) {
+    s.cbase = s.nchunks; s.cextra = 0;
+    if (KG == 1 && 2 * wgs < 3 * conv_cus() && s.C >= 32) {
         // volumes aim at three workgroups per CU (their chunks are long: 27 taps), images at one (measured on the
         // UNet levels: a finer split costs more in partial sums than it gains in occupancy)
         long k = cdiv((KD == 3 ? 3L : 1L) * conv_cus(), wgs);
         if (k > s.C / 16) k = s.C / 16;               // at least 16 input channels per split
         if (k > 16) k = 16;
         // slices in chunks, the remainder spread over the first ones: the larger slices are dispatched first
-        const int base = (int)(s.nchunks / k), extra = (int)(s.nchunks % k);
         s.ksplit = (int)k;
-        for (int i = 0; i < s.ksplit; i++) s.cb[i + 1] = s.cb[i] + base + (i < extra ? 1 : 0);
+        s.cbase = (int)(s.nchunks / k); s.cextra = (int)(s.nchunks % k);
     }
     const long ospatial = (long)s.D * s.H * s.W * (s.mode ? 4 : 1);
     s.osize = (long)(s.mode ? s.F / 4 : s.F) * ospatial;
@@ -529,7 +567,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     const bool pooled = e.pool != nullptr;
     if (pooled && (s.mode || s.D != 1 || (s.H & 1) || (s.W & 1) || (((uintptr_t)y | (uintptr_t)s.part) & 7))) return -1;   // the plan only asks for it on 2-D convs
     dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);
-    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
     HIP_OK(hipGetLastError());
     if (s.ksplit > 1 && pooled) {
         const long n = (long)s.F * (s.H / 2) * (s.W / 2);
@@ -600,6 +638,17 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
     s.ksplit = 1;
     s.ups = kind == 2 ? 1 : 0;
     if (kind == 2 && ((D | H | Wd) & 1)) return -1;
+    if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 4) {
+        // one 32 x 32 output tile per workgroup, the four waves share its input channels
+        s.P = KS == 3 ? s.W + 1 : s.W;
+        s.plane = s.H * s.P;
+        s.nchunks = (int)cdiv(s.C, cm_cc(KS * KS) * 4);
+        if (KS == 3) {
+            constexpr int NX2 = (cm_cc(9) * 4 * (32 / 32 + 2) * CM_TP + CM_THREADS - 1) / CM_THREADS;
+            return launch_nx<1, 3, 32, 32, NX2, true, 4>(x, wp, y, s, e, st);
+        }
+        return launch_nx<1, 1, 32, 32, cm_cc(1) * 4 * 32 / CM_THREADS, false, 4>(x, wp, y, s, e, st);
+    }
     const bool thin = conv_ft(s.F) == 32;
     if (kind == 1) {
         if (D != 1) return -1;

@@ -467,7 +467,8 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                 else if (o.kind == OP_CONV3D) { ok = o.KD == 3 && o.pad == 1; T = 27; }
                 else { ok = o.KH == 2 && o.KW == 2 && o.stride == 2 && o.pad == 0 && o.opad == 0; T = 1; tr = 1; }
                 if (ok && wide && !direct_only) {
-                    float* wp = fortis_conv_mfma_pack(o.w.data(), o.F, o.C, T, tr, nullptr);
+                    const int kg = o.kind == OP_CONV3D ? 1 : fortis_conv_mfma_kgroups(o.C, 1, o.H, o.W, tr ? 4 * o.F : o.F, 1, tr ? 1 : (int)o.KH);
+                    float* wp = fortis_conv_mfma_pack(o.w.data(), o.F, o.C, T, tr, nullptr, kg);
                     if (!wp) p->upload_failed = true; else p->owned.push_back(wp);
                     ex.Wmfma = wp;
                 }

@@ -151,7 +151,7 @@ static int conv_entry_mfma(const float* x, const float* w, float* y, long C, lon
     if (direct_only < 0) direct_only = getenv("FORTIS_CONV_DIRECT") != nullptr;
     if (direct_only || !(F >= 16 || (KD == 1 && KS == 1))) return -1;
     hipStream_t s = fortis_stream_get();
-    const float* wp = fortis_conv_mfma_pack_dev(w, F, C, (int)(KD * KS * KS), s);
+    const float* wp = fortis_conv_mfma_pack_dev(w, F, C, (int)(KD * KS * KS), s, fortis_conv_mfma_kgroups(C, D, H, Wd, F, (int)KD, (int)KS));
     if (!wp) return -1;
     ConvEpi e = { nullptr, nullptr, FORTIS_ACT_NONE, 0.f, nullptr };
     return fortis_launch_conv_mfma(x, wp, y, C, D, H, Wd, F, (int)KD, (int)KS, 0, e, s);

@@ -24,7 +24,12 @@ pytestmark = pytest.mark.gpu
                                                     (50, 33, 47, 40, 1, 1, 0), (130, 12, 12, 70, 3, 1, 1),
                                                     # the 32-column tiling of wide images: ragged height, widths of one tile, of
                                                     # whole tiles and with a mostly filled last tile, both channel-group widths
-                                                    (9, 45, 32, 24, 3, 1, 1), (16, 37, 96, 64, 3, 1, 1), (5, 130, 124, 33, 3, 1, 1)])
+                                                    (9, 45, 32, 24, 3, 1, 1), (16, 37, 96, 64, 3, 1, 1), (5, 130, 124, 33, 3, 1, 1),
+                                                    # few output tiles and at least 32 input channels: 32 x 32 tiles whose four waves
+                                                    # share the input channels (sums meet in LDS); partial last chunk of 16 (3 x 3) and
+                                                    # of 64 (1 x 1) channels, partial channel group, ragged height, a single tile
+                                                    (40, 33, 64, 72, 3, 1, 1), (96, 20, 60, 32, 3, 1, 1), (32, 32, 32, 256, 3, 1, 1),
+                                                    (100, 16, 16, 48, 1, 1, 0), (64, 1, 32, 32, 1, 1, 0)])
 def test_conv2d_bias_act_vs_oracle(L, gpu, C_, H, W, F, k, stride, pad):
     rng = np.random.default_rng(0)
     x = rng.standard_normal((C_, H, W)).astype(np.float32)
@@ -37,6 +42,24 @@ def test_conv2d_bias_act_vs_oracle(L, gpu, C_, H, W, F, k, stride, pad):
     p.conv2d(t0, t1, w, b, C_, H, W, stride, pad, "leaky", 0.1)
     p.finalize(t0, t1)
     assert maxrel(p.forward(x, ref.shape), ref) < TOL
+    p.close()
+
+
+def test_convt2d_channel_groups_vs_oracle(L, gpu):
+    """2 x 2 stride-2 transposed conv on a small, deep image (the UNet's first up-convolution in small): the kernel form
+    whose waves share the input channels, with bias and ReLU, written into a channel range of a wider tensor."""
+    rng = np.random.default_rng(4)
+    C_, H, W, F = 72, 12, 20, 24
+    x = rng.standard_normal((C_, H, W)).astype(np.float32)
+    w = (rng.standard_normal((C_, F, 2, 2)) / np.sqrt(C_)).astype(np.float32)
+    b = rng.standard_normal(F).astype(np.float32)
+    ref = np.maximum(O.convt2d(x, w, 2, 0) + b[:, None, None], 0)
+    p = P.Plan()
+    t0, t1 = p.tensor(x.size), p.tensor(2 * ref.size)
+    p.convt2d(t0, t1, w, b, C_, H, W, 2, 0, 0, "relu", 0.0, coff=F, ctot=2 * F)
+    p.finalize(t0, t1)
+    got = p.forward(x, (2 * F, 2 * H, 2 * W))
+    assert maxrel(got[F:], ref) < TOL
     p.close()
 
 
@@ -230,6 +253,16 @@ def test_memref_conv_entries_wide_shapes(L, gpu):
         L.fortis_h2d(dw.ptr, w2.ctypes.data, w2.nbytes)
         L.fortis_conv2d(*_memref(dx, x.shape), *_memref(dw, w.shape), *_memref(dy, ref.shape), *args)
         assert maxrel(dy.get(ref.shape), O.conv2d(x, w2, (1, 1), (k // 2, k // 2))) < TOL
+        for d in (dx, dw, dy):
+            d.free()
+    # few output tiles, 40 input channels: the form whose waves share the input channels, weights packed for it per call
+    x = rng.standard_normal((1, 40, 20, 64)).astype(np.float32)
+    for k in (3, 1):
+        w = (rng.standard_normal((48, 40, k, k)) / np.sqrt(40 * k * k)).astype(np.float32)
+        ref = O.conv2d(x, w, (1, 1), (k // 2, k // 2))
+        dx, dw, dy = DevBuf(L, x), DevBuf(L, w), DevBuf(L, nbytes=ref.nbytes)
+        L.fortis_conv2d(*_memref(dx, x.shape), *_memref(dw, w.shape), *_memref(dy, ref.shape), 1, 40, 20, 64, 48, k, k, 20, 64, 1, 1, k // 2, k // 2)
+        assert maxrel(dy.get(ref.shape), ref) < TOL
         for d in (dx, dw, dy):
             d.free()
     x3 = rng.standard_normal((1, 10, 9, 14, 11)).astype(np.float32)
