@@ -302,15 +302,63 @@ __device__ __forceinline__ void layer_narrow(v4f (&a)[4], const LayerRegs& R, co
 #undef FORTIS_LF
 }
 
-// All layers of a narrow network on the operand in a[]; the result is left in a[].
+// A last layer of at most four outputs as v_mfma_f32_4x4x1 products (a quarter of the matrix time of a 16-wide
+// n-tile that is mostly padding): a block of four lanes is four rows of one quarter q, lane i of it brings output
+// i's weight for the feature those rows bring, and every lane ends up with its row's four outputs summed over the 16
+// features per k group that its quarter carries (quarter 0 starts at the bias).  The quarters' sums are still to
+// be added: last_x4_sum does it across the lanes, (q0 + q2) + (q1 + q3), and applies the activation.
 template <bool WLDS>
-__device__ __forceinline__ void layers_narrow(v4f (&a)[4], const ChainDesc& d, int nlayers, const float* sWts, const gfloat* wall, int lane, int lq)
+__device__ __forceinline__ v4f last_x4_partial(const v4f (&a)[4], const LayerRegs& R, int x4off, const float* sWts, const gfloat* wall,
+                                               int lane, int lq)
 {
-    for (int l = 0; l < nlayers; l++) {
+    const int wo = x4off / 4 + (lq * 4 + (lane & 3)) * R.KG;
+    v4f acc;
+    if (WLDS) acc = ((const v4f*)sWts)[R.boff / 4]; else acc = ((const gv4f*)wall)[R.boff / 4];
+    if (lq) acc = (v4f)(0.f);
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+        if (u < R.KG) {
+            v4f w;
+            if (WLDS) w = ((const v4f*)sWts)[wo + u]; else w = ((const gv4f*)wall)[wo + u];
+            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(w.x, a[u].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(w.y, a[u].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(w.z, a[u].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(w.w, a[u].w, acc, 0, 0, 0);
+        }
+    return acc;
+}
+__device__ __forceinline__ v4f last_x4_sum(v4f acc, const LayerRegs& R)
+{
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        float v = acc[r];
+        v += __shfl_xor(v, 32);
+        v += __shfl_xor(v, 16);
+        acc[r] = apply_act(v, R.act, R.alpha);
+    }
+    return acc;
+}
+
+// All layers of a narrow network on the operand in a[]; the result is left in a[].  XSUM false: a last layer in the
+// 4x4x1 form leaves each quarter's partial sums in a[0] and returns true; the caller adds them, (q0 + q2) + (q1 + q3),
+// and applies the layer's activation.
+template <bool WLDS, bool XSUM = true>
+__device__ __forceinline__ bool layers_narrow(v4f (&a)[4], const ChainDesc& d, int nlayers, const float* sWts, const gfloat* wall, int lane, int lq)
+{
+    const int x4off = st_u(d.x4off);
+    const int nfull = x4off >= 0 ? nlayers - 1 : nlayers;
+    for (int l = 0; l < nfull; l++) {
         asm volatile("" ::: "memory");
         const LayerRegs R = layer_regs(d, l);
         layer_narrow<WLDS>(a, R, sWts, wall, lane, lq);
     }
+    if (x4off >= 0) {
+        asm volatile("" ::: "memory");
+        const LayerRegs R = layer_regs(d, nlayers - 1);
+        const v4f part = last_x4_partial<WLDS>(a, R, x4off, sWts, wall, lane, lq);
+        a[0] = XSUM ? last_x4_sum(part, R) : part;
+    }
+    return x4off >= 0;
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -849,8 +897,19 @@ void chain_stencil_rows_kernel(ChainParams params)
                 const v4f* src = (const v4f*)(sOp + (16 * T + lrow) * CSR_PITCH) + lq;
                 a[0] = src[0]; a[1] = src[4];
                 a[2] = a[3] = (v4f)(0.f);
-                layers_narrow<WLDS>(a, d, nlayers, sWts, wall, lane, lq);
-                if (lq == 0) ((v4f*)sOut)[32 * half + 16 * T + lrow] = a[0];
+                if (layers_narrow<WLDS, false>(a, d, nlayers, sWts, wall, lane, lq)) {
+                    // the quarters' partial sums of the last layer meet in the tile's own operand rows (consumed above)
+                    v4f* tmp = (v4f*)(sOp + 16 * T * CSR_PITCH);
+                    tmp[lq * 16 + lrow] = a[0];
+                    asm volatile("" ::: "memory");
+                    if (lq == 0) {
+                        const LayerRegs R = layer_regs(d, nlayers - 1);
+                        v4f o = (tmp[lrow] + tmp[32 + lrow]) + (tmp[16 + lrow] + tmp[48 + lrow]);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) o[r] = apply_act(o[r], R.act, R.alpha);
+                        ((v4f*)sOut)[32 * half + 16 * T + lrow] = o;
+                    }
+                } else if (lq == 0) ((v4f*)sOut)[32 * half + 16 * T + lrow] = a[0];
             }
             asm volatile("" ::: "memory");
         }
@@ -903,7 +962,22 @@ int fortis_chain_build(ChainDesc* d, int nlayers, const float* const* W, const f
         if (L.Np > wmax) wmax = L.Np;
     }
     total = cdiv(total, 4) * 4;
+    // A last layer of at most four outputs a second time, for v_mfma_f32_4x4x1: [q][n][k group][4] holds
+    // W[n][16 group + 4 q + s], the 16 features a lane of quarter q carries per k group.
+    const ChainLayer& LL = d->L[nlayers - 1];
+    d->x4off = -1;
+    if (LL.N <= 4 && LL.Kp <= 64) { d->x4off = (int)total; total += 16L * LL.Kp / 16 * 4; }
     float* h = (float*)calloc(total, sizeof(float));
+    if (d->x4off >= 0) {
+        const int KG = LL.Kp / 16;
+        for (int q = 0; q < 4; q++)
+            for (int n = 0; n < LL.N; n++)
+                for (int u = 0; u < KG; u++)
+                    for (int r = 0; r < 4; r++) {
+                        const int k = 16 * u + 4 * q + r;
+                        if (k < LL.K) h[d->x4off + ((q * 4 + n) * KG + u) * 4 + r] = W[nlayers - 1][(long)n * LL.K + k];
+                    }
+    }
     for (int l = 0; l < nlayers; l++) {
         const ChainLayer& L = d->L[l];
         const int KG = L.Kp / 16, NT = L.Np / 16;

@@ -50,6 +50,7 @@ struct ChainDesc {
     const float* out_mul;  // y * out_mul[c] after the last layer, or null
     int mask_tail;         // ReLU on the last mask_tail outputs
     int ld;                // LDS row pitch in floats
+    int x4off;             // last layer with at most 4 outputs: offset of its weights in 4x4x1 order [q][n][Kp/16][4], or -1
 };
 // Packs the layers (W[l] is [N][K] row-major, b[l] may be null) into one device blob and fills the
 // descriptor's shape fields; act/alpha/in_div/out_mul/mask_tail are left to the caller.

@@ -197,9 +197,15 @@ def test_fused_step_masked_cell_list_config2(L, gpu, ncells, lists):
     for kk in range(nz):
         L.fortis_stencil_scatter_dev(C.byref(st), ptrs(sb), C.c_void_p(dY + kk * ncells * 3 * 4), kk)
     L.fortis_sync()
-    assert bits_equal(plan.read(plan.out_tensor, (rows, 3)), Y)
+    # (the one-launch kernel ends the network on 4x4x1 matrix products, the small-batch MLP kernel of the unfused route
+    # on a 16-wide tile: the same sums in another order, equal within the tolerance, not bit for bit)
+    Yu = plan.read(plan.out_tensor, (rows, 3))
+    assert maxrel(Yu, Y) < TOL
+    ref_u = [a.copy() for a in host[:2]] + [np.zeros(n2, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+    for kk in range(nz):
+        O.stencil_scatter(sd, ref_u, Yu[kk * ncells:(kk + 1) * ncells], ncells, kk, cells=scells)
     for q in (3, 4):
-        assert bits_equal(sb[q].get((n3,)), out[q])
+        assert bits_equal(sb[q].get((n3,)), ref_u[q])
     for b in gb + sb:
         b.free()
     plan.close()
