@@ -27,13 +27,13 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # same command (see profiles/), or None where no counter run has been made for the workload.
 MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((1114.1 * 2 + 885.2) * 1024),
-                    "zb_ref": int((1006.5 * 2 + 885.2) * 1024), "zb_1028x1028x15": int((200550.7 * 2 + 193387.2) * 1024),
-                    "zb_ref_1028x1028x15": int((199443.3 * 2 + 196403.0) * 1024), "toy": None,
+                    "zb_ref": int((1005.6 * 2 + 885.2) * 1024), "zb_1028x1028x15": int((197919.5 * 2 + 192150.3) * 1024),
+                    "zb_ref_1028x1028x15": int((196300.7 * 2 + 195918.0) * 1024), "toy": None,
                     "zb_unfused_1028x1028x15": int((242212.5 * 2 + 1658926.8) * 1024),
                     "zb_unfused_1028x1028x15_f64": int((247386.7 * 2 + 1658898.9) * 1024),
                     # conv workloads: every conv, split-reduce and thin-head dispatch of a step summed, divided by the
                     # step's conv operations (18 and 19), like flop_per_launch
-                    "unet": int((1163560.2 * 2 + 727552.0) * 1024 / 7 / 18), "tsrgan": int((3255367.7 * 2 + 5167927.1) * 1024 / 7 / 19)}
+                    "unet": int((1131048.8 * 2 + 523265.4) * 1024 / 7 / 18), "tsrgan": int((3255367.7 * 2 + 5167927.1) * 1024 / 7 / 19)}
 
 
 def omp_threads():
