@@ -817,10 +817,14 @@ void chain_stencil_rows_kernel(ChainParams params)
         st_row(g, in.row < rows ? in.row : 0, i, j, kk);
         const unsigned goff = (unsigned)i * g_si + (unsigned)j * g_sj + (unsigned)kk * g_pl;
         in.soff = o_as_g ? goff : (unsigned)i * o_si + (unsigned)j * o_sj + (unsigned)kk * o_pl;
+        // every array spans less than 2^30 elements (checked by the launcher): a 32-bit byte offset beside a uniform
+        // base pointer, so a load needs no per-lane 64-bit address
+        const unsigned gbyte = goff << 2;
+        typedef __attribute__((address_space(1))) char gchar;
 #pragma unroll
-        for (int q = 0; q < NQ; q++) in.x[q] = st_uptr(st_g(g.refs[q].p))[goff];          // entries past the table's repeat slot 0
+        for (int q = 0; q < NQ; q++) in.x[q] = *(const gfloat*)((const gchar*)st_uptr(st_g(g.refs[q].p)) + gbyte);   // entries past the table's repeat slot 0
 #pragma unroll
-        for (int q = 0; q < NS; q++) in.gS[q] = st_uptr(st_g(g.scal[q].p))[goff];
+        for (int q = 0; q < NS; q++) in.gS[q] = *(const gfloat*)((const gchar*)st_uptr(st_g(g.scal[q].p)) + gbyte);
 #pragma unroll
         for (int q = 0; q < NS; q++) {
             const unsigned ssi = (unsigned)st_u(sc.scal[q].si), ssj = (unsigned)st_u(sc.scal[q].sj), spl = (unsigned)st_u((int)sc.scal[q].plane);
@@ -867,11 +871,12 @@ void chain_stencil_rows_kernel(ChainParams params)
             for (int q = 0; q < NS; q++) cell.S[q] = in.gS[q];
             st_cell_program(g, cell);
             st_chain_apply(g, cell, in.x);
+            // (slots past the network's inputs, which hold a copy of slot 0, are zeroed in the LDS tile below; rows past
+            // the end hold the first cell's values and their results are never stored: no per-slot select here)
+            if (in_div) {
 #pragma unroll
-            for (int q = 0; q < NQ; q++) {
-                float v = (valid && q < K0) ? in.x[q] : 0.f;
-                if (in_div && q < K0) v = __fdiv_rn(v, in_div[q]);
-                in.x[q] = v;
+                for (int q = 0; q < NQ; q++)
+                    if (q < K0) in.x[q] = __fdiv_rn(in.x[q], in_div[q]);
             }
         }
         // ---- two halves of 32 rows: their operands through the LDS tile, two m-tiles through the layers ------
@@ -887,6 +892,7 @@ void chain_stencil_rows_kernel(ChainParams params)
                     for (int r = 0; r < 4; r++) v[r] = 4 * q4 + r < NQ ? in.x[4 * q4 + r] : 0.f;
                     dst[q4] = v;
                 }
+                for (int c = K0; c < NQ; c++) ((float*)dst)[c] = 0.f;
             }
             asm volatile("" ::: "memory");
             // the slot registers are free once the second half is written: the next 64 rows' loads go out here
