@@ -901,8 +901,7 @@ void chain_stencil_rows_kernel(ChainParams params)
             for (int T = 0; T < 2; T++) {
                 v4f a[4];
                 const v4f* src = (const v4f*)(sOp + (16 * T + lrow) * CSR_PITCH) + lq;
-                a[0] = src[0]; a[1] = src[4];
-                a[2] = a[3] = (v4f)(0.f);
+                a[0] = src[0]; a[1] = src[4];      // (a[2], a[3]: a layer reads as many k groups as the one before it wrote n-tiles)
                 if (layers_narrow<WLDS, false>(a, d, nlayers, sWts, wall, lane, lq)) {
                     // the quarters' partial sums of the last layer meet in the tile's own operand rows (consumed above)
                     v4f* tmp = (v4f*)(sOp + 16 * T * CSR_PITCH);
