@@ -9,7 +9,7 @@ import pytest
 
 from fortis_amd import configs, plan as P, stencil as S, step as ST
 from oracle import oracle as O
-from util import TOL, bits_equal, maxrel
+from util import TOL, DevBuf, bits_equal, maxrel
 
 pytestmark = pytest.mark.gpu
 
@@ -413,3 +413,27 @@ def test_scatter_reuse_is_verified_against_the_host_arrays(L, gpu, golden):
     Txx = results["reuse"][0].reshape(15, 78, 68)
     assert maxrel(Txx[7], G["Txx"][1]) < TOL                       # layer 8 untouched
     assert np.abs(Txx[6]).max() > 0
+
+
+def test_measurement_aids(L, gpu):
+    """fortis_time_parts_ms clocks the parts of a step in order (every part ran once per iteration, every time is
+    positive, bad arguments are refused); fortis_probe_issue_ms returns three positive times and, on this part,
+    matrix and vector waves together take about as long as the two alone (0.8 .. 1.25 of the sum)."""
+    n = 1 << 20
+    a, b, c = DevBuf(L, np.arange(n, dtype=np.float32)), DevBuf(L, nbytes=4 * n), DevBuf(L, nbytes=4 * n)
+    calls = []
+    CB = C.CFUNCTYPE(None, C.c_void_p)
+    f1 = CB(lambda _: (calls.append(1), L.fortis_d2d(b.ptr, a.ptr, 4 * n)))
+    f2 = CB(lambda _: (calls.append(2), L.fortis_d2d(c.ptr, b.ptr, 4 * n)))
+    ms = (C.c_float * 2)()
+    assert L.fortis_time_parts_ms(2, (CB * 2)(f1, f2), None, 3, ms) == 0
+    assert calls == [1, 2] * 3 and ms[0] > 0 and ms[1] > 0
+    assert np.array_equal(c.get((n,)), np.arange(n, dtype=np.float32))
+    assert L.fortis_time_parts_ms(0, (CB * 2)(f1, f2), None, 3, ms) == -1
+    assert L.fortis_time_parts_ms(2, (CB * 2)(f1, f2), None, 0, ms) == -1
+    for d in (a, b, c):
+        d.free()
+    t = (C.c_float * 3)()
+    assert L.fortis_probe_issue_ms(2000, 0, 0, t) == 0
+    assert min(t) > 0 and 0.8 < t[2] / (t[0] + t[1]) < 1.25
+    assert L.fortis_probe_issue_ms(0, 0, 0, t) == -1
