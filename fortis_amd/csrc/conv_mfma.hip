@@ -58,7 +58,7 @@ __device__ __forceinline__ void cm_lds_barrier()
 // accumulates the same output tile over its channels and the groups' sums are added through LDS at the end, in
 // group order.  This is how a launch with few output tiles (deep, small images) still puts four waves on every
 // CU without partial sums in HBM and a second kernel: the tile shrinks to 32 x 32 and KG = 4.
-template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1>
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1, bool POOL = false>
 __global__ __launch_bounds__(CM_THREADS) __attribute__((amdgpu_waves_per_eu(KD == 3 && MT == 128 && FT == 64 && NX <= 8 ? 4 : 1)))
 void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
@@ -260,12 +260,34 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
         if (e.res) v = v + e.res[fo * ospatial + opos];
         y[fo * ospatial + opos] = v;
+        if constexpr (POOL) {
+            // the finished tile also goes to LDS as [channel][row][32 columns] for the 2 x 2 max pool below
+            ((float*)smem4)[((f - fg * FT) * TH + (mt0 + j)) * 32 + (lane & 31)] = v;
+        }
     };
     if constexpr (KG == 1) {
 #pragma unroll
         for (int j = 0; j < NMT; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) finish(j, r, acc[j][r]);
+        if constexpr (POOL) {
+            // 2 x 2 stride-2 max pool of the tile (H and W even, tiles start on even rows and columns: a 2 x 2 block
+            // lies inside the image or outside it as a whole); the loop above ended the staging, LDS is free
+            static_assert(TILE2D && KG == 1 && (MT / 32) % 2 == 0, "the in-kernel pool needs the 32-column tiling and an even tile height");
+            {
+                cm_lds_barrier();
+                const float* pt = (const float*)smem4;
+                const int Ho = s.H >> 1, Wo = s.W >> 1;
+                for (int idx = tid; idx < FT * (TH / 2) * 16; idx += CM_THREADS) {
+                    const int pc = idx & 15, pr = (idx >> 4) % (TH / 2), fl = idx / (16 * (TH / 2));
+                    const int f = fg * FT + fl, yo = (y0 >> 1) + pr, xo = (x0 >> 1) + pc;
+                    if (f >= s.F || yo >= Ho || xo >= Wo) continue;
+                    const float* q = pt + (fl * TH + 2 * pr) * 32 + 2 * pc;
+                    const float m0 = q[0] > q[1] ? q[0] : q[1], m1 = q[32] > q[33] ? q[32] : q[33];
+                    e.pool[((long)f * Ho + yo) * Wo + xo] = m0 > m1 ? m0 : m1;
+                }
+            }
+        }
     } else {
         // the loop above ended on a barrier: the staging buffers are free.  red[tile][group][register][lane]
         float* red = (float*)smem4 + wtile * (KG * 16 * 64);
@@ -521,7 +543,7 @@ const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, h
     return buf;
 }
 
-template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1>
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1, bool POOL = false>
 static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {
     constexpr int T = KD * KS * KS;
@@ -536,10 +558,11 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
     size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, 64) * 64) * sizeof(float);
     if (KG > 1 && shmem < 4 * 16 * 64 * sizeof(float)) shmem = 4 * 16 * 64 * sizeof(float);   // the groups' sums meet in LDS
+    if (POOL && shmem < (size_t)FT * MT * sizeof(float)) shmem = (size_t)FT * MT * sizeof(float);   // the finished tile, for its 2 x 2 max pool
     if (shmem > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
-        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         attr = shmem;
     }
     // A launch that leaves most CUs idle (deep, small images) is split over the input channels: each
@@ -547,7 +570,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     const long wgs = (long)s.D * s.tiles * cdiv(s.F, FT);
     s.ksplit = 1;
     s.cbase = s.nchunks; s.cextra = 0;
-    if (KG == 1 && 2 * wgs < 3 * conv_cus() && s.C >= 32) {
+    if (KG == 1 && !POOL && 2 * wgs < 3 * conv_cus() && s.C >= 32) {
         // volumes aim at three workgroups per CU (their chunks are long: 27 taps), images at one (measured on the
         // UNet levels: a finer split costs more in partial sums than it gains in occupancy)
         long k = cdiv((KD == 3 ? 3L : 1L) * conv_cus(), wgs);
@@ -567,7 +590,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     const bool pooled = e.pool != nullptr;
     if (pooled && (s.mode || s.D != 1 || (s.H & 1) || (s.W & 1) || (((uintptr_t)y | (uintptr_t)s.part) & 7))) return -1;   // the plan only asks for it on 2-D convs
     dim3 grid((unsigned)(s.D * s.tiles), (unsigned)cdiv(s.F, FT), (unsigned)s.ksplit);
-    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL>), grid, dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
     HIP_OK(hipGetLastError());
     if (s.ksplit > 1 && pooled) {
         const long n = (long)s.F * (s.H / 2) * (s.W / 2);
@@ -577,7 +600,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     } else if (s.ksplit > 1) {
         launch_split_reduce(s.part, y, s.osize, ospatial, s.ksplit, e, st);
         HIP_OK(hipGetLastError());
-    } else if (pooled) {
+    } else if (pooled && !POOL) {
         fortis_launch_maxpool2d(y, e.pool, s.F, s.H, s.W, 2, st);
     }
     return 0;
@@ -592,6 +615,13 @@ static int launch(const float* x, const float* wp, float* y, ConvMShape s, const
         // columns with a one-pixel border; the staging rounds are a compile-time count
         if (s.W >= 32 && cdiv(s.W, 32) * 32 * 4 <= 5L * s.W && getenv("FORTIS_CONV_LINEAR") == nullptr) {
             constexpr int NX2 = (cm_cc(9) * (MT / 32 + 2) * CM_TP + CM_THREADS - 1) / CM_THREADS;
+            // a conv with a 2 x 2 max pool behind it pools its own tiles (even tile height) unless the launch is one
+            // that gets split over its input channels, whose reduce kernel pools
+            if constexpr ((MT / 32) % 2 == 0) {
+                const long wgs = cdiv(s.W, 32) * cdiv(s.H, MT / 32) * cdiv(s.F, FT);
+                if (e.pool && !s.mode && !(s.H & 1) && !(s.W & 1) && (wgs >= conv_cus() || s.C < 32))
+                    return launch_nx<1, 3, MT, FT, NX2, true, 1, true>(x, wp, y, s, e, st);
+            }
             return launch_nx<1, 3, MT, FT, NX2, true>(x, wp, y, s, e, st);
         }
     }

@@ -45,6 +45,29 @@ def test_conv2d_bias_act_vs_oracle(L, gpu, C_, H, W, F, k, stride, pad):
     p.close()
 
 
+@pytest.mark.parametrize("C_,H,W,F", [(16, 38, 64, 24), (8, 130, 96, 40), (48, 12, 32, 64)])
+def test_conv2d_with_max_pool_behind(L, gpu, C_, H, W, F):
+    """3 x 3 conv + bias + ReLU followed by a 2 x 2 max pool: the conv pools its own tiles (32-column tiling, even tile
+    height; ragged last tile rows), or its channel-split reduce kernel does (the small, deep case).  Both outputs checked."""
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((C_, H, W)).astype(np.float32)
+    w = (rng.standard_normal((F, C_, 3, 3)) / np.sqrt(C_ * 9)).astype(np.float32)
+    b = rng.standard_normal(F).astype(np.float32)
+    ref = np.maximum(O.conv2d(x[None], w, (1, 1), (1, 1))[0] + b[:, None, None], 0)
+    pooled = ref.reshape(F, H // 2, 2, W // 2, 2).max(axis=(2, 4))
+    p = P.Plan()
+    t0, t1, t2 = p.tensor(x.size), p.tensor(ref.size), p.tensor(pooled.size)
+    p.conv2d(t0, t1, w, b, C_, H, W, 1, 1, "relu", 0.0)
+    p.maxpool2d(t1, t2, F, H, W, 2)
+    p.finalize(t0, t2)
+    got_pool = p.forward(x, pooled.shape)
+    got_full = p.read(t1, ref.shape)
+    assert maxrel(got_full, ref) < TOL
+    # the pool of the kernel's own full-resolution output, bit for bit
+    assert np.array_equal(got_pool, got_full.reshape(F, H // 2, 2, W // 2, 2).max(axis=(2, 4)))
+    p.close()
+
+
 def test_convt2d_channel_groups_vs_oracle(L, gpu):
     """2 x 2 stride-2 transposed conv on a small, deep image (the UNet's first up-convolution in small): the kernel form
     whose waves share the input channels, with bias and ReLU, written into a channel range of a wider tensor."""
