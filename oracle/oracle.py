@@ -293,7 +293,7 @@ def stencil_gather_typed(desc, arrays, count, nk, ilo=0, jlo=0, ni=1, cells=None
             tv = arrays[sl["array"]][_elem_index(desc["arrays"], sl, i, j, kk)].astype(np.float32)   # float tv = A[...]
             for e in desc["exprs"]:
                 env["tv"] = tv
-                tv = np.asarray(c_eval(e, env)).astype(np.float32) + np.zeros_like(tv)                 # tv = <expr>;
+                tv = np.broadcast_to(np.asarray(c_eval(e, env)).astype(np.float32), tv.shape).copy()   # tv = <expr>; (no arithmetic here: x + 0 would turn -0 into +0)
             X[kk * count:(kk + 1) * count, q] = tv
     return X
 
@@ -306,7 +306,7 @@ def stencil_scatter_typed(desc, arrays, Y, count, kk, ilo=0, jlo=0, ni=1, cells=
     for e in desc["exprs"]:
         for q in range(desc["n"]):
             env["tv"] = yv[q]
-            yv[q] = np.asarray(c_eval(e, env)).astype(np.float32) + np.zeros_like(yv[q])
+            yv[q] = np.broadcast_to(np.asarray(c_eval(e, env)).astype(np.float32), yv[q].shape).copy()
     for st in desc["stores"]:
         a = arrays[st["array"]]
         a[_elem_index(desc["arrays"], st, i, j, kk)] = yv[st["slot"]].astype(a.dtype)

@@ -68,6 +68,64 @@ def test_gather_scatter_other_grids_bit_exact(L, gpu, sx, sy, nz):
         b.free()
 
 
+def test_gather_scatter_expressions_on_special_operands(L, gpu):
+    """tv / (S0 + 1e-30f) in the gather and ((tv * S0) * S0) * S1 in the scatter with zeros of both signs, denormals, the
+    smallest and largest normals, powers of two near the ends of the exponent range, all-ones mantissas, infinities and
+    NaNs among numerators, divisors and factors: IEEE results bit for bit (any NaN equals any NaN), in the fp32 kernels
+    and, with the arrays in double precision, in the general ones."""
+    sx, sy, nz = 40, 30, 2
+    gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    rng = np.random.default_rng(21)
+    tiny, big = np.float32(1.1754944e-38), np.float32(3.4028235e38)
+    ones = np.array([0x3FFFFFFF, 0x007FFFFF, 0x7F7FFFFF, 0x00000001, 0x80000001, 0x00800000], np.uint32).view(np.float32)
+    special = np.concatenate([np.array([0.0, -0.0, 1e-45, -1e-45, 3e-39, tiny, -tiny, 2.0 ** -100, 2.0 ** -64, 2.0 ** -24, 1.0, -1.0, 3.0,
+                                        2.0 ** 64, 2.0 ** 100, 2.0 ** 126, big, -big, np.inf, -np.inf, np.nan], np.float32), ones])
+
+    def field(n, share):
+        a = rng.standard_normal(n).astype(np.float32)
+        pick = rng.random(n) < share
+        a[pick] = rng.choice(special, int(pick.sum()))
+        return a
+    n3 = sx * sy * nz
+    A = {"sh_xy_h": field(n3, 0.3), "sh_xx": field(n3, 0.3), "vort_xy_h": field(n3, 0.3), "norm_h": field(n3, 0.3), "kappa_h": field(sx * sy, 0.3)}
+    count = (sx - 4) * (sy - 4)
+
+    def same(a, b):
+        a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+        return bool(np.all((a.view(np.uint32) == b.view(np.uint32)) | (np.isnan(a) & np.isnan(b))))
+    with np.errstate(all="ignore"):
+        for f64 in (False, True):
+            gdd, sdd = [{**d, "arrays": [dict(a) for a in d["arrays"]]} for d in (gd, sd)]
+            ft = np.float64 if f64 else np.float32
+            if f64:
+                for d in (gdd, sdd):
+                    for a in d["arrays"]:
+                        a["elt"] = "f64"
+            gt, st = S.build_table(gdd, lp, kd, "gather"), S.build_table(sdd, lp, kd, "scatter")
+            garr = [A[k].astype(ft) for k in ("sh_xy_h", "sh_xx", "vort_xy_h", "norm_h")]
+            bufs = [DevBuf(L, a) for a in garr]
+            dX = DevBuf(L, nbytes=count * nz * 27 * 4)
+            L.fortis_stencil_gather_dev(C.byref(gt), ptrs(bufs), dX.ptr)
+            X = dX.get((count * nz, 27))
+            ref = O.stencil_gather_typed(gdd, garr, count, nz, 3, 3, sx - 4) if f64 else O.stencil_gather(gd, garr, count, nz, 3, 3, sx - 4)
+            assert same(X, ref), "gather, f64 arrays: %s" % f64
+            if not f64:
+                Y = field(count * nz * 3, 0.3).reshape(count * nz, 3)
+                host = [A["norm_h"], A["kappa_h"], np.zeros(sx * sy, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+                refs = [a.copy() for a in host]
+                sb = [DevBuf(L, a) for a in host]
+                dY = DevBuf(L, Y)
+                for kk in range(nz):
+                    L.fortis_stencil_scatter_dev(C.byref(st), ptrs(sb), C.c_void_p(dY.ptr + kk * count * 3 * 4), kk)
+                    O.stencil_scatter(sd, refs, Y[kk * count:(kk + 1) * count], count, kk, 3, 3, sx - 4)
+                for b, r in zip(sb[2:], refs[2:]):
+                    assert same(b.get(r.shape), r)
+                for b in sb + [dY]:
+                    b.free()
+            for b in bufs + [dX]:
+                b.free()
+
+
 @pytest.mark.parametrize("ncells", [4736, 2376])
 def test_gather_scatter_masked_cell_list_bit_exact(L, gpu, ncells):
     """480 x 240 grid with a 1-cell halo and a seeded ~30 % land mask; the first 4736 (2376) usable
