@@ -511,6 +511,14 @@ void chain_wave_kernel(ChainParams params)
         for (int l = 0; l < nlayers; l++) {
             asm volatile("" ::: "memory");
             const LayerRegs R = layer_regs(d, l);
+            if constexpr (NTMAX == 4) {
+                // a last layer of at most four outputs in its 4x4x1 form, as in layers_narrow: every form of the
+                // narrow-network kernels then ends the network on the same arithmetic
+                if (l == nlayers - 1 && st_u(d.x4off) >= 0) {
+                    a[0] = last_x4_sum(last_x4_partial<WLDS>(a, R, st_u(d.x4off), sWts, wall, lane, lq), R);
+                    break;
+                }
+            }
             // n-tiles in groups of four independent accumulators; the size of the last group is
             // dispatched once per layer
 #pragma unroll
