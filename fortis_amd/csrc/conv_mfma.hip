@@ -39,6 +39,8 @@ struct ConvMShape {
     int ksplit;                // channel chunks are split over blockIdx.z; > 1: raw partial sums go to `part`
     int cbase, cextra;         // slice k takes cbase chunks, the first cextra slices one more (larger slices first: they are dispatched first)
     float* part;               // [ksplit][output elements]
+    int sk_per, sk_items;      // streamed split: (tile, chunk) items per workgroup and in all (per group of output channels)
+    int sk_tile0;              // streamed split: its first tile (the tiles before it are computed whole by a launch of their own)
     int ups;                   // 1: the input tensor is (D/2, H/2, W/2) and is read through a nearest x2 upsample
     long osize;                // output elements
     StMagic mP, mR, mKR;       // exact division by P, R and KD * R (the staging map would otherwise spend its time dividing)
@@ -58,8 +60,14 @@ __device__ __forceinline__ void cm_lds_barrier()
 // accumulates the same output tile over its channels and the groups' sums are added through LDS at the end, in
 // group order.  This is how a launch with few output tiles (deep, small images) still puts four waves on every
 // CU without partial sums in HBM and a second kernel: the tile shrinks to 32 x 32 and KG = 4.
-template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1, bool POOL = false>
-__global__ __launch_bounds__(CM_THREADS) __attribute__((amdgpu_waves_per_eu(KD == 3 && MT == 128 && FT == 64 && NX <= 8 ? 4 : 1)))
+// SK (streamed split, volumes with fewer tiles than the chip needs): the launch's work is the list of (tile, chunk)
+// items, tile-major; every workgroup takes the same count of consecutive items, whatever tile boundaries fall
+// inside its run, and leaves one partial sum per tile it touched, in its accumulators' own register order
+// (part[slot][tile][register][thread], slot = the workgroup's rank among those that share the tile).
+// conv_sk_reduce_kernel adds a tile's slots in order and applies the epilogue.  Equal runs are what a split into
+// whole slices cannot give: 297 tiles in 3 slices are 891 workgroups, four on some CUs and three on others.
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1, bool POOL = false, bool SK = false>
+__global__ __launch_bounds__(CM_THREADS) __attribute__((amdgpu_waves_per_eu(SK ? 2 : KD == 3 && MT == 128 && FT == 64 && NX <= 8 ? 4 : 1)))
 void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
 {
@@ -85,9 +93,28 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // volumes: neighbouring tiles and planes on one XCD (input fetched once instead of 2-3 times; on images the
     // banded order measured 2 % slower)
-    const int bx = KD == 3 ? (int)fortis_xcd_band(blockIdx.x, gridDim.x) : (int)blockIdx.x;
-    const int z = bx / s.tiles, tile = bx - z * s.tiles;
+    const int wgx = KD == 3 ? (int)fortis_xcd_band(blockIdx.x, gridDim.x) : (int)blockIdx.x;
     const int fg = blockIdx.y;
+    static_assert(!SK || (KG == 1 && !POOL && !TILE2D), "the streamed split is for the plain volume kernel");
+    int it = 0, itend = 0;                                        // SK: the workgroup's run of items
+    if constexpr (SK) {
+        it = wgx * s.sk_per;
+        itend = it + s.sk_per < s.sk_items ? it + s.sk_per : s.sk_items;
+    }
+    for (;;) {                                                    // SK: once per tile of the run; otherwise once
+    int bx = wgx, ch0, ch1;
+    if constexpr (SK) {
+        if (it >= itend) break;
+        bx = it / s.nchunks;
+        ch0 = it - bx * s.nchunks;
+        bx += s.sk_tile0;
+        ch1 = ch0 + (itend - it) < s.nchunks ? ch0 + (itend - it) : s.nchunks;
+    } else {
+        const int kz = blockIdx.z;
+        ch0 = kz * s.cbase + (kz < s.cextra ? kz : s.cextra);
+        ch1 = ch0 + s.cbase + (kz < s.cextra ? 1 : 0);
+    }
+    const int z = bx / s.tiles, tile = bx - z * s.tiles;
     const int m0 = tile * MT;
     const int tyi = TILE2D ? tile / s.tiles_x : 0, y0 = tyi * TH, x0 = (tile - tyi * s.tiles_x) * 32;   // TILE2D: tile origin
     const long HW = (long)s.H * s.W, chan = (long)s.D * HW;
@@ -177,8 +204,6 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
-    const int kz = blockIdx.z;
-    const int ch0 = kz * s.cbase + (kz < s.cextra ? kz : s.cextra), ch1 = ch0 + s.cbase + (kz < s.cextra ? 1 : 0);
     auto multiply = [&](int buf) {
         const float* w = sW + buf * WCH + wbase;
         const float* xs = sX + buf * XCHP + xbase;
@@ -265,7 +290,21 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
             ((float*)smem4)[((f - fg * FT) * TH + (mt0 + j)) * 32 + (lane & 31)] = v;
         }
     };
-    if constexpr (KG == 1) {
+    if constexpr (SK) {
+        // the accumulators as they are: slot = this workgroup's rank among those whose runs share the tile
+        const int tl = bx - s.sk_tile0, slot = wgx - (tl * s.nchunks) / s.sk_per;
+        cm_v4f* pd = (cm_v4f*)s.part + (((long)slot * gridDim.y + fg) * (s.D * s.tiles - s.sk_tile0) + tl) * (NMT * 4 * CM_THREADS) + tid;
+#pragma unroll
+        for (int j = 0; j < NMT; j++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                cm_v4f v;
+                v[0] = acc[j][4 * q]; v[1] = acc[j][4 * q + 1]; v[2] = acc[j][4 * q + 2]; v[3] = acc[j][4 * q + 3];
+                pd[(j * 4 + q) * CM_THREADS] = v;
+            }
+        it += ch1 - ch0;
+        continue;
+    } else if constexpr (KG == 1) {
 #pragma unroll
         for (int j = 0; j < NMT; j++)
 #pragma unroll
@@ -303,6 +342,47 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
             for (int g = 1; g < KG; g++) v += red[(g * 16 + r) * 64 + lane];
             finish(0, r, v);
         }
+    }
+    break;
+    }
+}
+
+// Second kernel of the streamed split: threads as in conv_mfma_kernel (the same registers of the same lanes), a
+// workgroup per tile and group of four accumulator registers (a tile alone would be too few workgroups for a
+// kernel that only moves memory).  A tile's partial sums are added in slot order, i.e. in the order of the input
+// channels.  part[slot][channel group][tile][register quad][thread][4].
+template <int MT, int FT>
+__global__ __launch_bounds__(CM_THREADS) void conv_sk_reduce_kernel(float* __restrict__ y, ConvMShape s, ConvEpi e)
+{
+    constexpr int FW = FT / 32, NMT = MT / 32 / (4 / FW), NQ = NMT * 4;
+    const int tl = blockIdx.x, fg = blockIdx.y, rq = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int first = tl * s.nchunks, w0 = first / s.sk_per, nseg = (first + s.nchunks - 1) / s.sk_per - w0 + 1;
+    const long slot = (long)gridDim.x * gridDim.y * (NQ * CM_THREADS);
+    const cm_v4f* p = (const cm_v4f*)s.part + (((long)fg * gridDim.x + tl) * NQ + rq) * CM_THREADS + tid;
+    cm_v4f acc = *p;
+    for (int k = 1; k < nseg; k++) {
+        p += slot;
+        acc += *p;
+    }
+    const int bx = tl + s.sk_tile0, z = bx / s.tiles, tile = bx - z * s.tiles;
+    const int ft = wave % FW, mt0 = (wave / FW) * NMT;
+    const long ospatial = (long)s.D * s.H * s.W;
+    const int m = tile * MT + (mt0 + rq / 4) * 32 + (lane & 31);
+    unsigned yy, xx;
+    st_divmod((unsigned)m, s.mP, yy, xx);
+    if (m >= s.plane || (int)xx >= s.W) return;
+    const long opos = ((long)z * s.H + yy) * s.W + xx;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int f = fg * FT + ft * 32 + 8 * (rq & 3) + 4 * (lane >> 5) + q;      // register 4 * (rq & 3) + q of the m-tile
+        if (f >= s.F) continue;
+        float v = acc[q];
+        if (e.scale) v = v * e.scale[f];
+        if (e.shift) v = v + e.shift[f];
+        if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
+        else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
+        if (e.res) v = v + e.res[f * ospatial + opos];
+        y[f * ospatial + opos] = v;
     }
 }
 
@@ -563,6 +643,8 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     static size_t attr = 0;
     if (shmem > attr) {
         HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        if constexpr (KD == 3 && KG == 1 && !POOL && !TILE2D)
+            HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         attr = shmem;
     }
     // A launch that leaves most CUs idle (deep, small images) is split over the input channels: each
@@ -582,6 +664,42 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     }
     const long ospatial = (long)s.D * s.H * s.W * (s.mode ? 4 : 1);
     s.osize = (long)(s.mode ? s.F / 4 : s.F) * ospatial;
+    if constexpr (KD == 3 && KG == 1 && !POOL && !TILE2D) {
+        // Volumes whose tiles do not fill the chip evenly.  Fewer tiles than the chip needs (the launch would be split
+        // into whole slices): every tile is streamed, in equal runs of (tile, chunk) items.  More tiles than are
+        // resident at once, with a last round that would leave most CUs idle while its few workgroups finish: the
+        // full rounds run as they are, in a launch of their own, and only the tiles of the last round are streamed.
+        static const int sk_wgs = getenv("FORTIS_CONV_STREAMK") ? atoi(getenv("FORTIS_CONV_STREAMK")) : 2;   // streaming workgroups per CU; 0: off
+        if (!s.mode && !e.pool && sk_wgs > 0 && s.C >= 32) {
+            const long nfg = cdiv(s.F, FT), ntiles = (long)s.D * s.tiles;
+            long tile0 = -1;
+            if (s.ksplit > 1) tile0 = 0;
+            else if (MT == 128 && FT == 64 && NX <= 8) {                 // the form that runs four workgroups per CU
+                const long resident = 4L * conv_cus() / nfg, last = ntiles % resident;
+                if (ntiles > resident && last > 0 && 2 * last < resident) tile0 = ntiles - last;
+            }
+            const long items = tile0 < 0 ? 0 : (ntiles - tile0) * s.nchunks;
+            long per = cdiv(items, std::max(1L, (long)sk_wgs * conv_cus() / nfg));
+            if (per < 8) per = 8;                                         // at least 16 input channels per run
+            if (tile0 >= 0 && per < s.nchunks) {
+                const long slots = (s.nchunks - 2 + per) / per + 1;       // a tile's items meet at most this many runs
+                s.sk_per = (int)per; s.sk_items = (int)items; s.sk_tile0 = (int)tile0;
+                s.ksplit = 1;
+                s.cbase = s.nchunks; s.cextra = 0;
+                s.part = fortis_conv_split_scratch((size_t)slots * nfg * (ntiles - tile0) * MT * FT * sizeof(float));
+                if (!s.part) return -1;
+                if (tile0 > 0) {
+                    hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL>), dim3((unsigned)tile0, (unsigned)nfg, 1), dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+                    HIP_OK(hipGetLastError());
+                }
+                hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL, true>), dim3((unsigned)cdiv(items, per), (unsigned)nfg, 1), dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+                HIP_OK(hipGetLastError());
+                hipLaunchKernelGGL((conv_sk_reduce_kernel<MT, FT>), dim3((unsigned)(ntiles - tile0), (unsigned)nfg, (MT / 32 / (4 / (FT / 32))) * 4), dim3(CM_THREADS), 0, st, y, s, e);
+                HIP_OK(hipGetLastError());
+                return 0;
+            }
+        }
+    }
     if (s.ksplit > 1) {
         s.part = fortis_conv_split_scratch((size_t)s.ksplit * s.osize * sizeof(float));
         if (!s.part) return -1;

@@ -179,7 +179,13 @@ def test_op_micro_suite(L, gpu):
                                                (7, 12, 11, 10, 20, 3, 1), (6, 5, 90, 70, 80, 3, 1),
                                                # image-space heads (at most 4 output channels) whose input channels are split
                                                # over workgroups: even slices, and an odd channel count with a shorter last slice
-                                               (32, 8, 20, 20, 3, 3, 1), (17, 6, 10, 12, 4, 3, 1), (64, 5, 30, 33, 1, 3, 1)])
+                                               (32, 8, 20, 20, 3, 3, 1), (17, 6, 10, 12, 4, 3, 1), (64, 5, 30, 33, 1, 3, 1),
+                                               # streamed split (equal runs of (tile, chunk) items, partial sums per tile and run):
+                                               # two groups of output channels and ragged tiles; an odd chunk count
+                                               (64, 12, 20, 19, 128, 3, 1), (46, 10, 17, 23, 64, 3, 1),
+                                               # more tiles than are resident at once: whole rounds in one launch, the 26 tiles
+                                               # of the last round streamed
+                                               (32, 21, 80, 79, 64, 3, 1)])
 def test_conv3d_bias_act_residual_vs_oracle(L, gpu, C_, D, H, W, F, k, pad):
     rng = np.random.default_rng(1)
     x = rng.standard_normal((C_, D, H, W)).astype(np.float32)
