@@ -42,7 +42,7 @@ def test_noalloc_entry_equals_the_allocating_entry_on_two_calls_in_a_row(L, gpu)
     weights and partial sums in the scratch array: 64 -> 64 channels on small volumes splits its input channels
     over workgroups (partial sums in scratch), and both calls pack their weights into it."""
     rng = np.random.default_rng(21)
-    shapes = [((1, 64, 16, 18, 20), 64), ((1, 64, 9, 10, 11), 64),      # channel-split matrix-core launches
+    shapes = [((1, 64, 16, 18, 20), 64), ((1, 64, 9, 10, 11), 64),      # matrix-core launches with partial sums in scratch
               ((2, 32, 8, 20, 20), 3), ((1, 17, 6, 10, 12), 4),           # thin heads: split on the vector kernel, batch of 2
               ((1, 10, 9, 14, 11), 20)]                                   # no split: only the packed weights use scratch
     for (xs, F) in shapes:
@@ -52,9 +52,10 @@ def test_noalloc_entry_equals_the_allocating_entry_on_two_calls_in_a_row(L, gpu)
 
 
 def test_noalloc_entry_refuses_what_does_not_fit_its_scratch(L, gpu, capfd):
-    """64 -> 64 channels on 27 x 40 x 40 splits three ways: 3 x 11.06 MB of partial sums behind 0.44 MB of
-    packed weights is more than the 32 MiB array.  The call says so, returns -1 and computes nothing; the
-    allocating entry takes the shape, and the next no-alloc call works."""
+    """64 -> 64 channels on 27 x 40 x 40 is streamed over the chip in runs of 22 chunks: up to three partial sums for
+    each of its 351 tiles of 128 positions x 64 channels are 34.5 MB behind 0.44 MB of packed weights, more than the
+    32 MiB array.  The call says so, returns -1 and computes nothing; the allocating entry takes the shape, and the
+    next no-alloc call works."""
     rng = np.random.default_rng(22)
     x = rng.standard_normal((1, 64, 27, 40, 40)).astype(np.float32)
     w = (rng.standard_normal((64, 64, 3, 3, 3)) / np.sqrt(27 * 64)).astype(np.float32)
