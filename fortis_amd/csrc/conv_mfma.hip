@@ -59,7 +59,9 @@ __device__ __forceinline__ void cm_lds_barrier()
 // KG > 1: the workgroup's waves also divide the input channels of every chunk among KG groups; each group
 // accumulates the same output tile over its channels and the groups' sums are added through LDS at the end, in
 // group order.  This is how a launch with few output tiles (deep, small images) still puts four waves on every
-// CU without partial sums in HBM and a second kernel: the tile shrinks to 32 x 32 and KG = 4.
+// CU without partial sums in HBM and a second kernel: the tile shrinks to 32 x 32 and KG = 4.  KG = 2 (64 x 32
+// tiles: two rows of 32 columns, each wave pair halves the channels) is the same trade for launches of one to five
+// 64 x 64 tiles per CU: more, smaller workgroups keep the matrix pipes fed while others stage.
 // SK (streamed split, volumes with fewer tiles than the chip needs): the launch's work is the list of (tile, chunk)
 // items, tile-major; every workgroup takes the same count of consecutive items, whatever tile boundaries fall
 // inside its run, and leaves one partial sum per tile it touched, in its accumulators' own register order
@@ -287,9 +289,28 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         y[fo * ospatial + opos] = v;
         if constexpr (POOL) {
             // the finished tile also goes to LDS as [channel][row][32 columns] for the 2 x 2 max pool below
-            ((float*)smem4)[((f - fg * FT) * TH + (mt0 + j)) * 32 + (lane & 31)] = v;
+            // (behind the channel groups' sums, which other waves may still be reading)
+            ((float*)smem4)[(KG > 1 ? 4 * 16 * 64 : 0) + ((f - fg * FT) * TH + (mt0 + j)) * 32 + (lane & 31)] = v;
         }
     };
+    // 2 x 2 stride-2 max pool of the finished tile (H and W even, tiles start on even rows and columns: a 2 x 2
+    // block lies inside the image or outside it as a whole); staging has ended, LDS is free
+    auto pool_tile = [&]() __attribute__((always_inline)) {
+        if constexpr (POOL) {
+            cm_lds_barrier();
+            const float* pt = (const float*)smem4 + (KG > 1 ? 4 * 16 * 64 : 0);
+            const int Ho = s.H >> 1, Wo = s.W >> 1;
+            for (int idx = tid; idx < FT * (TH / 2) * 16; idx += CM_THREADS) {
+                const int pc = idx & 15, pr = (idx >> 4) % (TH / 2), fl = idx / (16 * (TH / 2));
+                const int f = fg * FT + fl, yo = (y0 >> 1) + pr, xo = (x0 >> 1) + pc;
+                if (f >= s.F || yo >= Ho || xo >= Wo) continue;
+                const float* q = pt + (fl * TH + 2 * pr) * 32 + 2 * pc;
+                const float m0 = q[0] > q[1] ? q[0] : q[1], m1 = q[32] > q[33] ? q[32] : q[33];
+                e.pool[((long)f * Ho + yo) * Wo + xo] = m0 > m1 ? m0 : m1;
+            }
+        }
+    };
+    static_assert(!POOL || (TILE2D && (MT / 32) % 2 == 0), "the in-kernel pool needs the 32-column tiling and an even tile height");
     if constexpr (SK) {
         // the accumulators as they are: slot = this workgroup's rank among those whose runs share the tile
         const int tl = bx - s.sk_tile0, slot = wgx - (tl * s.nchunks) / s.sk_per;
@@ -309,24 +330,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         for (int j = 0; j < NMT; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) finish(j, r, acc[j][r]);
-        if constexpr (POOL) {
-            // 2 x 2 stride-2 max pool of the tile (H and W even, tiles start on even rows and columns: a 2 x 2 block
-            // lies inside the image or outside it as a whole); the loop above ended the staging, LDS is free
-            static_assert(TILE2D && KG == 1 && (MT / 32) % 2 == 0, "the in-kernel pool needs the 32-column tiling and an even tile height");
-            {
-                cm_lds_barrier();
-                const float* pt = (const float*)smem4;
-                const int Ho = s.H >> 1, Wo = s.W >> 1;
-                for (int idx = tid; idx < FT * (TH / 2) * 16; idx += CM_THREADS) {
-                    const int pc = idx & 15, pr = (idx >> 4) % (TH / 2), fl = idx / (16 * (TH / 2));
-                    const int f = fg * FT + fl, yo = (y0 >> 1) + pr, xo = (x0 >> 1) + pc;
-                    if (f >= s.F || yo >= Ho || xo >= Wo) continue;
-                    const float* q = pt + (fl * TH + 2 * pr) * 32 + 2 * pc;
-                    const float m0 = q[0] > q[1] ? q[0] : q[1], m1 = q[32] > q[33] ? q[32] : q[33];
-                    e.pool[((long)f * Ho + yo) * Wo + xo] = m0 > m1 ? m0 : m1;
-                }
-            }
-        }
+        if constexpr (POOL) pool_tile();
     } else {
         // the loop above ended on a barrier: the staging buffers are free.  red[tile][group][register][lane]
         float* red = (float*)smem4 + wtile * (KG * 16 * 64);
@@ -342,6 +346,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
             for (int g = 1; g < KG; g++) v += red[(g * 16 + r) * 64 + lane];
             finish(0, r, v);
         }
+        if constexpr (POOL) pool_tile();
     }
     break;
     }
@@ -526,9 +531,12 @@ int fortis_launch_conv_split_reduce(const float* part, float* y, long osize, lon
     return 0;
 }
 
-// Channel groups inside a workgroup (the kernel's KG) for a conv on images: 4 when tiles of 64 positions x 64
-// channels would leave CUs without a workgroup (the launch would otherwise be split over the input channels into
-// partial sums and a reduce kernel), 1 otherwise.  Fg: output channels of the GEMM (4 F for the transposed conv).
+// Channel groups inside a workgroup (the kernel's KG) for a conv on images with at least 32 input channels, by the
+// number of 64 x 64 output tiles the launch would have: fewer than one per CU -> 4 (32 x 32 tiles whose four waves
+// divide the input channels; the launch would otherwise be split over the input channels into partial sums and a
+// reduce kernel); 3 x 3 convs with fewer than five per CU -> 2 (64 x 32 tiles, two waves per half of the channels:
+// twice to four times the workgroups of the plain form, which at one or two workgroups per CU leaves the matrix
+// pipes idle while a workgroup stages); 1 otherwise.  Fg: output channels of the GEMM (4 F for the transposed conv).
 // Weights are packed for the answer, so packing and launching ask with the same arguments.
 int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, int KS)
 {
@@ -536,8 +544,10 @@ int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, i
     if (off || KD != 1 || D != 1 || C < 32) return 1;
     if (KS == 3 && !(Wd >= 32 && cdiv(Wd, 32) * 32 * 4 <= 5L * Wd)) return 1;     // 3 x 3: the 32-column tiling only
     if (KS != 1 && KS != 3) return 1;
-    const long pos = KS == 3 ? H * (Wd + 1) : H * Wd;
-    return cdiv(pos, 64) * cdiv(Fg, 64) < conv_cus() ? 4 : 1;
+    const long pos = KS == 3 ? H * (Wd + 1) : H * Wd, tiles = cdiv(pos, 64) * cdiv(Fg, 64);
+    if (tiles < conv_cus()) return 4;
+    if (KS == 3 && tiles < 5L * conv_cus()) return 2;
+    return 1;
 }
 
 // Packs conv weights W[F][C][T] (T taps, row-major) into the kernel's order
@@ -548,7 +558,7 @@ int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, i
 float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats, int kg)
 {
     const long Fg = transposed ? 4 * F : F;
-    const long FT = kg == 4 ? 32 : conv_ft(Fg);
+    const long FT = kg > 1 ? 32 : conv_ft(Fg);
     const long CC = cm_cc(T) * kg, NCP = CC / 2;
     const long nfg = cdiv(Fg, FT), nch = cdiv(C, CC);
     const long wch = NCP * T * 2 * FT;
@@ -602,7 +612,7 @@ const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, h
 {
     static float* buf = nullptr;
     static size_t cap = 0;
-    const long FT = kg == 4 ? 32 : conv_ft(F), CC = cm_cc(T) * kg;
+    const long FT = kg > 1 ? 32 : conv_ft(F), CC = cm_cc(T) * kg;
     const long nch = cdiv(C, CC), n = cdiv(F, FT) * nch * (CC / 2) * T * 2 * FT;
     if (g_ws) {
         float* w = ws_take(0, (size_t)n * sizeof(float));
@@ -637,8 +647,8 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     }
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
     size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, 64) * 64) * sizeof(float);
-    if (KG > 1 && shmem < 4 * 16 * 64 * sizeof(float)) shmem = 4 * 16 * 64 * sizeof(float);   // the groups' sums meet in LDS
-    if (POOL && shmem < (size_t)FT * MT * sizeof(float)) shmem = (size_t)FT * MT * sizeof(float);   // the finished tile, for its 2 x 2 max pool
+    if (KG > 1 && shmem < 4 * 16 * 64 * sizeof(float)) shmem = 4 * 16 * 64 * sizeof(float);  // (4 / KG tiles) x KG groups x 16 registers x 64 lanes   // the groups' sums meet in LDS
+    if (POOL && shmem < (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float)) shmem = (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float);   // the finished tile, for its 2 x 2 max pool
     if (shmem > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
@@ -786,6 +796,15 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
     s.ksplit = 1;
     s.ups = kind == 2 ? 1 : 0;
     if (kind == 2 && ((D | H | Wd) & 1)) return -1;
+    if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 2) {
+        // 3 x 3 only: 64 x 32 output tiles (two rows of the 32-column tiling), two waves per row, each taking half of a chunk's channels
+        s.P = s.W + 1;
+        s.plane = s.H * s.P;
+        s.nchunks = (int)cdiv(s.C, cm_cc(9) * 2);
+        constexpr int NX2 = (cm_cc(9) * 2 * (64 / 32 + 2) * CM_TP + CM_THREADS - 1) / CM_THREADS;
+        if (e.pool && !s.mode && !(s.H & 1) && !(s.W & 1)) return launch_nx<1, 3, 64, 32, NX2, true, 2, true>(x, wp, y, s, e, st);
+        return launch_nx<1, 3, 64, 32, NX2, true, 2>(x, wp, y, s, e, st);
+    }
     if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 4) {
         // one 32 x 32 output tile per workgroup, the four waves share its input channels
         s.P = KS == 3 ? s.W + 1 : s.W;

@@ -29,7 +29,11 @@ pytestmark = pytest.mark.gpu
                                                     # share the input channels (sums meet in LDS); partial last chunk of 16 (3 x 3) and
                                                     # of 64 (1 x 1) channels, partial channel group, ragged height, a single tile
                                                     (40, 33, 64, 72, 3, 1, 1), (96, 20, 60, 32, 3, 1, 1), (32, 32, 32, 256, 3, 1, 1),
-                                                    (100, 16, 16, 48, 1, 1, 0), (64, 1, 32, 32, 1, 1, 0)])
+                                                    (100, 16, 16, 48, 1, 1, 0), (64, 1, 32, 32, 1, 1, 0),
+                                                    # between one and five 64 x 64 tiles per CU: 64 x 32 tiles whose waves share the input
+                                                    # channels in two groups; two groups of output channels with a partial one, a
+                                                    # partial last chunk of 8 channels, ragged width and height
+                                                    (44, 130, 126, 72, 3, 1, 1), (32, 128, 128, 64, 3, 1, 1)])
 def test_conv2d_bias_act_vs_oracle(L, gpu, C_, H, W, F, k, stride, pad):
     rng = np.random.default_rng(0)
     x = rng.standard_normal((C_, H, W)).astype(np.float32)
@@ -45,10 +49,11 @@ def test_conv2d_bias_act_vs_oracle(L, gpu, C_, H, W, F, k, stride, pad):
     p.close()
 
 
-@pytest.mark.parametrize("C_,H,W,F", [(16, 38, 64, 24), (8, 130, 96, 40), (48, 12, 32, 64)])
+@pytest.mark.parametrize("C_,H,W,F", [(16, 38, 64, 24), (8, 130, 96, 40), (48, 12, 32, 64), (44, 130, 126, 72), (32, 128, 160, 32)])
 def test_conv2d_with_max_pool_behind(L, gpu, C_, H, W, F):
     """3 x 3 conv + bias + ReLU followed by a 2 x 2 max pool: the conv pools its own tiles (32-column tiling, even tile
-    height; ragged last tile rows), or its channel-split reduce kernel does (the small, deep case).  Both outputs checked."""
+    height; ragged last tile rows; the last two shapes in the form whose waves share the input channels in two groups), or
+    its channel-split reduce kernel does (the small, deep case).  Both outputs checked."""
     rng = np.random.default_rng(11)
     x = rng.standard_normal((C_, H, W)).astype(np.float32)
     w = (rng.standard_normal((F, C_, 3, 3)) / np.sqrt(C_ * 9)).astype(np.float32)
