@@ -534,7 +534,7 @@ int fortis_launch_conv_split_reduce(const float* part, float* y, long osize, lon
 // Channel groups inside a workgroup (the kernel's KG) for a conv on images with at least 32 input channels, by the
 // number of 64 x 64 output tiles the launch would have: fewer than one per CU -> 4 (32 x 32 tiles whose four waves
 // divide the input channels; the launch would otherwise be split over the input channels into partial sums and a
-// reduce kernel); 3 x 3 convs with fewer than five per CU -> 2 (64 x 32 tiles, two waves per half of the channels:
+// reduce kernel); fewer than five per CU -> 2 (64 x 32 tiles, two waves per half of the channels:
 // twice to four times the workgroups of the plain form, which at one or two workgroups per CU leaves the matrix
 // pipes idle while a workgroup stages); 1 otherwise.  Fg: output channels of the GEMM (4 F for the transposed conv).
 // Weights are packed for the answer, so packing and launching ask with the same arguments.
@@ -546,7 +546,7 @@ int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, i
     if (KS != 1 && KS != 3) return 1;
     const long pos = KS == 3 ? H * (Wd + 1) : H * Wd, tiles = cdiv(pos, 64) * cdiv(Fg, 64);
     if (tiles < conv_cus()) return 4;
-    if (KS == 3 && tiles < 5L * conv_cus()) return 2;
+    if (tiles < 5L * conv_cus()) return 2;
     return 1;
 }
 
@@ -797,7 +797,13 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
     s.ups = kind == 2 ? 1 : 0;
     if (kind == 2 && ((D | H | Wd) & 1)) return -1;
     if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 2) {
-        // 3 x 3 only: 64 x 32 output tiles (two rows of the 32-column tiling), two waves per row, each taking half of a chunk's channels
+        if (KS == 1) {
+            s.P = s.W;
+            s.plane = s.H * s.P;
+            s.nchunks = (int)cdiv(s.C, cm_cc(1) * 2);
+            return launch_nx<1, 1, 64, 32, cm_cc(1) * 2 * 64 / CM_THREADS, false, 2>(x, wp, y, s, e, st);
+        }
+        // 64 x 32 output tiles (3 x 3: two rows of the 32-column tiling), two waves per 32 positions, each taking half of a chunk's channels
         s.P = s.W + 1;
         s.plane = s.H * s.P;
         s.nchunks = (int)cdiv(s.C, cm_cc(9) * 2);

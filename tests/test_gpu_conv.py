@@ -33,7 +33,9 @@ pytestmark = pytest.mark.gpu
                                                     # between one and five 64 x 64 tiles per CU: 64 x 32 tiles whose waves share the input
                                                     # channels in two groups; two groups of output channels with a partial one, a
                                                     # partial last chunk of 8 channels, ragged width and height
-                                                    (44, 130, 126, 72, 3, 1, 1), (32, 128, 128, 64, 3, 1, 1)])
+                                                    (44, 130, 126, 72, 3, 1, 1), (32, 128, 128, 64, 3, 1, 1),
+                                                    # the same form on a single tap (chunks of 32 channels, a partial last one)
+                                                    (48, 130, 127, 40, 1, 1, 0)])
 def test_conv2d_bias_act_vs_oracle(L, gpu, C_, H, W, F, k, stride, pad):
     rng = np.random.default_rng(0)
     x = rng.standard_normal((C_, H, W)).astype(np.float32)
@@ -73,11 +75,12 @@ def test_conv2d_with_max_pool_behind(L, gpu, C_, H, W, F):
     p.close()
 
 
-def test_convt2d_channel_groups_vs_oracle(L, gpu):
-    """2 x 2 stride-2 transposed conv on a small, deep image (the UNet's first up-convolution in small): the kernel form
-    whose waves share the input channels, with bias and ReLU, written into a channel range of a wider tensor."""
+@pytest.mark.parametrize("C_,H,W,F", [(72, 12, 20, 24), (40, 127, 130, 24)])
+def test_convt2d_channel_groups_vs_oracle(L, gpu, C_, H, W, F):
+    """2 x 2 stride-2 transposed conv on a small, deep image (the UNet's first up-convolution in small) and on a mid-sized
+    one: the kernel forms whose waves share the input channels in four and in two groups, with bias and ReLU, written
+    into a channel range of a wider tensor."""
     rng = np.random.default_rng(4)
-    C_, H, W, F = 72, 12, 20, 24
     x = rng.standard_normal((C_, H, W)).astype(np.float32)
     w = (rng.standard_normal((C_, F, 2, 2)) / np.sqrt(C_)).astype(np.float32)
     b = rng.standard_normal(F).astype(np.float32)
