@@ -29,6 +29,17 @@ typedef __attribute__((address_space(1))) v4f gv4f;   // 16 bytes of global memo
 #define CH_THREADS 256
 #define CH_NACC 4       // n-tiles a wave accumulates at once
 
+// max(v, 0) in one instruction.  fmaxf(v, 0.f) costs two on an accumulator that comes straight from a matrix
+// instruction: the compiler first quiets a possible signalling NaN with v_max_f32 v, v (it does not know that
+// matrix results are already canonical).  Same result for every input that is not a signalling NaN, -0 and quiet
+// NaNs (-> +0) included.
+__device__ __forceinline__ float relu_acc(float v)
+{
+    float d;
+    asm("v_max_f32 %0, 0, %1" : "=v"(d) : "v"(v));
+    return d;
+}
+
 __device__ __forceinline__ float apply_act(float v, int act, float alpha)
 {
     if (act == FORTIS_ACT_RELU) return v > 0.f ? v : 0.f;
@@ -276,7 +287,7 @@ __device__ __forceinline__ void layer_fixed(v4f (&a)[4], const float* sWts, cons
 #pragma unroll
         for (int u = 0; u < NT; u++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) a[u][r] = fmaxf(acc[u][r], 0.f);
+            for (int r = 0; r < 4; r++) a[u][r] = relu_acc(acc[u][r]);
     } else if (act == FORTIS_ACT_NONE) {
 #pragma unroll
         for (int u = 0; u < NT; u++) a[u] = acc[u];
@@ -536,7 +547,7 @@ void chain_wave_kernel(ChainParams params)
 #pragma unroll
                     for (int r = 0; r < 4; r++) a[u][r] = actf(o[u][r]);
             };
-            if (R.act == FORTIS_ACT_RELU) next_in([](float v) { return fmaxf(v, 0.f); });
+            if (R.act == FORTIS_ACT_RELU) next_in([](float v) { return relu_acc(v); });
             else if (R.act == FORTIS_ACT_NONE) next_in([](float v) { return v; });
             else next_in([&](float v) { return apply_act(v, R.act, R.alpha); });
         }
