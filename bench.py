@@ -249,12 +249,18 @@ def run_zb_unfused(L, args):
     ms = (C.c_float * 3)()
     assert L.fortis_time_parts_ms(3, parts, None, args.steps, ms) == 0
     g_ms, m_ms, s_ms = (v / args.steps for v in ms)
+    # the gather alone, launched back to back (what a kernel trace of a gather-only loop shows): reported beside the
+    # in-step figure, which is the one the roofline block is priced on
+    alone = (C.c_float * 1)()
+    assert L.fortis_time_parts_ms(1, (CB * 1)(gather_cb), None, max(10, args.steps), alone) == 0
+    ga_ms = alone[0] / max(10, args.steps)
     g_bytes = esz * 4 * n3 + 4 * 27 * rows                 # 4 planes read once, X written
     s_bytes = 4 * 3 * rows + esz * (n3 + nz * sx * sy + 3 * rows)  # Y read, norm + kappa read per layer, 3 outputs written
     gbs = g_bytes / (g_ms * 1e-3) / 1e9
     kname = "gather_generic_kernel (typed stencil gather, fp64 host arrays)" if args.f64 else "gather_kernel (stencil gather with lifted expressions)"
     roof = dict(bound="hbm", kernel=kname, achieved=round(gbs, 1), peak=PEAK_HBM_GBS,
                 unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(g_ms, 5), bytes_per_launch=g_bytes,
+                back_to_back_ms=round(ga_ms, 5), back_to_back_frac=round(g_bytes / (ga_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                 scatter_GBs=round(s_bytes / (s_ms * 1e-3) / 1e9, 1), scatter_ms_all_layers=round(s_ms, 5), mlp_ms=round(m_ms, 5),
                 traffic=MEASURED_TRAFFIC.get("zb_unfused_%dx%dx%d%s" % (sx, sy, nz, "_f64" if args.f64 else "")))
     out = dict(rows=rows, dt=dt, dtype="f32",
@@ -557,6 +563,9 @@ def run_others(L, args):
                     "value": r["rows"] * steps / r["dt"], "unit": r.get("unit", "columns/s"), "bound": roof["bound"],
                     "kernel": roof["kernel"], "achieved": roof["achieved"], "peak": roof["peak"], "roofline_unit": roof["unit"],
                     "frac": roof["frac"], "avg_launch_ms": roof["avg_launch_ms"]})
+        for k in ("back_to_back_ms", "back_to_back_frac"):     # the unfused step's gather launched alone
+            if k in roof:
+                out[-1][k] = roof[k]
     return out
 
 
