@@ -823,6 +823,7 @@ void chain_stencil_rows_kernel(ChainParams params)
     const int lrow = lane & 15, lq = lane >> 4;
     const gfloat* wall = st_g(d.wall);
     const gfloat* in_div = st_g(d.in_div);
+    const gfloat* in_rcp = st_g(d.in_rcp);
     const gfloat* out_mul = st_g(d.out_mul);
     const unsigned g_si = (unsigned)st_u(g.refs[0].si), g_sj = (unsigned)st_u(g.refs[0].sj), g_pl = (unsigned)st_u((int)g.refs[0].plane);
     const unsigned o_si = (unsigned)st_u(sc.refs[0].si), o_sj = (unsigned)st_u(sc.refs[0].sj), o_pl = (unsigned)st_u((int)sc.refs[0].plane);
@@ -889,10 +890,15 @@ void chain_stencil_rows_kernel(ChainParams params)
 #pragma unroll
             for (int q = 0; q < NS; q++) cell.S[q] = in.gS[q];
             st_cell_program(g, cell);
-            st_chain_apply(g, cell, in.x);
+            st_chain_apply<NQ, true>(g, cell, in.x);
             // (slots past the network's inputs, which hold a copy of slot 0, are zeroed in the LDS tile below; rows past
             // the end hold the first cell's values and their results are never stored: no per-slot select here)
-            if (in_div) {
+            if (in_rcp && st_div_wave_in_range(in.x, 1.f)) {
+                // divisors in range (checked when the step was built), numerators too: the short form of the division
+#pragma unroll
+                for (int q = 0; q < NQ; q++)
+                    if (q < K0) in.x[q] = st_div_inrange(in.x[q], in_div[q], in_rcp[q]);
+            } else if (in_div) {
 #pragma unroll
                 for (int q = 0; q < NQ; q++)
                     if (q < K0) in.x[q] = __fdiv_rn(in.x[q], in_div[q]);
@@ -962,6 +968,17 @@ void chain_stencil_rows_kernel(ChainParams params)
             for (int r = 0; r < 4; r++) if (r < NO) st_uptr(st_g(sc.refs[r].p))[soff] = ov[r];
         }
     }
+}
+
+__global__ void chain_rcp_kernel(const float* __restrict__ div, float* __restrict__ rcp, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) rcp[i] = st_div_rcp(div[i]);
+}
+void fortis_chain_fill_rcp(const float* div, float* rcp, int n, hipStream_t s)
+{
+    hipLaunchKernelGGL(chain_rcp_kernel, dim3((unsigned)cdiv(n, 64)), dim3(64), 0, s, div, rcp, n);
+    HIP_OK(hipGetLastError());
 }
 
 // ---- host side ---------------------------------------------------------------------------------------

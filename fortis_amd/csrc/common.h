@@ -47,6 +47,7 @@ struct ChainDesc {
     const float* wall;     // device blob: every layer's packed weights and zero-padded bias
     int wfloats;           // its length in floats (multiple of 4)
     const float* in_div;   // x / in_div[c] before layer 0, or null
+    const float* in_rcp;   // refined reciprocals of in_div (fortis_chain_fill_rcp) when every in_div[c] lies in [2^-40, 2^40], else null
     const float* out_mul;  // y * out_mul[c] after the last layer, or null
     int mask_tail;         // ReLU on the last mask_tail outputs
     int ld;                // LDS row pitch in floats
@@ -57,6 +58,9 @@ struct ChainDesc {
 int fortis_chain_build(ChainDesc* d, int nlayers, const float* const* W, const float* const* b, const int* K,
                        const int* N, float** blob_out);
 void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows, hipStream_t s);
+// rcp[c] = the refined reciprocal of div[c] exactly as the IEEE division sequence forms it (v_rcp_f32 and one Newton
+// step), computed on the device so that a kernel dividing many numerators by div[c] can take it from memory.
+void fortis_chain_fill_rcp(const float* div, float* rcp, int n, hipStream_t s);
 // ---- stencil tables as the kernels see them (stencil.hip) --------------------------------
 #define ST_KREFS 32     // slots a kernel launch handles: the fused-form kernels take tables up to this, the general ones chunk
 struct CellStep { int op, code, tv_left; };

@@ -327,6 +327,16 @@ static size_t try_chain(fortis_plan* p, size_t i, Exec* ex)
         for (size_t l = 0; l < lin.size(); l++) { d.L[l].act = lin[l]->act; d.L[l].alpha = lin[l]->alpha; }
     }
     if (in_div) d.in_div = (const float*)upload(p, in_div->v0.data(), in_div->v0.size() * 4);
+    if (in_div && d.in_div) {
+        // divisors all in [2^-40, 2^40]: their refined reciprocals go beside them, for the kernels' short division
+        bool ok = true;
+        for (float v : in_div->v0) { const float m = fabsf(v); ok = ok && m >= 0x1p-40f && m <= 0x1p40f; }
+        if (ok) {
+            std::vector<float> z(in_div->v0.size(), 0.f);
+            float* r = (float*)upload(p, z.data(), z.size() * 4);
+            if (r) { fortis_chain_fill_rcp(d.in_div, r, (int)z.size(), fortis_stream_get()); d.in_rcp = r; }
+        }
+    }
     if (out_mul) d.out_mul = (const float*)upload(p, out_mul->v0.data(), out_mul->v0.size() * 4);
     d.mask_tail = mask ? (int)mask->tail : 0;
     return j - i;

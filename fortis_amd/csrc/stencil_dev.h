@@ -151,10 +151,50 @@ __device__ __forceinline__ void st_prepare(const A& d, int i, int j, int kk, StC
     }
     st_cell_program(d, cell);
 }
+// ---- many numerators over one divisor ------------------------------------------------------------------------
+// The compiler's IEEE fp32 division is eleven instructions: v_div_scale_f32 of both operands, v_rcp_f32, a Newton
+// step on the reciprocal, the quotient with two residual corrections (the last one in v_div_fmas_f32) and
+// v_div_fixup_f32.  When numerator and divisor both lie in [2^-40, 2^40] neither v_div_scale scales (no operand or
+// quotient comes near the ends of the exponent range), v_div_fmas is a plain fma and v_div_fixup returns its input,
+// so the same result, bit for bit, comes from the reciprocal's two fmas once per divisor and a multiply and four
+// fmas per numerator.  st_div_key maps a value to its bit pattern without the sign: the range is then an unsigned
+// interval (zeros, denormals, infinities and NaNs fall outside), and a whole set of values is checked through its
+// smallest and largest key.
+#define ST_DIV_KEY_LO (87u << 24)       // 2^-40
+#define ST_DIV_KEY_HI (168u << 24)      // 2^41: keys below it have exponents up to 2^40
+__device__ __forceinline__ unsigned st_div_key(float v) { return __float_as_uint(v) << 1; }
+__device__ __forceinline__ float st_div_rcp(float d)
+{
+    const float r = __builtin_amdgcn_rcpf(d);
+    return fmaf(fmaf(-d, r, 1.f), r, r);
+}
+// n / d given rcp = st_div_rcp(d); both operands in range
+__device__ __forceinline__ float st_div_inrange(float n, float d, float rcp)
+{
+    const float q0 = __fmul_rn(n, rcp);
+    const float q1 = fmaf(fmaf(-d, q0, n), rcp, q0);
+    return fmaf(fmaf(-d, q1, n), rcp, q1);
+}
+// true when every lane of the wave has all its N values (and `also`) in range
+template <int N>
+__device__ __forceinline__ bool st_div_wave_in_range(const float (&v)[N], float also)
+{
+    unsigned lo = st_div_key(also), hi = lo;
+#pragma unroll
+    for (int t = 0; t < N; t++) {
+        const unsigned k = st_div_key(v[t]);
+        lo = k < lo ? k : lo;
+        hi = k > hi ? k : hi;
+    }
+    const bool out = lo < ST_DIV_KEY_LO || hi >= ST_DIV_KEY_HI;
+    return __builtin_amdgcn_ballot_w64(out) == 0;
+}
+
 // Runs the tv chain on N slot values at once: the loop over chain steps is a real loop (one table
 // read and one wave-uniform switch per step), each arm handles all N values, so the generated code
 // holds each operation once per arm instead of once per slot and step.
-template <int N, typename A, int NS, int NC>
+// FASTDIV: a division of all N values by the step's operand takes the short in-range form when the whole wave allows it.
+template <int N, bool FASTDIV = false, typename A, int NS, int NC>
 __device__ __forceinline__ void st_chain_apply(const A& d, const StCellT<NS, NC>& cell, float (&tv)[N])
 {
     const int nchain = st_u(d.nchain);
@@ -183,6 +223,12 @@ __device__ __forceinline__ void st_chain_apply(const A& d, const StCellT<NS, NC>
                 for (int t = 0; t < N; t++) tv[t] = __fdiv_rn(o, tv[t]);
                 break;
             default:
+                if (FASTDIV && st_div_wave_in_range(tv, o)) {
+                    const float rcp = st_div_rcp(o);
+#pragma unroll
+                    for (int t = 0; t < N; t++) tv[t] = st_div_inrange(tv[t], o, rcp);
+                    break;
+                }
 #pragma unroll
                 for (int t = 0; t < N; t++) tv[t] = __fdiv_rn(tv[t], o);
                 break;

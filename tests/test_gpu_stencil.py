@@ -320,6 +320,69 @@ def test_bench_grid_fused_equals_unfused_and_layer_vs_oracle(L, gpu):
     plan.close()
 
 
+
+def test_rows_form_divisions_with_operands_outside_the_short_range(L, gpu):
+    """The lane-per-row form of the fused step (taken from 786 k rows on) divides the short way only when a whole wave's
+    numerators and divisors lie in [2^-40, 2^40], in the lifted expression tv / (S0 + 1e-30f) and in the network's input
+    normalisation alike.  Here a share of the field values lies outside: zeros of both signs,
+    denormals, values just outside and on the ends of the range, all-ones mantissas, huge values, infinities, NaNs,
+    sparse enough that waves of both kinds occur.  The fused step must equal the unfused structure (whose gather kernel
+    always divides the long way) bit for bit in Y and in the written fields (any NaN equals any NaN), and its X of one
+    layer must equal the oracle's."""
+    sx, sy, nz = 600, 600, 3
+    gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    gt, st = S.build_table(gd, lp, kd, "gather"), S.build_table(sd, lp, kd, "scatter")
+    A = configs.zb_arrays(sx, sy, nz)
+    rng = np.random.default_rng(33)
+    ones = np.array([0x3FFFFFFF, 0x2B7FFFFF, 0x53FFFFFF, 0x007FFFFF, 0x7F7FFFFF, 0x00000001, 0x80000001], np.uint32).view(np.float32)
+    special = np.concatenate([np.array([0.0, -0.0, 1e-45, 3e-39, 1.1754944e-38, 2.0 ** -100, 2.0 ** -41, -2.0 ** -41, 2.0 ** -40, -2.0 ** -40,
+                                        2.0 ** 40, -2.0 ** 40, 2.0 ** 41, 2.0 ** 64, -2.0 ** 100, 3.4028235e38, np.inf, -np.inf, np.nan], np.float32), ones])
+    n2, n3 = sx * sy, sx * sy * nz
+    for k in ("sh_xy_h", "sh_xx", "vort_xy_h", "norm_h"):
+        a = A[k].reshape(-1)
+        pick = rng.random(a.size) < 2e-4
+        a[pick] = rng.choice(special, int(pick.sum()))
+    count = (sx - 4) * (sy - 4)
+    rows = count * nz
+    assert rows >= 786432
+    net = configs.zb_mlp()
+    # input normalisation as in the reference's network (x / in_norms before the first layer): the step's second division
+    in_norms = rng.uniform(0.5, 2.0, 27).astype(np.float32)
+    out_norms = rng.uniform(0.5, 2.0, 3).astype(np.float32)
+    plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows, in_norms=in_norms, out_norms=out_norms)
+    assert plan.num_kernels == 1
+    garr = [A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"]]
+    host = [A["norm_h"], A["kappa_h"], np.zeros(n3, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)]
+
+    def same(a, b):
+        a, b = np.ascontiguousarray(a, dtype=np.float32), np.ascontiguousarray(b, dtype=np.float32)
+        return a.shape == b.shape and bool(np.all((a.view(np.uint32) == b.view(np.uint32)) | (np.isnan(a) & np.isnan(b))))
+    with np.errstate(all="ignore"):
+        fused_out, fused_Y = _fused(L, gt, st, plan, garr, host, rows)
+        gb, sb = [DevBuf(L, a) for a in garr], [DevBuf(L, a) for a in host]
+        dX = L.fortis_plan_tensor_ptr(plan.handle, plan.in_tensor)
+        dY = L.fortis_plan_tensor_ptr(plan.handle, plan.out_tensor)
+        L.fortis_stencil_gather_dev(C.byref(gt), ptrs(gb), C.c_void_p(dX))
+        X = np.empty((rows, 27), np.float32)
+        L.fortis_d2h(X.ctypes.data, C.c_void_p(dX), X.nbytes)
+        plan.run()
+        for kk in range(nz):
+            L.fortis_stencil_scatter_dev(C.byref(st), ptrs(sb), C.c_void_p(dY + kk * count * 3 * 4), kk)
+        L.fortis_sync()
+        Y = np.empty((rows, 3), np.float32)
+        L.fortis_d2h(Y.ctypes.data, C.c_void_p(dY), Y.nbytes)
+        assert same(Y, fused_Y)
+        for q in (3, 4):
+            assert same(sb[q].get(host[q].shape), fused_out[q])
+        # rows with an operand outside the range, and rows without, both occur in numbers
+        bad = ~np.all((np.abs(X) >= 2.0 ** -80) & (np.abs(X) <= 2.0 ** 80), axis=1)
+        assert 1000 < int(bad.sum()) < rows // 4
+        assert same(X[:count], O.stencil_gather(gd, garr, count, nz, 3, 3, sx - 4)[:count])
+    for b in gb + sb:
+        b.free()
+    plan.close()
+
+
 @pytest.mark.parametrize("form", ["16", "64"])
 @pytest.mark.parametrize("sx,sy,nz,hidden", [(68, 78, 15, (64, 64)), (37, 29, 3, (20,)), (133, 70, 2, (48, 16, 8))])
 def test_fused_step_both_fast_forms(L, gpu, form, sx, sy, nz, hidden):
