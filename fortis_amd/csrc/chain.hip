@@ -842,14 +842,16 @@ void chain_stencil_rows_kernel(ChainParams params)
         const unsigned gbyte = goff << 2;
         typedef __attribute__((address_space(1))) char gchar;
 #pragma unroll
-        for (int q = 0; q < NQ; q++) in.x[q] = *(const gfloat*)((const gchar*)st_uptr(st_g(g.refs[q].p)) + gbyte);   // entries past the table's repeat slot 0
+        // (the slot pointers straight from the kernel arguments, by literal index: scalar loads, where the copy of the
+        // arguments in LDS costs a vector read and two v_readfirstlane per pointer and tile)
+        for (int q = 0; q < NQ; q++) in.x[q] = *(const gfloat*)((const gchar*)st_uptr(st_g(params.g.refs[q].p)) + gbyte);   // entries past the table's repeat slot 0
 #pragma unroll
-        for (int q = 0; q < NS; q++) in.gS[q] = *(const gfloat*)((const gchar*)st_uptr(st_g(g.scal[q].p)) + gbyte);
+        for (int q = 0; q < NS; q++) in.gS[q] = *(const gfloat*)((const gchar*)st_uptr(st_g(params.g.scal[q].p)) + gbyte);
 #pragma unroll
         for (int q = 0; q < NS; q++) {
-            const unsigned ssi = (unsigned)st_u(sc.scal[q].si), ssj = (unsigned)st_u(sc.scal[q].sj), spl = (unsigned)st_u((int)sc.scal[q].plane);
+            const unsigned ssi = (unsigned)st_u(params.sc.scal[q].si), ssj = (unsigned)st_u(params.sc.scal[q].sj), spl = (unsigned)st_u((int)params.sc.scal[q].plane);
             const unsigned off = (ssi == o_si && ssj == o_sj && spl == o_pl) ? in.soff : (unsigned)i * ssi + (unsigned)j * ssj + (unsigned)kk * spl;
-            in.sS[q] = st_uptr(st_g(sc.scal[q].p))[off];
+            in.sS[q] = st_uptr(st_g(params.sc.scal[q].p))[off];
         }
     };
 
@@ -965,7 +967,7 @@ void chain_stencil_rows_kernel(ChainParams params)
         st_chain_apply(sc, cell, ov);
         if (valid) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) if (r < NO) st_uptr(st_g(sc.refs[r].p))[soff] = ov[r];
+            for (int r = 0; r < 4; r++) if (r < NO) st_uptr(st_g(params.sc.refs[r].p))[soff] = ov[r];
         }
     }
 }
