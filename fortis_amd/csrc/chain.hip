@@ -29,15 +29,17 @@ typedef __attribute__((address_space(1))) v4f gv4f;   // 16 bytes of global memo
 #define CH_THREADS 256
 #define CH_NACC 4       // n-tiles a wave accumulates at once
 
-// max(v, 0) in one instruction.  fmaxf(v, 0.f) costs two on an accumulator that comes straight from a matrix
-// instruction: the compiler first quiets a possible signalling NaN with v_max_f32 v, v (it does not know that
-// matrix results are already canonical).  Same result for every input that is not a signalling NaN, -0 and quiet
-// NaNs (-> +0) included.
+// max(v, 0) in one instruction, on the bit pattern: a float with the sign bit set is a negative integer, so the signed
+// integer maximum with 0 leaves positive values as they are and turns negative ones and -0 into +0 (a NaN keeps its
+// bits if its sign is clear and becomes +0 otherwise).  fmaxf(v, 0.f) costs two instructions on an accumulator that
+// comes straight from a matrix instruction: the compiler first quiets a possible signalling NaN with v_max_f32 v, v
+// (it does not know that matrix results are already canonical, and it rewrites v_med3_f32(v, 0, inf) to the same
+// pair).  Written in C, not as inline assembly: the compiler then keeps its own bookkeeping of the wait states between
+// a matrix instruction and a reader of its result (an asm statement escapes it and read accumulators too early).
 __device__ __forceinline__ float relu_acc(float v)
 {
-    float d;
-    asm("v_max_f32 %0, 0, %1" : "=v"(d) : "v"(v));
-    return d;
+    const int b = __float_as_int(v);
+    return __int_as_float(b > 0 ? b : 0);
 }
 
 __device__ __forceinline__ float apply_act(float v, int act, float alpha)
@@ -258,7 +260,8 @@ __device__ __forceinline__ void layer_group(const v4f (&a)[KGMAX], v4f* o, const
 // compile-time, so every weight and bias read is a per-lane base (set once per layer) plus a literal offset, no
 // branch separates the reads from the MFMAs and the compiler is free to issue the reads ahead.  The activation is
 // applied in place: a[0 .. NT) leave as the next layer's operand.
-template <int NT, int KG, bool WLDS>
+// RELU: the activation is known to be ReLU (no choice left in the code).
+template <int NT, int KG, bool WLDS, bool RELU = false>
 __device__ __forceinline__ void layer_fixed(v4f (&a)[4], const float* sWts, const gfloat* wall, int woff4, int boff, int lane,
                                             int lq, int act, float alpha)
 {
@@ -283,7 +286,7 @@ __device__ __forceinline__ void layer_fixed(v4f (&a)[4], const float* sWts, cons
 #pragma unroll
         for (int u = 0; u < NT; u++) acc[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u].w, a[kg].w, acc[u], 0, 0, 0);
     }
-    if (act == FORTIS_ACT_RELU) {
+    if (RELU || act == FORTIS_ACT_RELU) {
 #pragma unroll
         for (int u = 0; u < NT; u++)
 #pragma unroll
@@ -318,7 +321,7 @@ __device__ __forceinline__ void layer_narrow(v4f (&a)[4], const LayerRegs& R, co
 // i's weight for the feature those rows bring, and every lane ends up with its row's four outputs summed over the 16
 // features per k group that its quarter carries (quarter 0 starts at the bias).  The quarters' sums are still to
 // be added: last_x4_sum does it across the lanes, (q0 + q2) + (q1 + q3), and applies the activation.
-template <bool WLDS>
+template <bool WLDS, int KGX = 0>      // KGX > 0: the layer's k groups, known at compile time
 __device__ __forceinline__ v4f last_x4_partial(const v4f (&a)[4], const LayerRegs& R, int x4off, const float* sWts, const gfloat* wall,
                                                int lane, int lq)
 {
@@ -328,7 +331,7 @@ __device__ __forceinline__ v4f last_x4_partial(const v4f (&a)[4], const LayerReg
     if (lq) acc = (v4f)(0.f);
 #pragma unroll
     for (int u = 0; u < 4; u++)
-        if (u < R.KG) {
+        if (KGX ? u < KGX : u < R.KG) {
             v4f w;
             if (WLDS) w = ((const v4f*)sWts)[wo + u]; else w = ((const gv4f*)wall)[wo + u];
             acc = __builtin_amdgcn_mfma_f32_4x4x1f32(w.x, a[u].x, acc, 0, 0, 0);
@@ -353,9 +356,30 @@ __device__ __forceinline__ v4f last_x4_sum(v4f acc, const LayerRegs& R)
 // All layers of a narrow network on the operand in a[]; the result is left in a[].  XSUM false: a last layer in the
 // 4x4x1 form leaves each quarter's partial sums in a[0] and returns true; the caller adds them, (q0 + q2) + (q1 + q3),
 // and applies the layer's activation.
-template <bool WLDS, bool XSUM = true>
+// SIG: the network's shape when the launcher has matched it (chain_signature), 0 otherwise.  A matched network runs as
+// straight-line code; the general path picks each layer's code by a switch on its shape, whose arms the compiler joins
+// with copies of the operand registers -- 16 moves per layer and 16 rows.
+//   SIG 1: Kp 32 -> 64 -> 64 -> at most 4 outputs (4x4x1 form), ReLU behind both hidden layers
+//   SIG 2: Kp 32 -> 32 -> at most 4 outputs (4x4x1 form), ReLU behind the hidden layer
+template <bool WLDS, bool XSUM = true, int SIG = 0>
 __device__ __forceinline__ bool layers_narrow(v4f (&a)[4], const ChainDesc& d, int nlayers, const float* sWts, const gfloat* wall, int lane, int lq)
 {
+    if constexpr (SIG == 1 || SIG == 2) {
+        asm volatile("" ::: "memory");
+        const LayerRegs R0 = layer_regs(d, 0);
+        if constexpr (SIG == 1) layer_fixed<4, 2, WLDS, true>(a, sWts, wall, R0.woff / 4, R0.boff, lane, lq, FORTIS_ACT_RELU, 0.f);
+        else layer_fixed<2, 2, WLDS, true>(a, sWts, wall, R0.woff / 4, R0.boff, lane, lq, FORTIS_ACT_RELU, 0.f);
+        if constexpr (SIG == 1) {
+            asm volatile("" ::: "memory");
+            const LayerRegs R1 = layer_regs(d, 1);
+            layer_fixed<4, 4, WLDS, true>(a, sWts, wall, R1.woff / 4, R1.boff, lane, lq, FORTIS_ACT_RELU, 0.f);
+        }
+        asm volatile("" ::: "memory");
+        const LayerRegs R = layer_regs(d, SIG == 1 ? 2 : 1);
+        const v4f part = last_x4_partial<WLDS, SIG == 1 ? 4 : 2>(a, R, st_u(d.x4off), sWts, wall, lane, lq);
+        a[0] = XSUM ? last_x4_sum(part, R) : part;
+        return true;
+    }
     const int x4off = st_u(d.x4off);
     const int nfull = x4off >= 0 ? nlayers - 1 : nlayers;
     for (int l = 0; l < nfull; l++) {
@@ -802,7 +826,7 @@ void chain_stencil_fast_kernel(ChainParams params)
 // as the slot registers are free, i.e. before the four m-tiles are multiplied.
 #define CSR_PITCH 36
 #define CSR_THREADS 512      // eight waves share one LDS copy of the weights: four waves per SIMD stay resident
-template <bool WLDS, int NQ>
+template <bool WLDS, int NQ, int SIG = 0>
 __global__ __launch_bounds__(CSR_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void chain_stencil_rows_kernel(ChainParams params)
 {
@@ -929,7 +953,7 @@ void chain_stencil_rows_kernel(ChainParams params)
                 v4f a[4];
                 const v4f* src = (const v4f*)(sOp + (16 * T + lrow) * CSR_PITCH) + lq;
                 a[0] = src[0]; a[1] = src[4];      // (a[2], a[3]: a layer reads as many k groups as the one before it wrote n-tiles)
-                if (layers_narrow<WLDS, false>(a, d, nlayers, sWts, wall, lane, lq)) {
+                if (layers_narrow<WLDS, false, SIG>(a, d, nlayers, sWts, wall, lane, lq)) {
                     // the quarters' partial sums of the last layer meet in the tile's own operand rows (consumed above)
                     v4f* tmp = (v4f*)(sOp + 16 * T * CSR_PITCH);
                     tmp[lq * 16 + lrow] = a[0];
@@ -1216,22 +1240,33 @@ static void launch_stencil_fast(ChainParams& P, hipStream_t s)
     HIP_OK(hipGetLastError());
 }
 
-template <bool WLDS, int NQ>
+// The shapes layers_narrow has straight-line code for (its SIG), 0 for any other network.
+static int chain_signature(const ChainDesc& d)
+{
+    static const int off = getenv("FORTIS_CHAIN_SIGNATURE") != nullptr && atoi(getenv("FORTIS_CHAIN_SIGNATURE")) == 0;
+    if (off || d.x4off < 0) return 0;
+    auto hidden = [&](int l, int Kp, int Np) { return d.L[l].Kp == Kp && d.L[l].Np == Np && d.L[l].act == FORTIS_ACT_RELU; };
+    if (d.nlayers == 3 && hidden(0, 32, 64) && hidden(1, 64, 64) && d.L[2].Kp == 64) return 1;
+    if (d.nlayers == 2 && hidden(0, 32, 32) && d.L[1].Kp == 32) return 2;
+    return 0;
+}
+
+template <bool WLDS, int NQ, int SIG = 0>
 static void launch_stencil_rows(ChainParams& P, hipStream_t s)
 {
     const size_t shmem = ((size_t)(WLDS ? P.d.wfloats : 0) + (CSR_THREADS / 64) * (32 * CSR_PITCH + 64 * 4)) * sizeof(float);
     static size_t attr = 0;
     static long slots = 0;
     if (shmem > attr || !slots) {
-        HIP_OK(hipFuncSetAttribute((const void*)chain_stencil_rows_kernel<WLDS, NQ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        HIP_OK(hipFuncSetAttribute((const void*)chain_stencil_rows_kernel<WLDS, NQ, SIG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         attr = shmem;
         int occ = 0;
-        HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void*)chain_stencil_rows_kernel<WLDS, NQ>, CSR_THREADS, shmem));
+        HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void*)chain_stencil_rows_kernel<WLDS, NQ, SIG>, CSR_THREADS, shmem));
         slots = (long)(occ < 1 ? 1 : occ) * num_cus();
     }
     long grid = cdiv(P.rows, CSR_THREADS);
     if (grid > slots) grid = slots;
-    hipLaunchKernelGGL((chain_stencil_rows_kernel<WLDS, NQ>), dim3((unsigned)grid), dim3(CSR_THREADS), shmem, s, P);
+    hipLaunchKernelGGL((chain_stencil_rows_kernel<WLDS, NQ, SIG>), dim3((unsigned)grid), dim3(CSR_THREADS), shmem, s, P);
     HIP_OK(hipGetLastError());
 }
 
@@ -1253,6 +1288,10 @@ void fortis_launch_chain_stencil(const ChainDesc& d, const StencilDev& g, const 
         const bool wlds = chain_wave_wlds(P.d);
         if (v1) { if (wlds) launch_stencil_fast<true>(P, s); else launch_stencil_fast<false>(P, s); return; }
         const int k0 = P.d.L[0].K;
+        // the two ZB networks (27 -> 64 -> 64 -> 3 and the reference's 27 -> 20 -> 3) as straight-line code
+        const int sig = wlds && k0 > 16 && k0 <= 28 ? chain_signature(P.d) : 0;
+        if (sig == 1) { launch_stencil_rows<true, 28, 1>(P, s); return; }
+        if (sig == 2) { launch_stencil_rows<true, 28, 2>(P, s); return; }
         if (wlds) { if (k0 <= 16) launch_stencil_rows<true, 16>(P, s); else if (k0 <= 28) launch_stencil_rows<true, 28>(P, s); else launch_stencil_rows<true, 32>(P, s); }
         else { if (k0 <= 16) launch_stencil_rows<false, 16>(P, s); else if (k0 <= 28) launch_stencil_rows<false, 28>(P, s); else launch_stencil_rows<false, 32>(P, s); }
         return;
