@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # same command (see profiles/), or None where no counter run has been made for the workload.
 MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((1114.1 * 2 + 885.2) * 1024),
-                    "zb_ref": int((1005.6 * 2 + 885.2) * 1024), "zb_1028x1028x15": int((194914.8 * 2 + 191641.6) * 1024),
+                    "zb_ref": int((1005.6 * 2 + 885.2) * 1024), "zb_1028x1028x15": int((200333.1 * 2 + 192541.4) * 1024),
                     "zb_ref_1028x1028x15": int((196300.7 * 2 + 195918.0) * 1024), "toy": None,
                     "zb_unfused_1028x1028x15": int((242212.5 * 2 + 1658926.8) * 1024),
                     "zb_unfused_1028x1028x15_f64": int((247386.7 * 2 + 1658898.9) * 1024),
