@@ -170,14 +170,17 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         // uniform base + 32-bit byte offset per lane: no address arithmetic here.  Padding elements read
         // offset 0 (a valid address); they are replaced by zero only when stored, so nothing waits here.
         const char* xsrc = (const char*)(x + (long)ch * CC * schan);
-        if ((ch + 1) * CC <= s.C) {
+        if ((ch + 1) * CC > s.C) {
+            // partial last chunk: channels past the last one read offset 0 too.  It is the last chunk this tile loads,
+            // so the offsets are clamped in place (one load site; a second one with clamped copies cost every chunk a
+            // move per offset where the two join); the empty asm keeps this a branch
+            asm volatile("" ::: "memory");
+            const unsigned lim = chunk_lim(ch);
 #pragma unroll
-            for (int i = 0; i < NX; i++) r.rx[i] = *(const float*)(xsrc + goff[i]);
-        } else {
-            const unsigned lim = chunk_lim(ch);      // partial last chunk: channels past the last one read offset 0 too
-#pragma unroll
-            for (int i = 0; i < NX; i++) r.rx[i] = *(const float*)(xsrc + (goff[i] < lim ? goff[i] : 0u));
+            for (int i = 0; i < NX; i++) goff[i] = goff[i] < lim ? goff[i] : 0u;
         }
+#pragma unroll
+        for (int i = 0; i < NX; i++) r.rx[i] = *(const float*)(xsrc + goff[i]);
     };
     auto store_chunk = [&](const Regs& r, int buf, int ch) {
         cm_v4f* wdst = (cm_v4f*)(sW + buf * WCH);
