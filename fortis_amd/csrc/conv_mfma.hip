@@ -128,11 +128,13 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     // group, (c * schan + offset in the channel) * 4.  Padding elements load from offset 0 (goff) and carry
     // the mark 0xffffffff in gchk, which the store compares with the chunk's limit.
     unsigned goff[NX], gchk[NX];
+    bool inb[NX];                // the element lies inside the tensor (not padding, not past the staged run)
 #pragma unroll
     for (int i = 0; i < NX; i++) {
         const int el = tid + i * CM_THREADS;
         goff[i] = 0;
         gchk[i] = 0xffffffffu;
+        inb[i] = false;
         if (el < XCH) {
             unsigned c, rem, kd, r, yp, xp;
             int zz, yy, xx;
@@ -147,6 +149,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
             }
             if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W) {
                 goff[i] = gchk[i] = (unsigned)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh)) * 4u;
+                inb[i] = true;
             }
         }
     }
@@ -182,6 +185,10 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 #pragma unroll
         for (int i = 0; i < NX; i++) r.rx[i] = *(const float*)(xsrc + goff[i]);
     };
+    // An element that is padding is padding in every chunk: its LDS slots are zeroed once per tile (zero_padding) and
+    // a chunk's store skips it under the lane mask `inb` (kept in scalar registers: no vector instruction per element,
+    // where a select of the value against zero cost two).  Only a partial last chunk still selects: its channels past
+    // the last one store zeros.
     auto store_chunk = [&](const Regs& r, int buf, int ch) {
         cm_v4f* wdst = (cm_v4f*)(sW + buf * WCH);
 #pragma unroll
@@ -190,11 +197,23 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
             if (f4 < WCH / 4) wdst[f4] = r.rw[i];
         }
         float* xdst = sX + buf * XCHP + tid;
-        const unsigned lim = chunk_lim(ch);
-        const int el0 = st_u(tid & ~63);          // the wave's first element of round 0: the bound check is per wave
+        if ((ch + 1) * CC <= s.C) {
 #pragma unroll
-        for (int i = 0; i < NX; i++)
-            if (i * CM_THREADS + el0 < XCHP) xdst[i * CM_THREADS] = gchk[i] < lim ? r.rx[i] : 0.f;
+            for (int i = 0; i < NX; i++)
+                if (inb[i]) xdst[i * CM_THREADS] = r.rx[i];
+        } else {
+            const unsigned lim = chunk_lim(ch);
+#pragma unroll
+            for (int i = 0; i < NX; i++)
+                if (inb[i]) xdst[i * CM_THREADS] = gchk[i] < lim ? r.rx[i] : 0.f;
+        }
+    };
+    auto zero_padding = [&]() {
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < NX; i++)
+                if (!inb[i] && tid + i * CM_THREADS < XCHP) sX[b * XCHP + tid + i * CM_THREADS] = 0.f;
     };
 
     const int kgi = wave % KG, wtile = wave / KG;                 // channel group; the wave's tile among the workgroup's
@@ -249,6 +268,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         cm_lds_barrier();
     };
     load_chunk(rg[0], ch0);
+    zero_padding();
     store_chunk(rg[0], 0, ch0);
     cm_lds_barrier();
     load_chunk(rg[1], ch0 + 1 < ch1 ? ch0 + 1 : ch0);     // unconditional for the same reason (a lone chunk is fetched twice)
