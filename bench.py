@@ -33,7 +33,7 @@ MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((1114.1 * 2 + 
                     "zb_unfused_1028x1028x15_f64": int((247386.7 * 2 + 1658898.9) * 1024),
                     # conv workloads: every conv, split-reduce and thin-head dispatch of a step summed, divided by the
                     # step's conv operations (18 and 19), like flop_per_launch
-                    "unet": int((1130192.0 * 2 + 544769.0) * 1024 / 7 / 18), "tsrgan": int((3431145.0 * 2 + 5032349.0) * 1024 / 7 / 19)}
+                    "unet": int((1131516.0 * 2 + 544769.0) * 1024 / 7 / 18), "tsrgan": int((3423671.0 * 2 + 5019823.0) * 1024 / 7 / 19)}
 
 
 def omp_threads():

@@ -176,9 +176,9 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         if ((ch + 1) * CC > s.C) {
             // partial last chunk: channels past the last one read offset 0 too.  It is the last chunk this tile loads,
             // so the offsets are clamped in place (one load site; a second one with clamped copies cost every chunk a
-            // move per offset where the two join); the empty asm keeps this a branch
-            asm volatile("" ::: "memory");
-            const unsigned lim = chunk_lim(ch);
+            // move per offset where the two join)
+            unsigned lim = chunk_lim(ch);
+            asm volatile("" : "+s"(lim));            // opaque here: the clamps below cannot be hoisted out of the branch
 #pragma unroll
             for (int i = 0; i < NX; i++) goff[i] = goff[i] < lim ? goff[i] : 0u;
         }
