@@ -545,11 +545,11 @@ def run_workload(L, args, workload):
 OTHERS = [("toy 1024x(64-256-256-32)", "toy", None, 200, 50),
           ("zb 68x78x15 fused, 27-64-64-3", "zb", None, 200, 50),
           ("zb 68x78x15 fused, reference net 27-20-3", "zb_ref", None, 200, 50),
-          ("zb 1028x1028x15 fused, 27-64-64-3", "zb", "1028x1028x15", 10, 3),
-          ("zb 1028x1028x15 fused, reference net 27-20-3", "zb_ref", "1028x1028x15", 10, 3),
-          ("zb 1028x1028x15 unfused (gather kernel is the roofline)", "zb_unfused", "1028x1028x15", 10, 3),
-          ("unet 1x4x256x256", "unet", None, 50, 20),
-          ("tsrgan 33^3 -> 66^3", "tsrgan", None, 20, 10)]
+          ("zb 1028x1028x15 fused, 27-64-64-3", "zb", "1028x1028x15", 40, 20),
+          ("zb 1028x1028x15 fused, reference net 27-20-3", "zb_ref", "1028x1028x15", 40, 20),
+          ("zb 1028x1028x15 unfused (gather kernel is the roofline)", "zb_unfused", "1028x1028x15", 20, 10),
+          ("unet 1x4x256x256", "unet", None, 100, 30),
+          ("tsrgan 33^3 -> 66^3", "tsrgan", None, 40, 15)]
 
 
 def run_others(L, args):
