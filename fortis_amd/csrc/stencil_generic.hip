@@ -99,6 +99,27 @@ __device__ __forceinline__ void sg_apply(float* mine, int n, bool left, double c
     else for (int q = 0; q < n; q++) mine[q] = (float)f(c, (double)mine[q]);
 }
 
+// fp64 division of fp32 slot values by one divisor: the compiler's sequence (v_div_scale_f64 of both operands,
+// v_rcp_f64 with two Newton steps, quotient, residual, v_div_fmas_f64, v_div_fixup_f64) neither scales nor fixes
+// anything up when the numerators are finite non-zero floats (as doubles their exponents lie in [-149, 127]) and the
+// divisor's exponent lies in [-400, 400]: no operand, reciprocal or quotient comes near the ends of the double range.
+// A numerator of +0 also comes out right through the short form (0 * r carries the quotient's sign, the residual is
+// +0); -0 does not (the last fma adds zeros of opposite sign) and goes the long way with infinities and NaNs.
+// True when the short form holds for every active lane of the wave.
+__device__ __forceinline__ bool sg_div_wave_in_range(const float* mine, int n, double c)
+{
+    const unsigned ce = ((unsigned)(__double_as_longlong(c) >> 52)) & 0x7ffu;
+    unsigned lo = 0xffffffffu, hi = 0;
+    for (int q = 0; q < n; q++) {
+        // sign rotated to the bottom and flipped: -0 -> 0, +0 -> 1, infinities and NaNs -> 0xff000000 and above
+        const unsigned k = __builtin_rotateleft32(__float_as_uint(mine[q]), 1) ^ 1u;
+        lo = k < lo ? k : lo;
+        hi = k > hi ? k : hi;
+    }
+    const bool out = ce < 1023u - 400u || ce > 1023u + 400u || lo == 0u || hi >= 0xff000000u;
+    return __builtin_amdgcn_ballot_w64(out) == 0;
+}
+
 // One step of the chain form on all n slot values of the row: the operator is decoded once, not once per slot.
 // Same arithmetic as sg_eval: operands as doubles, an fp32 operation converts them to float first.
 __device__ __forceinline__ void sg_chain_step(int opw, bool left, double c, float* mine, int n)
@@ -118,7 +139,18 @@ __device__ __forceinline__ void sg_chain_step(int opw, bool left, double c, floa
             else sg_apply(mine, n, left, c, [](double x, double y) { return (double)__fmul_rn((float)x, (float)y); });
             break;
         case FORTIS_OP_DIV:
-            if (f64) sg_apply(mine, n, left, c, [](double x, double y) { return __ddiv_rn(x, y); });
+            if (f64 && left && sg_div_wave_in_range(mine, n, c)) {
+                // every slot value of the row over the same divisor, all operands clear of the ranges in which the
+                // IEEE sequence would scale or fix up (see sg_div_wave_in_range): its reciprocal and two Newton steps
+                // once per row, then a multiply and two fmas per slot -- the same operations, hence the same bits
+                double r = __builtin_amdgcn_rcp(c);
+                r = __fma_rn(r, __fma_rn(-c, r, 1.0), r);
+                r = __fma_rn(r, __fma_rn(-c, r, 1.0), r);
+                for (int q = 0; q < n; q++) {
+                    const double x = (double)mine[q], q0 = __dmul_rn(x, r);
+                    mine[q] = (float)__fma_rn(__fma_rn(-c, q0, x), r, q0);
+                }
+            } else if (f64) sg_apply(mine, n, left, c, [](double x, double y) { return __ddiv_rn(x, y); });
             else sg_apply(mine, n, left, c, [](double x, double y) { return (double)__fdiv_rn((float)x, (float)y); });
             break;
         case FORTIS_OP_MAX: sg_apply(mine, n, left, c, [](double x, double y) { return (double)fmaxf((float)x, (float)y); }); break;

@@ -90,6 +90,32 @@ def test_general_gather_bit_exact(L, gpu, exprs, g64):
         assert not bits_equal(ref32, ref)
 
 
+def test_fp64_division_with_operands_at_the_ends_of_the_range(L, gpu):
+    """tv / S0 with S0 an fp64 array: the general gather divides a row's slot values by one double.  Numerators of
+    either zero, infinities, NaNs, denormals and the largest floats, and divisors that are zero, infinite, NaN,
+    denormal or beyond 2^+-400, sprinkled over otherwise ordinary data, must give the bits of an IEEE double
+    division rounded to float, whichever way a row's division is carried out."""
+    gd, sd, lp, kd, garr, _ = _case(gexprs=["(tv / S0)"], g64=(3,))
+    rng = np.random.default_rng(23)
+    xs = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1e-39, 3.4028235e38, -3.4028235e38, 1.1754944e-38], np.float32)
+    cs = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 5e-324, 1e-310, 1e-200, -1e-200, 1e200, -1e200, 1.7e308,
+                   2.0 ** -400, 2.0 ** 400, 2.0 ** -401, 2.0 ** 401, -3.0, 1e-30, 1e30], np.float64)
+    for a in garr[:3]:
+        at = rng.random(a.size) < 0.02
+        a[at] = rng.choice(xs, at.sum())
+        pz = rng.random(a.size) < 0.05                          # +0 alone is common (masked cells) and stays on the short form
+        a[pz] = 0.0
+    at = rng.random(garr[3].size) < 0.15
+    garr[3][at] = rng.choice(cs, at.sum())
+    with np.errstate(all="ignore"):
+        ref = O.stencil_gather_typed(gd, garr, COUNT, NZ, 3, 3, SX - 4)
+    X = _gather(L, gd, lp, kd, garr)
+    same = (X.view(np.uint32) == ref.view(np.uint32)) | (np.isnan(X) & np.isnan(ref))
+    assert same.all()
+    fin = np.isfinite(ref)
+    assert 0.3 < fin.mean() < 0.99 and (ref == 0).sum() > 100 and np.signbit(ref[ref == 0]).any()
+
+
 @pytest.mark.parametrize("g64", [(), (1, 3)])
 def test_wide_stencil_and_long_expression(L, gpu, g64):
     """A 5 x 5 neighbourhood of three arrays (75 slots) with a 21-operation expression: more slots than one
