@@ -387,29 +387,37 @@ __global__ __launch_bounds__(CM_THREADS) void conv_sk_reduce_kernel(float* __res
     const int first = tl * s.nchunks, w0 = first / s.sk_per, nseg = (first + s.nchunks - 1) / s.sk_per - w0 + 1;
     const long slot = (long)gridDim.x * gridDim.y * (NQ * CM_THREADS);
     const cm_v4f* p = (const cm_v4f*)s.part + (((long)fg * gridDim.x + tl) * NQ + rq) * CM_THREADS + tid;
-    cm_v4f acc = *p;
-    for (int k = 1; k < nseg; k++) {
-        p += slot;
-        acc += *p;
-    }
+    // a thread's loads all leave before the first is needed: the first four slots (a tile always has two) and the
+    // residual values; the sums are then added in slot order
+    const cm_v4f a0 = p[0], a1 = p[slot];
+    const cm_v4f a2 = p[nseg > 2 ? 2 * slot : 0], a3 = p[nseg > 3 ? 3 * slot : 0];
     const int bx = tl + s.sk_tile0, z = bx / s.tiles, tile = bx - z * s.tiles;
     const int ft = wave % FW, mt0 = (wave / FW) * NMT;
     const long ospatial = (long)s.D * s.H * s.W;
     const int m = tile * MT + (mt0 + rq / 4) * 32 + (lane & 31);
     unsigned yy, xx;
     st_divmod((unsigned)m, s.mP, yy, xx);
-    if (m >= s.plane || (int)xx >= s.W) return;
-    const long opos = ((long)z * s.H + yy) * s.W + xx;
+    const bool inside = m < s.plane && (int)xx < s.W;
+    const long opos = inside ? ((long)z * s.H + yy) * s.W + xx : 0;
+    const int f0 = fg * FT + ft * 32 + 8 * (rq & 3) + 4 * (lane >> 5);             // registers 4 * (rq & 3) ... + 3 of the m-tile
+    float res[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) res[q] = e.res && f0 + q < s.F ? e.res[(f0 + q) * ospatial + opos] : 0.f;
+    cm_v4f acc = a0 + a1;
+    if (nseg > 2) acc += a2;
+    if (nseg > 3) acc += a3;
+    for (int k = 4; k < nseg; k++) acc += p[k * slot];
+    if (!inside) return;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        const int f = fg * FT + ft * 32 + 8 * (rq & 3) + 4 * (lane >> 5) + q;      // register 4 * (rq & 3) + q of the m-tile
+        const int f = f0 + q;
         if (f >= s.F) continue;
         float v = acc[q];
         if (e.scale) v = v * e.scale[f];
         if (e.shift) v = v + e.shift[f];
         if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
         else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
-        if (e.res) v = v + e.res[f * ospatial + opos];
+        if (e.res) v = v + res[q];
         y[f * ospatial + opos] = v;
     }
 }
