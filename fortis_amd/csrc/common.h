@@ -94,6 +94,7 @@ void fortis_launch_scatter_generic(const fortis_stencil_t& t, const int* dcells,
 // ---- elementwise / layout kernels (elementwise.hip) --------------------------------------
 void fortis_launch_scale(const float* src, float* dst, const float* vec, long rows, long n, int divide, hipStream_t s);
 void fortis_launch_mask_relu(const float* src, float* dst, long rows, long n, long tail, hipStream_t s);
+void fortis_launch_zero(float* dst, long n, hipStream_t s);
 void fortis_launch_boundary_pre(const void* A, float* X, long NI, long NK, const void* mean, const void* vmax,
                                 const void* vmin, int host_esz, hipStream_t s);
 void fortis_launch_boundary_post(const float* Y, void* B, long NI, long NK, const void* scale, int host_esz, hipStream_t s);

@@ -32,6 +32,18 @@ __global__ void mask_relu_kernel(const float* __restrict__ src, float* __restric
     const float v = src[idx];
     dst[idx] = (idx % n >= n - tail && v < 0.f) ? 0.f : v;
 }
+// dst[0 .. n) = 0 as a kernel: a memset node recorded into a captured graph is not replayed reliably here.
+__global__ void zero_kernel(float* __restrict__ dst, long n)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < n) dst[idx] = 0.f;
+}
+void fortis_launch_zero(float* dst, long n, hipStream_t s)
+{
+    if (n <= 0) return;
+    hipLaunchKernelGGL(zero_kernel, dim3((unsigned)cdiv(n, EW_THREADS)), dim3(EW_THREADS), 0, s, dst, n);
+    HIP_OK(hipGetLastError());
+}
 void fortis_launch_mask_relu(const float* src, float* dst, long rows, long n, long tail, hipStream_t s)
 {
     const long total = rows * n;

@@ -136,6 +136,10 @@ void fortis_gemm(float* Aa, float* A, long Ao, long As0, long As1, long At0, lon
 {
     (void)Aa; (void)As0; (void)As1; (void)At0; (void)At1; (void)Wa; (void)Ws0; (void)Ws1; (void)Wt0; (void)Wt1;
     (void)Ca; (void)Cs0; (void)Cs1; (void)Ct0; (void)Ct1;
+    // Empty problems as the reference's SGEMM call treats them (runtime/fortis_rt.c:69-74, beta = 0): no rows or no
+    // columns, nothing happens; no k, the sum is empty and C becomes zero.
+    if (B <= 0 || N <= 0 || K < 0) return;
+    if (K == 0) { fortis_launch_zero(C + Co, B * N, fortis_stream_get()); return; }
     if (fortis_launch_gemm(A + Ao, W + Wo, nullptr, C + Co, B, N, K, FORTIS_ACT_NONE, 0.f, nullptr, 0, fortis_stream_get()) != 0)
         fprintf(stderr, "fortis_gemm: unsupported shape B%ld N%ld K%ld\n", B, N, K);
 }

@@ -161,6 +161,22 @@ def test_fortis_gemm_entry(L, gpu, B, N, K):
         d.free()
 
 
+def test_fortis_gemm_entry_empty_problems(L, gpu, capfd):
+    """B = 0 or N = 0: nothing is written and nothing is printed; K = 0: the empty sum, C = 0 (what the reference's
+    SGEMM call with beta = 0 does, runtime/fortis_rt.c:69-74)."""
+    Cin = np.full(6 * 5, 7.0, np.float32)
+    dA, dW, dC = DevBuf(L, np.ones(64, np.float32)), DevBuf(L, np.ones(64, np.float32)), DevBuf(L, Cin)
+    for B, N, K in ((0, 5, 4), (6, 0, 4)):
+        L.fortis_gemm(dA.ptr, dA.ptr, 0, B, K, K, 1, dW.ptr, dW.ptr, 0, N, K, K, 1, dC.ptr, dC.ptr, 0, B, N, N, 1, B, N, K)
+        assert np.array_equal(dC.get((30,)), Cin)
+    L.fortis_gemm(dA.ptr, dA.ptr, 0, 4, 0, 0, 1, dW.ptr, dW.ptr, 0, 5, 0, 0, 1, dC.ptr, dC.ptr, 0, 4, 5, 5, 1, 4, 5, 0)
+    got = dC.get((30,))
+    assert np.array_equal(got[:20], np.zeros(20, np.float32)) and np.array_equal(got[20:], Cin[20:])
+    assert "fortis" not in capfd.readouterr().err
+    for d in (dA, dW, dC):
+        d.free()
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("NI,NK", [(384, 124), (50, 33), (1, 1)])
 def test_boundary_pre_post_bit_exact(L, gpu, dtype, NI, NK):
