@@ -124,6 +124,21 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     const int sh = s.ups ? 1 : 0;
     const long srcW = s.W >> sh, sHW = (long)(s.H >> sh) * srcW, schan = (long)(s.D >> sh) * sHW;
 
+    // Two register sets: while LDS holds chunk k, set (k+1)&1 carries chunk k+1 (loaded one step ago) and
+    // set k&1 receives chunk k+2, so a chunk's global loads have two multiply phases to arrive in.
+    struct Regs { cm_v4f rw[NW]; float rx[NX]; };
+    Regs rg[2];
+    auto load_weights = [&](Regs& r, int ch) {
+        const cm_v4f* wsrc = (const cm_v4f*)(wp + ((long)fg * s.nchunks + ch) * WCH);
+#pragma unroll
+        for (int i = 0; i < NW; i++) {
+            const int f4 = tid + i * CM_THREADS;
+            r.rw[i] = wsrc[f4 < WCH / 4 ? f4 : 0];
+        }
+    };
+    // the first chunk's weights need nothing of the staging map below: they are on their way while it is worked out
+    load_weights(rg[0], ch0);
+
     // per-thread staging map of the input run (same for every chunk): byte offset inside a chunk's channel
     // group, (c * schan + offset in the channel) * 4.  Padding elements load from offset 0 (goff) and carry
     // the mark 0xffffffff in gchk, which the store compares with the chunk's limit.
@@ -159,17 +174,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         const int cleft = s.C - ch * CC;
         return (unsigned)((cleft < CC ? cleft : CC) * schan) * 4u;
     };
-    // Two register sets: while LDS holds chunk k, set (k+1)&1 carries chunk k+1 (loaded one step ago) and
-    // set k&1 receives chunk k+2, so a chunk's global loads have two multiply phases to arrive in.
-    struct Regs { cm_v4f rw[NW]; float rx[NX]; };
-    Regs rg[2];
-    auto load_chunk = [&](Regs& r, int ch) {
-        const cm_v4f* wsrc = (const cm_v4f*)(wp + ((long)fg * s.nchunks + ch) * WCH);
-#pragma unroll
-        for (int i = 0; i < NW; i++) {
-            const int f4 = tid + i * CM_THREADS;
-            r.rw[i] = wsrc[f4 < WCH / 4 ? f4 : 0];
-        }
+    auto load_input = [&](Regs& r, int ch) {
         // uniform base + 32-bit byte offset per lane: no address arithmetic here.  Padding elements read
         // offset 0 (a valid address); they are replaced by zero only when stored, so nothing waits here.
         const char* xsrc = (const char*)(x + (long)ch * CC * schan);
@@ -185,6 +190,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 #pragma unroll
         for (int i = 0; i < NX; i++) r.rx[i] = *(const float*)(xsrc + goff[i]);
     };
+    auto load_chunk = [&](Regs& r, int ch) { load_weights(r, ch); load_input(r, ch); };
     // An element that is padding is padding in every chunk: its LDS slots are zeroed once per tile (zero_padding) and
     // a chunk's store skips it under the lane mask `inb` (kept in scalar registers: no vector instruction per element,
     // where a select of the value against zero cost two).  Only a partial last chunk still selects: its channels past
@@ -267,7 +273,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         if (ch + 1 < ch1) store_chunk(near, buf ^ 1, ch + 1);
         cm_lds_barrier();
     };
-    load_chunk(rg[0], ch0);
+    load_input(rg[0], ch0);
     zero_padding();
     store_chunk(rg[0], 0, ch0);
     cm_lds_barrier();
