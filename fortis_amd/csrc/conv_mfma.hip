@@ -153,7 +153,15 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         if (el < XCH) {
             unsigned c, rem, kd, r, yp, xp;
             int zz, yy, xx;
-            if (TILE2D) {
+            if constexpr (KD == 1 && KS == 1) {
+                // a 1 x 1 conv stages MT consecutive positions of each channel: no borders, no row structure
+                c = (unsigned)el / MT; r = (unsigned)el % MT;
+                if (m0 + (int)r < s.plane) {
+                    goff[i] = gchk[i] = (unsigned)(c * schan + m0 + r) * 4u;
+                    inb[i] = true;
+                }
+                continue;
+            } else if (TILE2D) {
                 c = (unsigned)el / R2; r = (unsigned)el % R2;    // compile-time divisors
                 zz = z; yy = y0 + (int)(r / CM_TP) - 1; xx = x0 + (int)(r % CM_TP) - 1;
             } else {
@@ -832,7 +840,7 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
     s.mode = kind == 1 ? 1 : 0;
     s.ksplit = 1;
     s.ups = kind == 2 ? 1 : 0;
-    if (kind == 2 && ((D | H | Wd) & 1)) return -1;
+    if (kind == 2 && (KD != 3 || ((D | H | Wd) & 1))) return -1;     // the fused upsample is a form of the volume kernel
     if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 2) {
         if (KS == 1) {
             s.P = s.W;
