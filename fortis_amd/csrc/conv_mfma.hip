@@ -19,6 +19,7 @@
 // On wide 2-D images that run is mostly halo (two whole rows for one tile's worth of positions), so 3 x 3
 // convs on images at least 64 wide use a second tiling (TILE2D): a workgroup's positions are MT / 32 rows of
 // 32 columns, staged with a one-pixel border at a fixed pitch of 34, tap (kh, kw) = element + kh*34 + kw.
+#include <type_traits>
 #include "stencil_dev.h"      // StMagic / st_divmod: exact division by a launch constant
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -298,36 +299,84 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 
     // epilogue: a lane holds one position and 16 output channels per m-tile
     const long ospatial = s.mode ? 4 * chan : chan;
-    auto finish = [&](const int j, const int r, float v) __attribute__((always_inline)) {
+    // Registers r0 .. r0 + N - 1 of m-tile j at once.  Every step of the epilogue runs over all of them before the next
+    // begins (a step's loads, from addresses clamped into the tensors, leave together and are waited for once; the
+    // null checks of the epilogue's pointers are taken once, not per element).  Per element the operations and their
+    // order are those of the reference's fused epilogue: scale, shift, activation, residual.
+    auto finish_regs = [&](const int j, const int r0, auto nc, float* v) __attribute__((always_inline)) {
+        constexpr int N = decltype(nc)::value;
         unsigned yy, xx;
+        bool inside;
         if (TILE2D) {
             yy = (unsigned)(y0 + mt0 + j); xx = (unsigned)(x0 + (lane & 31));
-            if ((int)yy >= s.H) return;
+            inside = (int)yy < s.H;
         } else {
             const int m = m0 + (mt0 + j) * 32 + (lane & 31);
-            if (m >= s.plane) return;
-            st_divmod((unsigned)m, s.mP, yy, xx);
+            inside = m < s.plane;
+            st_divmod((unsigned)(inside ? m : 0), s.mP, yy, xx);
         }
-        if ((int)xx >= s.W) return;
-        const int f = fg * FT + ft * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (f >= s.F) return;
-        int fo = f;
-        long opos = ((long)z * s.H + yy) * s.W + xx;
-        if (s.mode) {
-            fo = f >> 2;
-            opos = (long)(2 * yy + ((f >> 1) & 1)) * (2 * s.W) + 2 * xx + (f & 1);
+        inside = inside && (int)xx < s.W;
+        if (!inside) { yy = 0; xx = 0; }
+        const int fb = fg * FT + ft * 32 + 4 * (lane >> 5);
+        const unsigned opos = (unsigned)(((long)z * s.H + yy) * s.W + xx);
+        int fo[N];
+        unsigned off[N];             // element offsets: the launcher keeps every tensor below 2^31 elements
+        bool ok[N];
+#pragma unroll
+        for (int q = 0; q < N; q++) {
+            const int r = r0 + q, f = fb + 8 * (r >> 2) + (r & 3);
+            ok[q] = inside && f < s.F;
+            const int fc = f < s.F ? f : 0;
+            if (s.mode) {
+                fo[q] = fc >> 2;
+                off[q] = (unsigned)(fo[q] * ospatial) + (2 * yy + ((fc >> 1) & 1)) * (2 * s.W) + 2 * xx + (fc & 1);
+            } else {
+                fo[q] = fc;
+                off[q] = (unsigned)(fc * ospatial) + opos;
+            }
         }
-        if (s.ksplit > 1) { s.part[blockIdx.z * s.osize + fo * ospatial + opos] = v; return; }
-        if (e.scale) v = v * e.scale[fo];
-        if (e.shift) v = v + e.shift[fo];
-        if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
-        else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
-        if (e.res) v = v + e.res[fo * ospatial + opos];
-        y[fo * ospatial + opos] = v;
-        if constexpr (POOL) {
-            // the finished tile also goes to LDS as [channel][row][32 columns] for the 2 x 2 max pool below
-            // (behind the channel groups' sums, which other waves may still be reading)
-            ((float*)smem4)[(KG > 1 ? 4 * 16 * 64 : 0) + ((f - fg * FT) * TH + (mt0 + j)) * 32 + (lane & 31)] = v;
+        if (s.ksplit > 1) {
+            float* part = s.part + blockIdx.z * s.osize;
+#pragma unroll
+            for (int q = 0; q < N; q++) if (ok[q]) part[off[q]] = v[q];
+            return;
+        }
+        float t[N];
+        if (e.scale) {
+#pragma unroll
+            for (int q = 0; q < N; q++) t[q] = e.scale[fo[q]];
+#pragma unroll
+            for (int q = 0; q < N; q++) v[q] = v[q] * t[q];
+        }
+        if (e.shift) {
+#pragma unroll
+            for (int q = 0; q < N; q++) t[q] = e.shift[fo[q]];
+#pragma unroll
+            for (int q = 0; q < N; q++) v[q] = v[q] + t[q];
+        }
+        if (e.act == FORTIS_ACT_RELU) {
+#pragma unroll
+            for (int q = 0; q < N; q++) v[q] = v[q] > 0.f ? v[q] : 0.f;
+        } else if (e.act == FORTIS_ACT_LEAKY) {
+#pragma unroll
+            for (int q = 0; q < N; q++) v[q] = v[q] > 0.f ? v[q] : e.alpha * v[q];
+        }
+        if (e.res) {
+#pragma unroll
+            for (int q = 0; q < N; q++) t[q] = e.res[off[q]];
+#pragma unroll
+            for (int q = 0; q < N; q++) v[q] = v[q] + t[q];
+        }
+#pragma unroll
+        for (int q = 0; q < N; q++) {
+            if (!ok[q]) continue;
+            y[off[q]] = v[q];
+            if constexpr (POOL) {
+                // the finished tile also goes to LDS as [channel][row][32 columns] for the 2 x 2 max pool below
+                // (behind the channel groups' sums, which other waves may still be reading)
+                const int r = r0 + q, f = fb + 8 * (r >> 2) + (r & 3);
+                ((float*)smem4)[(KG > 1 ? 4 * 16 * 64 : 0) + ((f - fg * FT) * TH + (mt0 + j)) * 32 + (lane & 31)] = v[q];
+            }
         }
     };
     // 2 x 2 stride-2 max pool of the finished tile (H and W even, tiles start on even rows and columns: a 2 x 2
@@ -363,10 +412,18 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         it += ch1 - ch0;
         continue;
     } else if constexpr (KG == 1) {
+        // registers finished at a time: all 16 of an m-tile, or 4 in the form that keeps four workgroups on a CU
+        // (its 128 registers have no room for 16 offsets and 16 loaded values beside the accumulators)
+        constexpr int EN = (KD == 3 && MT == 128 && FT == 64 && NX <= 8) ? 4 : 16;
 #pragma unroll
         for (int j = 0; j < NMT; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) finish(j, r, acc[j][r]);
+            for (int r0 = 0; r0 < 16; r0 += EN) {
+                float v[EN];
+#pragma unroll
+                for (int q = 0; q < EN; q++) v[q] = acc[j][r0 + q];
+                finish_regs(j, r0, std::integral_constant<int, EN>(), v);
+            }
         if constexpr (POOL) pool_tile();
     } else {
         // the loop above ended on a barrier: the staging buffers are free.  red[tile][group][register][lane]
@@ -375,14 +432,15 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         for (int r = 0; r < 16; r++) red[(kgi * 16 + r) * 64 + lane] = acc[0][r];
         cm_lds_barrier();
         // group g finishes registers g * 16 / KG ...: the groups' sums are added in group order
+        float v[16 / KG];
 #pragma unroll
         for (int q = 0; q < 16 / KG; q++) {
             const int r = kgi * (16 / KG) + q;
-            float v = red[r * 64 + lane];
+            v[q] = red[r * 64 + lane];
 #pragma unroll
-            for (int g = 1; g < KG; g++) v += red[(g * 16 + r) * 64 + lane];
-            finish(0, r, v);
+            for (int g = 1; g < KG; g++) v[q] += red[(g * 16 + r) * 64 + lane];
         }
+        finish_regs(0, kgi * (16 / KG), std::integral_constant<int, 16 / KG>(), v);
         if constexpr (POOL) pool_tile();
     }
     break;
