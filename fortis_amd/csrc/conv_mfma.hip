@@ -45,6 +45,7 @@ struct ConvMShape {
     int ups;                   // 1: the input tensor is (D/2, H/2, W/2) and is read through a nearest x2 upsample
     long osize;                // output elements
     StMagic mP, mR, mKR;       // exact division by P, R and KD * R (the staging map would otherwise spend its time dividing)
+    StMagic mT, mTX, mNC, mPer; // ... by tiles, tiles_x, nchunks and sk_per (a scalar division costs some forty instructions at the head of every workgroup)
 };
 
 // FT output channels per workgroup: 64 (waves 2 x 2 over channels x positions) or 32 (4 waves over positions).
@@ -108,18 +109,22 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     int bx = wgx, ch0, ch1;
     if constexpr (SK) {
         if (it >= itend) break;
-        bx = it / s.nchunks;
-        ch0 = it - bx * s.nchunks;
-        bx += s.sk_tile0;
+        unsigned tq, cq;
+        st_divmod((unsigned)it, s.mNC, tq, cq);
+        bx = (int)tq + s.sk_tile0;
+        ch0 = (int)cq;
         ch1 = ch0 + (itend - it) < s.nchunks ? ch0 + (itend - it) : s.nchunks;
     } else {
         const int kz = blockIdx.z;
         ch0 = kz * s.cbase + (kz < s.cextra ? kz : s.cextra);
         ch1 = ch0 + s.cbase + (kz < s.cextra ? 1 : 0);
     }
-    const int z = bx / s.tiles, tile = bx - z * s.tiles;
+    unsigned zq = 0, tileq = (unsigned)bx, tyq = 0, txq = 0;
+    if constexpr (KD != 1) st_divmod((unsigned)bx, s.mT, zq, tileq);          // images have one plane (the launcher sees to it)
+    if constexpr (TILE2D) st_divmod(tileq, s.mTX, tyq, txq);
+    const int z = (int)zq, tile = (int)tileq;
     const int m0 = tile * MT;
-    const int tyi = TILE2D ? tile / s.tiles_x : 0, y0 = tyi * TH, x0 = (tile - tyi * s.tiles_x) * 32;   // TILE2D: tile origin
+    const int tyi = (int)tyq, y0 = tyi * TH, x0 = (int)txq * 32;               // TILE2D: tile origin
     const long HW = (long)s.H * s.W, chan = (long)s.D * HW;
     // source geometry: the tensor itself, or the half-resolution tensor a fused nearest upsample reads
     const int sh = s.ups ? 1 : 0;
@@ -147,22 +152,20 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     bool inb[NX];                // the element lies inside the tensor (not padding, not past the staged run)
 #pragma unroll
     for (int i = 0; i < NX; i++) {
+        // straight-line: an element past the staged run or outside the tensor works its numbers out like any other
+        // (nothing is read with them) and is switched off at the end
         const int el = tid + i * CM_THREADS;
-        goff[i] = 0;
-        gchk[i] = 0xffffffffu;
-        inb[i] = false;
-        if (el < XCH) {
-            unsigned c, rem, kd, r, yp, xp;
+        unsigned c, r, off;
+        bool in = el < XCH;
+        if constexpr (KD == 1 && KS == 1) {
+            // a 1 x 1 conv stages MT consecutive positions of each channel: no borders, no row structure
+            c = (unsigned)el / MT; r = (unsigned)el % MT;
+            in = in && m0 + (int)r < s.plane;
+            off = (unsigned)(c * schan + m0 + r) * 4u;
+        } else {
+            unsigned rem, kd, yp, xp;
             int zz, yy, xx;
-            if constexpr (KD == 1 && KS == 1) {
-                // a 1 x 1 conv stages MT consecutive positions of each channel: no borders, no row structure
-                c = (unsigned)el / MT; r = (unsigned)el % MT;
-                if (m0 + (int)r < s.plane) {
-                    goff[i] = gchk[i] = (unsigned)(c * schan + m0 + r) * 4u;
-                    inb[i] = true;
-                }
-                continue;
-            } else if (TILE2D) {
+            if (TILE2D) {
                 c = (unsigned)el / R2; r = (unsigned)el % R2;    // compile-time divisors
                 zz = z; yy = y0 + (int)(r / CM_TP) - 1; xx = x0 + (int)(r % CM_TP) - 1;
             } else {
@@ -171,11 +174,12 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                 st_divmod((unsigned)(m0 + r), s.mP, yp, xp);
                 zz = z + (int)kd - (KD / 2); yy = (int)yp - PADK; xx = (int)xp - PADK;
             }
-            if (zz >= 0 && zz < s.D && yy >= 0 && yy < s.H && xx >= 0 && xx < s.W) {
-                goff[i] = gchk[i] = (unsigned)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh)) * 4u;
-                inb[i] = true;
-            }
+            in = in & ((unsigned)zz < (unsigned)s.D) & ((unsigned)yy < (unsigned)s.H) & ((unsigned)xx < (unsigned)s.W);
+            off = (unsigned)(c * schan + (zz >> sh) * sHW + (long)(yy >> sh) * srcW + (xx >> sh)) * 4u;
         }
+        goff[i] = in ? off : 0u;
+        gchk[i] = in ? off : 0xffffffffu;
+        inb[i] = in;
     }
 
     // byte offsets at or beyond chunk_lim belong to channels past the last one (only in a partial last chunk)
@@ -399,7 +403,10 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     static_assert(!POOL || (TILE2D && (MT / 32) % 2 == 0), "the in-kernel pool needs the 32-column tiling and an even tile height");
     if constexpr (SK) {
         // the accumulators as they are: slot = this workgroup's rank among those whose runs share the tile
-        const int tl = bx - s.sk_tile0, slot = wgx - (tl * s.nchunks) / s.sk_per;
+        const int tl = bx - s.sk_tile0;
+        unsigned w0q, rr;
+        st_divmod((unsigned)(tl * s.nchunks), s.mPer, w0q, rr);
+        const int slot = wgx - (int)w0q;
         cm_v4f* pd = (cm_v4f*)s.part + (((long)slot * gridDim.y + fg) * (s.D * s.tiles - s.sk_tile0) + tl) * (NMT * 4 * CM_THREADS) + tid;
 #pragma unroll
         for (int j = 0; j < NMT; j++)
@@ -456,14 +463,20 @@ __global__ __launch_bounds__(CM_THREADS) void conv_sk_reduce_kernel(float* __res
 {
     constexpr int FW = FT / 32, NMT = MT / 32 / (4 / FW), NQ = NMT * 4;
     const int tl = blockIdx.x, fg = blockIdx.y, rq = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int first = tl * s.nchunks, w0 = first / s.sk_per, nseg = (first + s.nchunks - 1) / s.sk_per - w0 + 1;
+    const int first = tl * s.nchunks;
+    unsigned w0q, w1q, rr;
+    st_divmod((unsigned)first, s.mPer, w0q, rr);
+    st_divmod((unsigned)(first + s.nchunks - 1), s.mPer, w1q, rr);
+    const int nseg = (int)(w1q - w0q) + 1;
     const long slot = (long)gridDim.x * gridDim.y * (NQ * CM_THREADS);
     const cm_v4f* p = (const cm_v4f*)s.part + (((long)fg * gridDim.x + tl) * NQ + rq) * CM_THREADS + tid;
     // a thread's loads all leave before the first is needed: the first four slots (a tile always has two) and the
     // residual values; the sums are then added in slot order
     const cm_v4f a0 = p[0], a1 = p[slot];
     const cm_v4f a2 = p[nseg > 2 ? 2 * slot : 0], a3 = p[nseg > 3 ? 3 * slot : 0];
-    const int bx = tl + s.sk_tile0, z = bx / s.tiles, tile = bx - z * s.tiles;
+    unsigned zq, tileq;
+    st_divmod((unsigned)(tl + s.sk_tile0), s.mT, zq, tileq);
+    const int z = (int)zq, tile = (int)tileq;
     const int ft = wave % FW, mt0 = (wave / FW) * NMT;
     const long ospatial = (long)s.D * s.H * s.W;
     const int m = tile * MT + (mt0 + rq / 4) * 32 + (lane & 31);
@@ -472,9 +485,14 @@ __global__ __launch_bounds__(CM_THREADS) void conv_sk_reduce_kernel(float* __res
     const bool inside = m < s.plane && (int)xx < s.W;
     const long opos = inside ? ((long)z * s.H + yy) * s.W + xx : 0;
     const int f0 = fg * FT + ft * 32 + 8 * (rq & 3) + 4 * (lane >> 5);             // registers 4 * (rq & 3) ... + 3 of the m-tile
-    float res[4];
+    float res[4], sc[4], sf[4];
 #pragma unroll
-    for (int q = 0; q < 4; q++) res[q] = e.res && f0 + q < s.F ? e.res[(f0 + q) * ospatial + opos] : 0.f;
+    for (int q = 0; q < 4; q++) {
+        const int fc = f0 + q < s.F ? f0 + q : 0;
+        res[q] = e.res ? e.res[fc * ospatial + opos] : 0.f;
+        sc[q] = e.scale ? e.scale[fc] : 0.f;
+        sf[q] = e.shift ? e.shift[fc] : 0.f;
+    }
     cm_v4f acc = a0 + a1;
     if (nseg > 2) acc += a2;
     if (nseg > 3) acc += a3;
@@ -485,8 +503,8 @@ __global__ __launch_bounds__(CM_THREADS) void conv_sk_reduce_kernel(float* __res
         const int f = f0 + q;
         if (f >= s.F) continue;
         float v = acc[q];
-        if (e.scale) v = v * e.scale[f];
-        if (e.shift) v = v + e.shift[f];
+        if (e.scale) v = v * sc[q];
+        if (e.shift) v = v + sf[q];
         if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
         else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
         if (e.res) v = v + res[q];
@@ -749,6 +767,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
         s.R = (MT / 32 + 2) * CM_TP;
     }
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
+    s.mT = st_magic((unsigned)s.tiles); s.mTX = st_magic((unsigned)(TILE2D ? s.tiles_x : 1)); s.mNC = st_magic((unsigned)s.nchunks); s.mPer = st_magic(1u);
     size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, 64) * 64) * sizeof(float);
     if (KG > 1 && shmem < 4 * 16 * 64 * sizeof(float)) shmem = 4 * 16 * 64 * sizeof(float);  // (4 / KG tiles) x KG groups x 16 registers x 64 lanes   // the groups' sums meet in LDS
     if (POOL && shmem < (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float)) shmem = (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float);   // the finished tile, for its 2 x 2 max pool
@@ -797,6 +816,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
             if (tile0 >= 0 && per < s.nchunks) {
                 const long slots = (s.nchunks - 2 + per) / per + 1;       // a tile's items meet at most this many runs
                 s.sk_per = (int)per; s.sk_items = (int)items; s.sk_tile0 = (int)tile0;
+                s.mPer = st_magic((unsigned)per);
                 s.ksplit = 1;
                 s.cbase = s.nchunks; s.cextra = 0;
                 s.part = fortis_conv_split_scratch((size_t)slots * nfg * (ntiles - tile0) * MT * FT * sizeof(float));
@@ -891,6 +911,7 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
                             int KS, int kind, const ConvEpi& e, hipStream_t st)
 {
     if (C * D * H * Wd >= 2147483647L || F * D * H * Wd * (kind == 1 ? 4 : 1) >= 2147483647L) return -1;
+    if (KD == 1 && D != 1) return -1;                  // the image kernels take one plane
     ConvMShape s;
     memset(&s, 0, sizeof s);
     s.C = (int)C; s.D = (int)D; s.H = (int)H; s.W = (int)Wd;
