@@ -458,58 +458,64 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 // workgroup per tile and group of four accumulator registers (a tile alone would be too few workgroups for a
 // kernel that only moves memory).  A tile's partial sums are added in slot order, i.e. in the order of the input
 // channels.  part[slot][channel group][tile][register quad][thread][4].
+#define CM_RQB 2      // register quads per workgroup of the reduce kernel
 template <int MT, int FT>
 __global__ __launch_bounds__(CM_THREADS) void conv_sk_reduce_kernel(float* __restrict__ y, ConvMShape s, ConvEpi e)
 {
     constexpr int FW = FT / 32, NMT = MT / 32 / (4 / FW), NQ = NMT * 4;
-    const int tl = blockIdx.x, fg = blockIdx.y, rq = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tl = blockIdx.x, fg = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int first = tl * s.nchunks;
     unsigned w0q, w1q, rr;
     st_divmod((unsigned)first, s.mPer, w0q, rr);
     st_divmod((unsigned)(first + s.nchunks - 1), s.mPer, w1q, rr);
     const int nseg = (int)(w1q - w0q) + 1;
     const long slot = (long)gridDim.x * gridDim.y * (NQ * CM_THREADS);
-    const cm_v4f* p = (const cm_v4f*)s.part + (((long)fg * gridDim.x + tl) * NQ + rq) * CM_THREADS + tid;
-    // a thread's loads all leave before the first is needed: the first four slots (a tile always has two) and the
-    // residual values; the sums are then added in slot order
-    const cm_v4f a0 = p[0], a1 = p[slot];
-    const cm_v4f a2 = p[nseg > 2 ? 2 * slot : 0], a3 = p[nseg > 3 ? 3 * slot : 0];
-    unsigned zq, tileq;
-    st_divmod((unsigned)(tl + s.sk_tile0), s.mT, zq, tileq);
-    const int z = (int)zq, tile = (int)tileq;
-    const int ft = wave % FW, mt0 = (wave / FW) * NMT;
-    const long ospatial = (long)s.D * s.H * s.W;
-    const int m = tile * MT + (mt0 + rq / 4) * 32 + (lane & 31);
-    unsigned yy, xx;
-    st_divmod((unsigned)m, s.mP, yy, xx);
-    const bool inside = m < s.plane && (int)xx < s.W;
-    const long opos = inside ? ((long)z * s.H + yy) * s.W + xx : 0;
-    const int f0 = fg * FT + ft * 32 + 8 * (rq & 3) + 4 * (lane >> 5);             // registers 4 * (rq & 3) ... + 3 of the m-tile
-    float res[4], sc[4], sf[4];
+    // a workgroup takes CM_RQB register quads of its tile, one after the other in the code and together in flight
+    auto quad = [&](const int rq) __attribute__((always_inline)) {
+        const cm_v4f* p = (const cm_v4f*)s.part + (((long)fg * gridDim.x + tl) * NQ + rq) * CM_THREADS + tid;
+        // a thread's loads all leave before the first is needed: the first four slots (a tile always has two) and the
+        // residual values; the sums are then added in slot order
+        const cm_v4f a0 = p[0], a1 = p[slot];
+        const cm_v4f a2 = p[nseg > 2 ? 2 * slot : 0], a3 = p[nseg > 3 ? 3 * slot : 0];
+        unsigned zq, tileq;
+        st_divmod((unsigned)(tl + s.sk_tile0), s.mT, zq, tileq);
+        const int z = (int)zq, tile = (int)tileq;
+        const int ft = wave % FW, mt0 = (wave / FW) * NMT;
+        const long ospatial = (long)s.D * s.H * s.W;
+        const int m = tile * MT + (mt0 + rq / 4) * 32 + (lane & 31);
+        unsigned yy, xx;
+        st_divmod((unsigned)m, s.mP, yy, xx);
+        const bool inside = m < s.plane && (int)xx < s.W;
+        const long opos = inside ? ((long)z * s.H + yy) * s.W + xx : 0;
+        const int f0 = fg * FT + ft * 32 + 8 * (rq & 3) + 4 * (lane >> 5);             // registers 4 * (rq & 3) ... + 3 of the m-tile
+        float res[4], sc[4], sf[4];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int fc = f0 + q < s.F ? f0 + q : 0;
-        res[q] = e.res ? e.res[fc * ospatial + opos] : 0.f;
-        sc[q] = e.scale ? e.scale[fc] : 0.f;
-        sf[q] = e.shift ? e.shift[fc] : 0.f;
-    }
-    cm_v4f acc = a0 + a1;
-    if (nseg > 2) acc += a2;
-    if (nseg > 3) acc += a3;
-    for (int k = 4; k < nseg; k++) acc += p[k * slot];
-    if (!inside) return;
+        for (int q = 0; q < 4; q++) {
+            const int fc = f0 + q < s.F ? f0 + q : 0;
+            res[q] = e.res ? e.res[fc * ospatial + opos] : 0.f;
+            sc[q] = e.scale ? e.scale[fc] : 0.f;
+            sf[q] = e.shift ? e.shift[fc] : 0.f;
+        }
+        cm_v4f acc = a0 + a1;
+        if (nseg > 2) acc += a2;
+        if (nseg > 3) acc += a3;
+        for (int k = 4; k < nseg; k++) acc += p[k * slot];
+        if (!inside) return;
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int f = f0 + q;
-        if (f >= s.F) continue;
-        float v = acc[q];
-        if (e.scale) v = v * sc[q];
-        if (e.shift) v = v + sf[q];
-        if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
-        else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
-        if (e.res) v = v + res[q];
-        y[f * ospatial + opos] = v;
-    }
+        for (int q = 0; q < 4; q++) {
+            const int f = f0 + q;
+            if (f >= s.F) continue;
+            float v = acc[q];
+            if (e.scale) v = v * sc[q];
+            if (e.shift) v = v + sf[q];
+            if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
+            else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
+            if (e.res) v = v + res[q];
+            y[f * ospatial + opos] = v;
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < CM_RQB; u++) quad((int)blockIdx.z * CM_RQB + u);
 }
 
 // Sums the partial results of a channel-split launch in split order (deterministic) and applies the
@@ -827,7 +833,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
                 }
                 hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL, true>), dim3((unsigned)cdiv(items, per), (unsigned)nfg, 1), dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
                 HIP_OK(hipGetLastError());
-                hipLaunchKernelGGL((conv_sk_reduce_kernel<MT, FT>), dim3((unsigned)(ntiles - tile0), (unsigned)nfg, (MT / 32 / (4 / (FT / 32))) * 4), dim3(CM_THREADS), 0, st, y, s, e);
+                hipLaunchKernelGGL((conv_sk_reduce_kernel<MT, FT>), dim3((unsigned)(ntiles - tile0), (unsigned)nfg, (MT / 32 / (4 / (FT / 32))) * 4 / CM_RQB), dim3(CM_THREADS), 0, st, y, s, e);
                 HIP_OK(hipGetLastError());
                 return 0;
             }
