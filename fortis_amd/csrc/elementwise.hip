@@ -96,10 +96,36 @@ __global__ __launch_bounds__(256) void transpose4_kernel(const float* __restrict
     }
 }
 
+// One side short (channels-last <-> channels-first with a handful of channels): a thread takes all the elements of
+// one index of the long side, so its loads (ROWS: one per row, each coalesced over the threads) or its stores are
+// the short run, contiguous from thread to thread; a 32 x 32 tile would be mostly empty.
+template <typename TI, typename TO, typename F, bool ROWS>
+__global__ void transpose_short_kernel(const TI* __restrict__ src, TO* __restrict__ dst, long R, long Cc, F f)
+{
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (ROWS) {                       // R <= 8 rows: thread per column c
+        if (i >= Cc) return;
+        for (long r = 0; r < R; r++) dst[i * R + r] = f(src[r * Cc + i], r, i);
+    } else {                          // Cc <= 8 columns: thread per row r
+        if (i >= R) return;
+        for (long c = 0; c < Cc; c++) dst[c * R + i] = f(src[i * Cc + c], i, c);
+    }
+}
+
 template <typename TI, typename TO, typename F>
 static void launch_transpose(const TI* src, TO* dst, long R, long Cc, F f, hipStream_t s)
 {
     if (R <= 0 || Cc <= 0) return;
+    if (R <= 8 && Cc >= 256) {
+        hipLaunchKernelGGL((transpose_short_kernel<TI, TO, F, true>), dim3((unsigned)cdiv(Cc, 256)), dim3(256), 0, s, src, dst, R, Cc, f);
+        HIP_OK(hipGetLastError());
+        return;
+    }
+    if (Cc <= 8 && R >= 256) {
+        hipLaunchKernelGGL((transpose_short_kernel<TI, TO, F, false>), dim3((unsigned)cdiv(R, 256)), dim3(256), 0, s, src, dst, R, Cc, f);
+        HIP_OK(hipGetLastError());
+        return;
+    }
     if constexpr (std::is_same<TI, float>::value && std::is_same<TO, float>::value) {
         if (R % 4 == 0 && Cc % 4 == 0 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
             hipLaunchKernelGGL((transpose4_kernel<F>), dim3((unsigned)cdiv(Cc, 64), (unsigned)cdiv(R, 64)), dim3(256), 0, s, src, dst, R, Cc, f);

@@ -331,3 +331,19 @@ def test_config5_tsrgan(L, gpu, D, ch, nblocks):
     y = plan.forward(case["x"], (2 * D, 2 * D, 2 * D, case["cout"]))
     assert maxrel(y, tsrgan_ref(case)) < TOL
     plan.close()
+
+
+@pytest.mark.parametrize("C_,S", [(3, 35937), (3, 100), (5, 1000), (8, 256), (12, 4096), (64, 7)])
+def test_permute_channels_last_and_back_bit_exact(L, gpu, C_, S):
+    """Channels-last <-> channels-first copies (the TSRGAN step's first and last operation: NDHWC <-> NCDHW), with few
+    channels (a thread per position), few positions and the tiled form: a permutation of the same bits."""
+    x = np.random.default_rng(C_ * 1000 + S).standard_normal((S, C_)).astype(np.float32)
+    for first in (True, False):
+        src = x if first else np.ascontiguousarray(x.T)          # [S][C] -> [C][S], or back
+        p = P.Plan()
+        t0, t1 = p.tensor(src.size), p.tensor(src.size)
+        p.permute(t0, t1, C_, S, first)
+        p.finalize(t0, t1)
+        got = p.forward(src, src.T.shape)
+        p.close()
+        assert np.array_equal(got.view(np.uint32), np.ascontiguousarray(src.T).view(np.uint32))
