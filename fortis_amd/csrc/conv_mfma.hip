@@ -92,7 +92,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R rounded up to a wave's 64 lanes]
     const int RR = TILE2D ? R2 : KS == 1 ? MT : s.R;              // staged elements per channel and kd (s.R, a constant where it can be)
     const int XCH = CC * KD * RR;
-    const int XCHP = (XCH + 63) / 64 * 64;
+    const int XCHP = (XCH + 64) / 64 * 64;                        // at least one spare slot behind the staged elements (see XDUMP)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // volumes: neighbouring tiles and planes on one XCD (input fetched once instead of 2-3 times; on images the
@@ -150,6 +150,13 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     // the mark 0xffffffff in gchk, which the store compares with the chunk's limit.
     unsigned goff[NX], gchk[NX];
     bool inb[NX];                // the element lies inside the tensor (not padding, not past the staged run)
+    // XDUMP: a chunk's store is unconditional -- an element that is padding sends its (unused) value to the spare slot
+    // behind the buffer's staged elements instead of being masked off.  One select per element and tile, where the
+    // mask cost a save, a branch and a restore of the lane mask per element and chunk.  Not in the form that runs
+    // four workgroups per CU, nor in the streamed one with 16 staging rounds: their registers have none to spare for
+    // the addresses.
+    constexpr bool XDUMP = SK ? NX <= 8 : !(KD == 3 && MT == 128 && FT == 64 && NX <= 8);
+    unsigned xslot[XDUMP ? NX : 1];
 #pragma unroll
     for (int i = 0; i < NX; i++) {
         // straight-line: an element past the staged run or outside the tensor works its numbers out like any other
@@ -180,6 +187,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         goff[i] = in ? off : 0u;
         gchk[i] = in ? off : 0xffffffffu;
         inb[i] = in;
+        if constexpr (XDUMP) xslot[i] = in ? (unsigned)el : (unsigned)XCH;
     }
 
     // byte offsets at or beyond chunk_lim belong to channels past the last one (only in a partial last chunk)
@@ -217,9 +225,15 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         }
         float* xdst = sX + buf * XCHP + tid;
         if ((ch + 1) * CC <= s.C) {
+            if constexpr (XDUMP) {
+                float* xb = sX + buf * XCHP;
 #pragma unroll
-            for (int i = 0; i < NX; i++)
-                if (inb[i]) xdst[i * CM_THREADS] = r.rx[i];
+                for (int i = 0; i < NX; i++) xb[xslot[i]] = r.rx[i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < NX; i++)
+                    if (inb[i]) xdst[i * CM_THREADS] = r.rx[i];
+            }
         } else {
             const unsigned lim = chunk_lim(ch);
 #pragma unroll
@@ -774,7 +788,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     }
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
     s.mT = st_magic((unsigned)s.tiles); s.mTX = st_magic((unsigned)(TILE2D ? s.tiles_x : 1)); s.mNC = st_magic((unsigned)s.nchunks); s.mPer = st_magic(1u);
-    size_t shmem = (size_t)2 * (CC * T * FT + cdiv((long)CC * KD * s.R, 64) * 64) * sizeof(float);
+    size_t shmem = (size_t)2 * (CC * T * FT + ((long)CC * KD * s.R + 64) / 64 * 64) * sizeof(float);
     if (KG > 1 && shmem < 4 * 16 * 64 * sizeof(float)) shmem = 4 * 16 * 64 * sizeof(float);  // (4 / KG tiles) x KG groups x 16 registers x 64 lanes   // the groups' sums meet in LDS
     if (POOL && shmem < (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float)) shmem = (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float);   // the finished tile, for its 2 x 2 max pool
     if (shmem > 160 * 1024) return -1;
