@@ -919,15 +919,18 @@ void chain_stencil_rows_kernel(ChainParams params)
             st_chain_apply<NQ, true>(g, cell, in.x);
             // (slots past the network's inputs, which hold a copy of slot 0, are zeroed in the LDS tile below; rows past
             // the end hold the first cell's values and their results are never stored: no per-slot select here)
+            // The divisors are the same for every row: scalar loads, all of them out before the first division.  Slots
+            // past the network's inputs (zeroed below) divide by slot 0's divisor rather than sit behind a branch each.
             if (in_rcp && st_div_wave_in_range(in.x, 1.f)) {
                 // divisors in range (checked when the step was built), numerators too: the short form of the division
+                const cfloat* cd = st_c(d.in_div);
+                const cfloat* cr = st_c(d.in_rcp);
 #pragma unroll
-                for (int q = 0; q < NQ; q++)
-                    if (q < K0) in.x[q] = st_div_inrange(in.x[q], in_div[q], in_rcp[q]);
+                for (int q = 0; q < NQ; q++) { const int qc = q < K0 ? q : 0; in.x[q] = st_div_inrange(in.x[q], cd[qc], cr[qc]); }
             } else if (in_div) {
+                const cfloat* cd = st_c(d.in_div);
 #pragma unroll
-                for (int q = 0; q < NQ; q++)
-                    if (q < K0) in.x[q] = __fdiv_rn(in.x[q], in_div[q]);
+                for (int q = 0; q < NQ; q++) { const int qc = q < K0 ? q : 0; in.x[q] = __fdiv_rn(in.x[q], cd[qc]); }
             }
         }
         // ---- two halves of 32 rows: their operands through the LDS tile, two m-tiles through the layers ------
@@ -977,7 +980,7 @@ void chain_stencil_rows_kernel(ChainParams params)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             ov[r] = o4[r];
-            if (out_mul && r < NO) ov[r] = __fmul_rn(ov[r], out_mul[r]);
+            if (out_mul) ov[r] = __fmul_rn(ov[r], st_c(d.out_mul)[r < NO ? r : 0]);      // (outputs past the last are not stored)
         }
         gfloat* Yraw = st_g(P.Yraw);
         if (Yraw && valid) {

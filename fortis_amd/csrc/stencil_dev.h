@@ -33,6 +33,11 @@ __device__ __forceinline__ unsigned st_xcd_band_block() { return fortis_xcd_band
 typedef __attribute__((address_space(1))) float gfloat;
 __device__ __forceinline__ const gfloat* st_g(const float* p) { return (const gfloat*)p; }
 __device__ __forceinline__ gfloat* st_g(float* p) { return (gfloat*)p; }
+// A table that no kernel writes, read at an index that is the same in every lane: through the constant address
+// space such reads are scalar loads (one request per wave, neighbours fetched together), where a global load of a
+// uniform address is a vector instruction that every lane waits for.
+typedef __attribute__((address_space(4))) float cfloat;
+__device__ __forceinline__ const cfloat* st_c(const float* p) { return (const cfloat*)p; }
 __device__ __forceinline__ int st_u(int v) { return __builtin_amdgcn_readfirstlane(v); }   // wave-uniform value
 struct StIns { int op, a, b; float ca, cb; };          // per-cell instruction, constants inlined
 struct StStep { int op, code, tv_left; float cv; };    // tv chain step, constant inlined
