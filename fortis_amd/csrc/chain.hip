@@ -729,6 +729,18 @@ void chain_stencil_fast_kernel(ChainParams params)
             in.sS[q] = ssp[q][off];
         }
     };
+    // the input divisors of the lane's eight slots: the same for every tile, loaded once (slots past the network's
+    // inputs take slot 0's; their quotients are replaced by zero)
+    float dv[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) dv[t] = 1.f;
+    if (in_div) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const int q = 16 * (t >> 2) + 4 * lq + (t & 3);
+            dv[t] = in_div[q < K0 ? q : 0];
+        }
+    }
     auto process = [&](TileIn& in) __attribute__((always_inline)) {
         const unsigned row = in.row0 + lrow;
         const bool valid = row < rows;
@@ -745,9 +757,14 @@ void chain_stencil_fast_kernel(ChainParams params)
 #pragma unroll
             for (int t = 0; t < 8; t++) {
                 const int q = 16 * (t >> 2) + 4 * lq + (t & 3);
-                float v = (valid && q < K0) ? tv[t] : 0.f;
-                if (in_div && q < K0) v = __fdiv_rn(v, in_div[q]);
-                a[t >> 2][t & 3] = v;
+                a[t >> 2][t & 3] = (valid && q < K0) ? tv[t] : 0.f;
+            }
+            if (in_div) {
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    const int q = 16 * (t >> 2) + 4 * lq + (t & 3);
+                    a[t >> 2][t & 3] = (valid && q < K0) ? __fdiv_rn(tv[t], dv[t]) : 0.f;
+                }
             }
             a[2] = a[3] = (v4f)(0.f);
         }
@@ -762,7 +779,10 @@ void chain_stencil_fast_kernel(ChainParams params)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             ov[r] = a[0][r];
-            if (out_mul && r < NO) ov[r] = __fmul_rn(ov[r], out_mul[r]);
+        }
+        if (out_mul) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) ov[r] = __fmul_rn(ov[r], st_c(d.out_mul)[r < NO ? r : 0]);      // (outputs past the last are not stored)
         }
         gfloat* Yraw = st_g(P.Yraw);
         if (Yraw && valid && lq == 0) {
