@@ -1000,7 +1000,10 @@ void chain_stencil_rows_kernel(ChainParams params)
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             ov[r] = o4[r];
-            if (out_mul) ov[r] = __fmul_rn(ov[r], st_c(d.out_mul)[r < NO ? r : 0]);      // (outputs past the last are not stored)
+        }
+        if (out_mul) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) ov[r] = __fmul_rn(ov[r], st_c(d.out_mul)[r < NO ? r : 0]);      // (outputs past the last are not stored)
         }
         gfloat* Yraw = st_g(P.Yraw);
         if (Yraw && valid) {
