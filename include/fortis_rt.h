@@ -44,7 +44,8 @@ void  fortis_pool_set_allocator(int (*raw_alloc)(void** p, unsigned long nbytes)
 void  fortis_pool_stats(int* held, int* used);
 
 /* ---- GEMM -------------------------------------------------------------------------------- */
-/* C[B][N] = A[B][K] . W[N][K]^T, fp32, beta = 0.                     runtime/fortis_rt.c:45-75 */
+/* C[B][N] = A[B][K] . W[N][K]^T, fp32, beta = 0.                     runtime/fortis_rt.c:45-75
+ * Empty problems as the reference's SGEMM call leaves them: B = 0 or N = 0 does nothing, K = 0 sets C to zero. */
 void fortis_gemm(float* Aa, float* A, long Ao, long As0, long As1, long At0, long At1,
                  float* Wa, float* W, long Wo, long Ws0, long Ws1, long Wt0, long Wt1,
                  float* Ca, float* C, long Co, long Cs0, long Cs1, long Ct0, long Ct1,
