@@ -541,7 +541,9 @@ void chain_wave_kernel(ChainParams params)
                 }
         }
         if constexpr (NTMAX == 4 && !STENCIL) {           // (the general stencil form has no registers to spare for it)
+            __builtin_amdgcn_s_setprio(3);          // as in the fused forms: the matrix phase outranks the other waves' loads and stores
             layers_narrow<WLDS, true, SIG>(a, d, nlayers, sWts, wall, lane, lq);
+            __builtin_amdgcn_s_setprio(0);
         } else
         for (int l = 0; l < nlayers; l++) {
             asm volatile("" ::: "memory");
