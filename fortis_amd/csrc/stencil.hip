@@ -42,9 +42,11 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
             // pointer plus that offset (unused table entries repeat slot 0)
             const long off = st_off(d.refs[0], i, j, kk);
 #pragma unroll
-            for (int q = 0; q < NQ; q++) tv[q] = st_g(d.refs[q].p)[off];
+            // (the pointers straight from the kernel arguments, by literal index: scalar loads, where the copy in LDS
+            // costs a vector read and two v_readfirstlane per pointer)
+            for (int q = 0; q < NQ; q++) tv[q] = st_g(args.refs[q].p)[off];
 #pragma unroll
-            for (int sI = 0; sI < ST_SCAL_MAX; sI++) cell.S[sI] = st_g(d.scal[sI].p)[off];
+            for (int sI = 0; sI < ST_SCAL_MAX; sI++) cell.S[sI] = st_g(args.scal[sI].p)[off];
             st_cell_program(d, cell);
         } else {
 #pragma unroll
