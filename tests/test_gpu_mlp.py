@@ -178,7 +178,7 @@ def test_fortis_gemm_entry_empty_problems(L, gpu, capfd):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("NI,NK", [(384, 124), (50, 33), (1, 1)])
+@pytest.mark.parametrize("NI,NK", [(384, 124), (50, 33), (1, 1), (300, 5), (6, 400)])
 def test_boundary_pre_post_bit_exact(L, gpu, dtype, NI, NK):
     """E3SM boundary shapes (384 x 124 f64 in, trt_backend/e3sm_boundary.cu:9-20) and ragged ones;
     host-type arithmetic then cast, bit-exact against the oracle."""
