@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused inference step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload climsim|zb|zb_ref|zb_unfused|toy|unet|tsrgan|copy|issue_probe] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload climsim|zb|zb_ref|zb_unfused|toy|unet|tsrgan|copy] [--no-cpu]
 
 One "step" is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  Prints ONE JSON line: columns/s for the whole job, the roofline figure of the dominant
@@ -170,25 +170,6 @@ def run_copy(L, args):
                              frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(avg, 5), bytes_per_launch=2 * n * 4, traffic=None))
     p.close()
     return out
-
-
-def run_issue_probe(L, args):
-    """Do a SIMD's fp32 matrix instructions and vector instructions of other waves run at the same time?  Prints the
-    probe's three times (matrix waves alone, vector waves alone, both) for both matrix shapes and for floating-point
-    and integer vector work; `value` is (alone + alone) / both: 1.0 = no overlap at all, up to 2.0 = full overlap."""
-    rows, worst = [], 2.0
-    t0 = time.perf_counter()
-    for big in (0, 1):
-        for ints in (0, 1):
-            ms = (C.c_float * 3)()
-            assert L.fortis_probe_issue_ms(20000, big, ints, ms) == 0
-            rows.append({"matrix": "32x32x2" if big else "16x16x4", "vector": "v_add_u32/v_xor_b32" if ints else "v_fma_f32",
-                         "matrix_alone_ms": round(ms[0], 3), "vector_alone_ms": round(ms[1], 3), "both_ms": round(ms[2], 3)})
-            worst = min(worst, (ms[0] + ms[1]) / ms[2])
-    dt = time.perf_counter() - t0
-    return dict(rows=0, dt=dt, dtype="f32", metric="(matrix alone + vector alone) / both, smallest of the four pairings", unit="ratio", value=round(worst, 3),
-                config={"workload": "issue_probe_fp32_mfma_vs_valu", "launches_per_step": 0, "pairings": rows},
-                roofline=dict(bound="mfma", kernel="issue_probe_kernel", achieved=None, peak=PEAK_F32_MFMA_TFLOPS, unit="TFLOP/s", frac=None, traffic=None))
 
 
 def run_zb_unfused(L, args):
@@ -492,7 +473,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20, help="untimed steps first; the clocks need about ten steps of this size to settle")
-    ap.add_argument("--workload", default=None, help="default: climsim, followed by short runs of the other configurations (others)", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan", "issue_probe"])
+    ap.add_argument("--workload", default=None, help="default: climsim, followed by short runs of the other configurations (others)", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other configurations that follow the default workload")
     ap.add_argument("--f64", action="store_true", help="zb_unfused only: double-precision host arrays (the general stencil kernels)")
@@ -531,8 +512,6 @@ def run_workload(L, args, workload):
         return run_toy(L, args)
     if workload == "copy":
         return run_copy(L, args)
-    if workload == "issue_probe":
-        return run_issue_probe(L, args)
     if workload in ("unet", "tsrgan"):
         return run_conv(L, args, workload)
     if workload == "zb_unfused":

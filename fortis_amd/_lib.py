@@ -91,7 +91,7 @@ PROTOTYPES = {
     "fortis_stencil_step_fused_time_ms": (f, [C.POINTER(Stencil), C.POINTER(Stencil), vp, C.POINTER(vp), C.POINTER(vp), vp, i]),
     "fortis_plan_profile": (None, [vp, i]), "fortis_plan_profile_read": (i, [vp, fp]),
     "fortis_plan_kernel_name": (C.c_char_p, [vp, i]),
-    "fortis_time_ms": (f, [vp, vp, i]), "fortis_time_parts_ms": (i, [i, vp, vp, i, fp]), "fortis_probe_issue_ms": (i, [i, i, i, fp]),
+    "fortis_time_ms": (f, [vp, vp, i]), "fortis_time_parts_ms": (i, [i, vp, vp, i, fp]),
     "fortis_plan_time_ms": (f, [vp, i, i]),
 }
 DATA_SYMBOLS = ["fortis_capturing"]

@@ -242,11 +242,6 @@ float fortis_time_ms(void (*fn)(void*), void* arg, int iters);
  * HIP event between the parts and no host wait inside: ms_out[k] receives the elapsed milliseconds of
  * part k summed over the iterations.  Returns -1 on bad arguments. */
 int   fortis_time_parts_ms(int nparts, void (*const* fns)(void*), void* const* args, int iters, float* ms_out);
-/* Measurement aid without a counterpart in the reference: times a probe kernel whose workgroups put four waves of
- * independent fp32 matrix instructions (16x16x4, or 32x32x2 when big) and four waves of independent vector
- * instructions (fp32 fma, or integer add/xor when ints) on the same four SIMDs.  out_ms[0..2] = milliseconds per
- * launch of the matrix waves alone, the vector waves alone, and both together.  Returns -1 on bad arguments or no memory. */
-int   fortis_probe_issue_ms(int iters, int big, int ints, float* out_ms);
 /* Same clock around `iters` enqueues of a plan (use_graph: captured once, then replayed) and of
  * the fused stencil step. */
 float fortis_plan_time_ms(fortis_plan* p, int iters, int use_graph);
