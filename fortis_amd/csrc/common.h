@@ -20,6 +20,7 @@
 // caller that gets -1 must not launch anything on the pointer.
 int  fortis_dev_malloc(void** p, size_t nbytes, const char* what);
 void fortis_dev_free(void* p);
+bool fortis_pool_on_device();   // false while a test has replaced the raw allocator (fortis_pool_set_allocator)
 
 extern "C" long fortis_step_generation(void);   // plan.hip: count of forward passes of the bound step
 static inline hipStream_t fortis_stream_get() { return (hipStream_t)mgpuStreamCreate(); }

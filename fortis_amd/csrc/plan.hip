@@ -350,7 +350,6 @@ static size_t try_chain(fortis_plan* p, size_t i, Exec* ex)
 // graph names them) and every buffer the walk touched stays marked in use in the pool until the plan is
 // destroyed.  The model's input and output, and tensors no kernel writes (filled by the caller), keep their
 // buffer throughout; a tensor no kernel touches (folded into a neighbour at fusion) gets none.
-void fortis_pool_hold(void* p);   // rt.hip: marks a pool buffer in use again
 static int assign_buffers(fortis_plan* p)
 {
     const int nt = (int)p->tbytes.size(), ne = (int)p->exec.size();
@@ -371,22 +370,34 @@ static int assign_buffers(fortis_plan* p)
     for (void* b : p->bufs) fortis_free(b);
     p->bufs.clear();
     p->tptr.assign(nt, nullptr);
+    // The sharing is done on a list of the plan's own: a buffer the walk has handed back stays marked in use in the
+    // pool, so the pool's release-everything-unused-and-retry (when a later raw allocation fails) can never free a
+    // buffer an earlier tensor of this walk already points to.  Best fit among the walk's released buffers, like
+    // the pool's own choice; a tensor that finds none takes a new buffer from the pool.
+    std::vector<long> bsize;
+    std::vector<char> bfree;
     int rc = 0;
     auto take = [&](int t) {
-        void* d = fortis_alloc(p->tbytes[t]);
-        if (!d) { rc = -1; return; }
-        p->tptr[t] = d;
-        bool seen = false;
-        for (void* b : p->bufs) if (b == d) seen = true;
-        if (!seen) p->bufs.push_back(d);
+        const long n = p->tbytes[t];
+        int best = -1;
+        for (size_t b = 0; b < p->bufs.size(); b++)
+            if (bfree[b] && bsize[b] >= n && (best < 0 || bsize[b] < bsize[best])) best = (int)b;
+        if (best < 0) {
+            void* d = fortis_alloc(n);
+            if (!d) { rc = -1; return; }
+            p->bufs.push_back(d); bsize.push_back(n); bfree.push_back(0);
+            best = (int)p->bufs.size() - 1;
+        }
+        bfree[best] = 0;
+        p->tptr[t] = p->bufs[best];
     };
+    auto give = [&](void* d) { for (size_t b = 0; b < p->bufs.size(); b++) if (p->bufs[b] == d) bfree[b] = 1; };
     for (int t = 0; t < nt && rc == 0; t++) if (p->view_of[t] < 0 && first[t] == -1) take(t);
     for (int i = 0; i < ne && rc == 0; i++) {
         for (int t = 0; t < nt && rc == 0; t++) if (p->view_of[t] < 0 && first[t] == i) take(t);
-        for (int t = 0; t < nt; t++) if (p->view_of[t] < 0 && last[t] == i && p->tptr[t]) fortis_free(p->tptr[t]);
+        for (int t = 0; t < nt; t++) if (p->view_of[t] < 0 && last[t] == i && p->tptr[t]) give(p->tptr[t]);
     }
-    for (void* b : p->bufs) fortis_pool_hold(b);
-    if (rc != 0) return -1;
+    if (rc != 0) { p->tptr.assign(nt, nullptr); return -1; }
     for (int t = 0; t < nt; t++)
         if (p->view_of[t] >= 0 && p->tptr[p->view_of[t]]) p->tptr[t] = (char*)p->tptr[p->view_of[t]] + p->view_off[t];
     return 0;
@@ -527,9 +538,9 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
     p->rows0 = rowwise ? rows : 0;
     if (p->upload_failed) return bad("finalize: out of device memory for the weights");
     if (assign_buffers(p) != 0) return bad("finalize: out of device memory for the activations");
-    (void)fortis_stream_get();
     p->finalized = true;
-    HIP_OK(hipDeviceSynchronize());
+    // (with a test's host allocator in place of the device's there is no device to wait for, and no launch may follow)
+    if (fortis_pool_on_device()) { (void)fortis_stream_get(); HIP_OK(hipDeviceSynchronize()); }
     return 0;
 }
 

@@ -73,13 +73,7 @@ int fortis_dev_malloc(void** p, size_t nbytes, const char* what)
     return -1;
 }
 void fortis_dev_free(void* p) { if (p) g_free(p); }
-
-// A buffer the pool handed out earlier and has since taken back is claimed again by its address (the plan
-// fixes its buffers once and keeps them while it lives).  A pointer the pool does not hold is ignored.
-void fortis_pool_hold(void* p)
-{
-    for (int i = 0; i < FORTIS_POOL; i++) if (g_pool[i].p == p) { g_pool[i].used = 1; return; }
-}
+bool fortis_pool_on_device() { return g_alloc == dev_alloc; }
 
 extern "C" {
 // Test hook: replaces the raw allocator (null restores hipMalloc/hipFree) and empties the pool table.

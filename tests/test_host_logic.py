@@ -292,3 +292,55 @@ def test_bench_contract_without_a_gpu():
     for key in ("climsim", "zb", "zb_ref", "zb_1028x1028x15", "zb_unfused_1028x1028x15", "zb_unfused_1028x1028x15_f64", "unet", "tsrgan"):
         assert bench.MEASURED_TRAFFIC[key] > 0
     assert bench.PEAK_HBM_GBS == 8000.0 and bench.PEAK_F32_MFMA_TFLOPS == 157.3
+
+
+def _mask_relu_stack(L, sizes):
+    """A plan of weightless row-wise ops t0 -> t1 -> ... (one tensor per entry of sizes, in floats)."""
+    p = L.fortis_plan_create()
+    ts = [L.fortis_plan_tensor(p, 4 * n) for n in sizes]
+    for a, b, n in zip(ts[:-1], ts[1:], sizes[1:]):
+        assert L.fortis_plan_mask_relu(p, a, b, 1, min(n, sizes[ts.index(a)]), 0) == 0
+    return p, ts
+
+
+def test_buffer_walk_survives_a_raw_allocation_that_fails_once(pool):
+    """The walk that gives tensors their buffers hands a temporary back behind its last reader.  When a later raw
+    allocation fails, the pool frees every buffer it holds unused and retries (runtime/fortis_rt.c:24-35): none of
+    those may be a buffer an earlier tensor of the same walk still points to.  One raw allocation is made to fail
+    once in the middle of the walk; afterwards every tensor's buffer is a live allocation, tensors alive at the same
+    time have different buffers, and destroying the plan hands everything back."""
+    L, dev = pool
+    dev.capacity = 1 << 20
+    fail_at, real = [4], dev.a                       # the walk's 4th raw allocation fails once (t3: larger than released t1)
+
+    def flaky(pp, n):
+        fail_at[0] -= 1
+        return -1 if fail_at[0] == 0 else real(pp, n)
+
+    fa = ALLOC(flaky)
+    L.fortis_pool_set_allocator(C.cast(fa, C.c_void_p), C.cast(dev.f, C.c_void_p))
+    sizes = [8, 16, 16, 32, 8]                       # t0 in, t1, t2, t3 (needs a new, larger buffer), t4 out
+    p, ts = _mask_relu_stack(L, sizes)
+    assert L.fortis_plan_finalize(p, ts[0], ts[-1]) == 0
+    ptr = [L.fortis_plan_tensor_ptr(p, t) for t in ts]
+    assert all(q in dev.live for q in ptr), "a tensor points at a buffer the raw allocator has taken back"
+    for a, b in zip(ptr[:-1], ptr[1:]):
+        assert a != b                                # a kernel's source and destination never share
+    assert ptr[0] not in ptr[1:]                     # the model's input is never shared
+    held, used = stats(L)
+    assert used == len(set(ptr)) and held == used    # every buffer of the plan stays in use in the pool; nothing else is held
+    L.fortis_plan_destroy(p)
+    assert stats(L)[1] == 0
+
+
+def test_buffer_walk_that_runs_out_of_memory_fails_cleanly(pool, capfd):
+    """A walk whose later tensor finds no memory even after the pool has released what it can: finalize returns -1,
+    no tensor pointer is handed out, and destroy returns every buffer exactly once."""
+    L, dev = pool                                    # 1000 bytes
+    p, ts = _mask_relu_stack(L, [50, 50, 50, 200, 50])      # 200 + 200 + 200 + 800 bytes > 1000
+    assert L.fortis_plan_finalize(p, ts[0], ts[-1]) == -1
+    assert "out of device memory for the activations" in capfd.readouterr().err
+    assert L.fortis_plan_tensor_ptr(p, ts[1]) is None
+    frees0 = dev.frees
+    L.fortis_plan_destroy(p)
+    assert stats(L)[1] == 0 and dev.frees == frees0  # handed back to the pool (still held there), none freed twice
