@@ -6,8 +6,9 @@
 One "step" is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  Prints ONE JSON line: columns/s for the whole job, the roofline figure of the dominant
 kernel (duration measured with HIP events on the library's own stream inside the timed region) and
-a CPU baseline (the oracle's port of the reference's native Fortran forward, timed on this host on a
-bounded sample of the same workload).  Only the cpu_baseline leg touches oracle/.
+a CPU baseline (PyTorch CPU eval of the same network, the reference's CPU path for the column MLPs, with the oracle's
+port of the reference's native Fortran forward beside it, both timed on this host on a bounded sample of the same
+workload).  Only the cpu_baseline leg touches oracle/.
 """
 import argparse
 import ctypes as C
@@ -34,6 +35,22 @@ MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((1114.1 * 2 + 
                     # conv workloads: every conv, split-reduce and thin-head dispatch of a step summed, divided by the
                     # step's conv operations (18 and 19), like flop_per_launch
                     "unet": int((1131516.0 * 2 + 544769.0) * 1024 / 7 / 18), "tsrgan": int((3423671.0 * 2 + 5019823.0) * 1024 / 7 / 19)}
+
+
+TRAFFIC_SOURCE = {"climsim": "profiles/gemm_bias_act_climsim.txt", "zb": "profiles/mlp_chain_stencil_zb.txt",
+                  "zb_ref": "profiles/mlp_chain_stencil_zb.txt", "zb_1028x1028x15": "profiles/mlp_chain_stencil_zb.txt",
+                  "zb_ref_1028x1028x15": "profiles/mlp_chain_stencil_zb.txt",
+                  "zb_unfused_1028x1028x15": "profiles/stencil_gather_scatter_zb_1028x1028x15.txt",
+                  "zb_unfused_1028x1028x15_f64": "profiles/stencil_gather_scatter_zb_1028x1028x15.txt",
+                  "unet": "profiles/conv_mfma_unet_tsrgan.txt", "tsrgan": "profiles/conv_mfma_unet_tsrgan.txt"}
+
+
+def traffic(key):
+    """roofline.traffic and where it comes from: a constant from a rocprofv3 --pmc run of this command recorded under
+    profiles/ (counters cannot be read from inside this process), never a figure of the present run."""
+    t = MEASURED_TRAFFIC.get(key)
+    return dict(traffic=t, traffic_source=None if t is None else
+                "constant from %s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes of this command); not measured in this run" % TRAFFIC_SOURCE[key])
 
 
 def omp_threads():
@@ -94,6 +111,17 @@ def cpu_torch_mlp(case, sample_rows, X, min_seconds=4.0, in_norms=None, out_norm
                 sample=f"PyTorch {torch.__version__} CPU eval fp32 of the same network, {sample_rows} rows x {reps} passes, {dt:.1f} s")
 
 
+def cpu_baseline_both(case, sample_rows, X, port_seconds, torch_seconds, **norms):
+    """The stated CPU baseline is the reference's own CPU path for the column MLPs, PyTorch CPU eval of the exporter's
+    module (benchmarks/climsim/export_climsim.py:32-34 writes its reference output that way); the oracle's port of
+    the native Fortran loop nest (mom6_zb/fwd_native_zb.f90:30-48) on the same sample rides inside it."""
+    t = cpu_torch_mlp(case, sample_rows, X, min_seconds=torch_seconds, **norms)
+    port = cpu_baseline_mlp(case, sample_rows, X, min_seconds=port_seconds, **norms)
+    return dict(value=t["value"], unit=t["unit"], cores=t["threads"], kind="port", path="pytorch_cpu_eval",
+                sample=t["sample"] + " (a restated nn.Module with the same seeded weights; the reference's exporter is not imported)",
+                native_loop_port=port)
+
+
 def timed_steps(L, plan, steps):
     """Two passes of `steps` steps each: the first, with nothing but the step's own launches on the stream,
     is the clocked one (-> value, ms_per_step); the second records a HIP event on the library's stream
@@ -138,11 +166,10 @@ def run_climsim(L, args):
                roofline=dict(bound="mfma", kernel="gemm_bias_act (fp32 MFMA 32x32x2)", achieved=round(achieved, 3),
                              peak=PEAK_F32_MFMA_TFLOPS, unit="TFLOP/s", frac=round(achieved / PEAK_F32_MFMA_TFLOPS, 4),
                              avg_launch_ms=round(avg_launch_ms, 5), flop_per_launch=flops_per_launch,
-                             traffic=MEASURED_TRAFFIC["climsim"]))
+                             **traffic("climsim")))
     if not args.no_cpu:
         X = np.ascontiguousarray(case["A"][:2048])
-        out["cpu_baseline"] = cpu_baseline_mlp(case, 2048, X)
-        out["cpu_baseline"]["torch_cpu"] = cpu_torch_mlp(case, 2048, X)
+        out["cpu_baseline"] = cpu_baseline_both(case, 2048, X, 8.0, 6.0)
     plan.close()
     return out
 
@@ -243,7 +270,7 @@ def run_zb_unfused(L, args):
                 unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(g_ms, 5), bytes_per_launch=g_bytes,
                 back_to_back_ms=round(ga_ms, 5), back_to_back_frac=round(g_bytes / (ga_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                 scatter_GBs=round(s_bytes / (s_ms * 1e-3) / 1e9, 1), scatter_ms_all_layers=round(s_ms, 5), mlp_ms=round(m_ms, 5),
-                traffic=MEASURED_TRAFFIC.get("zb_unfused_%dx%dx%d%s" % (sx, sy, nz, "_f64" if args.f64 else "")))
+                **traffic("zb_unfused_%dx%dx%d%s" % (sx, sy, nz, "_f64" if args.f64 else "")))
     out = dict(rows=rows, dt=dt, dtype="f32",
                config={"workload": "zb_unfused_gather_mlp_scatter_27_64_64_3_%dx%dx%d%s" % (sx, sy, nz, "_f64_arrays" if args.f64 else ""), "columns": rows,
                        "cells_per_layer": count, "layers": nz, "launches_per_step": 1 + nz + plan.num_kernels},
@@ -283,6 +310,7 @@ def run_conv(L, args, which):
     ev_total = sum(kern.values())
     step_ms = dt / passes * 1e3
     conv_ms = step_ms * sum(v for k, v in kern.items() if k in ("conv2d", "conv3d", "convt2d")) / ev_total
+    raw = dict(kern)                                   # as clocked by the events, idle stream per launch included
     kern = {k: v * step_ms / ev_total for k, v in kern.items()}
     nconv = sum(v for k, v in count.items() if k in ("conv2d", "conv3d", "convt2d"))
     achieved = case["flops"] / (conv_ms * 1e-3) / 1e12
@@ -293,7 +321,9 @@ def run_conv(L, args, which):
                              peak=PEAK_F32_MFMA_TFLOPS, unit="TFLOP/s", frac=round(achieved / PEAK_F32_MFMA_TFLOPS, 4),
                              avg_launch_ms=round(conv_ms / nconv, 5), flop_per_launch=case["flops"] / nconv,
                              conv_share_of_step=round(conv_ms / step_ms, 4), event_pass_ms_per_step=round(ev_total, 4),
-                             traffic=MEASURED_TRAFFIC.get(which)))
+                             frac_basis="estimate: the convolutions' share of the event pass (event_pass_ms_by_kernel) applied to the clocked step",
+                             event_pass_ms_by_kernel={k: round(v, 4) for k, v in raw.items()},
+                             **traffic(which)))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_conv(case, which)
     plan.close()
@@ -351,10 +381,9 @@ def run_toy(L, args):
                config={"workload": "toy_mlp_1024x64_256_256_32", "columns": case["rows"], "launches_per_step": plan.num_kernels},
                roofline=dict(bound="mfma", kernel="mlp_chain (LDS-resident, fp32 MFMA)", achieved=round(achieved, 4),
                              peak=PEAK_F32_MFMA_TFLOPS, unit="TFLOP/s", frac=round(achieved / PEAK_F32_MFMA_TFLOPS, 5),
-                             avg_launch_ms=round(avg, 5), flop_per_launch=case["flops"], traffic=MEASURED_TRAFFIC["toy"]))
+                             avg_launch_ms=round(avg, 5), flop_per_launch=case["flops"], **traffic("toy")))
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline_mlp(case, case["rows"], case["X"], min_seconds=3.0)
-        out["cpu_baseline"]["torch_cpu"] = cpu_torch_mlp(case, case["rows"], case["X"], min_seconds=2.0)
+        out["cpu_baseline"] = cpu_baseline_both(case, case["rows"], case["X"], 3.0, 2.0)
     plan.close()
     return out
 
@@ -414,7 +443,7 @@ def run_zb(L, args, reference_net=False):
                 unit="TFLOP/s" if bound == "mfma" else "GB/s",
                 frac=round((tf / PEAK_F32_MFMA_TFLOPS) if bound == "mfma" else (gbs / PEAK_HBM_GBS), 5),
                 avg_launch_ms=round(avg, 5), flop_per_launch=flops, bytes_per_launch=nbytes,
-                hbm_GBs=round(gbs, 2), mfma_TFLOPs=round(tf, 3), traffic=MEASURED_TRAFFIC.get(("zb_ref" if reference_net else "zb") + ("_%dx%dx%d" % (sx, sy, nz) if args.grid else "")))
+                hbm_GBs=round(gbs, 2), mfma_TFLOPs=round(tf, 3), **traffic(("zb_ref" if reference_net else "zb") + ("_%dx%dx%d" % (sx, sy, nz) if args.grid else "")))
     # dt covers the validating launch too; whole-job throughput uses the clocked launches only
     out = dict(rows=rows, dt=ms * 1e-3, wall_dt=dt, dtype="f32",
                config={"workload": "zb_gather_mlp_scatter_%s_%dx%dx%d" % ("27_20_3" if reference_net else "27_64_64_3", sx, sy, nz),
@@ -429,9 +458,8 @@ def run_zb(L, args, reference_net=False):
             from oracle import oracle as O
             X = O.stencil_gather(gd, garr, int(gt.count), int(gt.nk), 3, 3, 64)
             case = dict(net, rows=rows)
-            out["cpu_baseline"] = cpu_baseline_mlp(case, rows, X, min_seconds=5.0, **extra)
+            out["cpu_baseline"] = cpu_baseline_both(case, rows, X, 5.0, 3.0, **extra)
             out["cpu_baseline"]["sample"] += " (MLP part only; the gather and scatter loops of the host are not included)"
-            out["cpu_baseline"]["torch_cpu"] = cpu_torch_mlp(case, rows, X, min_seconds=3.0, **extra)
     plan.close()
     for d in held:
         L.fortis_free(d)

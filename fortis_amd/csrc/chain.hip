@@ -31,7 +31,8 @@ typedef __attribute__((address_space(1))) v4f gv4f;   // 16 bytes of global memo
 
 // max(v, 0) in one instruction, on the bit pattern: a float with the sign bit set is a negative integer, so the signed
 // integer maximum with 0 leaves positive values as they are and turns negative ones and -0 into +0 (a NaN keeps its
-// bits if its sign is clear and becomes +0 otherwise).  fmaxf(v, 0.f) costs two instructions on an accumulator that
+// bits if its sign is clear and becomes +0 otherwise, where apply_act below turns every NaN into 0: the forms of a
+// network agree bit for bit on everything but NaN activations, which the parity contract leaves open).  fmaxf(v, 0.f) costs two instructions on an accumulator that
 // comes straight from a matrix instruction: the compiler first quiets a possible signalling NaN with v_max_f32 v, v
 // (it does not know that matrix results are already canonical, and it rewrites v_med3_f32(v, 0, inf) to the same
 // pair).  Written in C, not as inline assembly: the compiler then keeps its own bookkeeping of the wait states between

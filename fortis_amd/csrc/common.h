@@ -143,6 +143,7 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
 // (grown on demand, null when the device has no memory left) and the kernel that adds ksplit slices of
 // osize floats and applies the epilogue.
 float* fortis_conv_split_scratch(size_t bytes);
+void fortis_conv_forget_buffers();
 // While a workspace is set (base non-null) the packed weights of fortis_conv_mfma_pack_dev and the partial sums come
 // out of it and nothing in the convolution path allocates; fortis_conv_workspace_overflowed() is the size a
 // refused request would have needed (0: every request fitted).

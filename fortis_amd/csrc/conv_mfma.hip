@@ -638,7 +638,7 @@ static int conv_cus()
     return n;
 }
 
-// A caller-provided workspace replaces the two buffers this file otherwise grows with hipMalloc (the packed
+// A caller-provided workspace replaces the two buffers this file otherwise grows with fortis_dev_malloc (the packed
 // weights of fortis_conv_mfma_pack_dev first, the partial sums of channel-split launches behind them) until it is
 // taken away again with (null, 0).  A request that does not fit returns null, which the launchers turn into -1
 // before anything is launched, and is remembered for fortis_conv_workspace_overflowed().
@@ -655,14 +655,24 @@ static float* ws_take(size_t offset, size_t need)
 // Partial sums of channel-split launches: one buffer for every shape (launches on the library's stream run
 // one after the other).  It grows on the first, eager run of a plan; replays and captured runs find it in
 // place.  An outgrown buffer stays allocated: a graph captured earlier may still name it.
+static float* g_split = nullptr;   // the partial sums' buffer and the packed weights' one, with their sizes
+static size_t g_split_cap = 0;
+static float* g_pack = nullptr;
+static size_t g_pack_cap = 0;
+// The raw allocator was swapped (a test's hook): buffers of the old allocator are forgotten, not freed.
+void fortis_conv_forget_buffers() { g_split = g_pack = nullptr; g_split_cap = g_pack_cap = 0; }
+// Grows the partial sums' buffer ahead of time (a caller about to capture a graph; tests of the allocation
+// path): 0, or -1 when the device has no memory for it.
+extern "C" int fortis_conv_scratch_reserve(long bytes) { return bytes >= 0 && fortis_conv_split_scratch((size_t)bytes) ? 0 : -1; }
+
 float* fortis_conv_split_scratch(size_t need)
 {
     if (g_ws) return ws_take(g_ws_pack, need);
-    static float* scratch = nullptr;
-    static size_t cap = 0;
-    if (need > cap) {
+    float*& scratch = g_split;
+    size_t& cap = g_split_cap;
+    if (need > cap || !scratch) {
         float* p = nullptr;
-        if (hipMalloc((void**)&p, need) != hipSuccess) { (void)hipGetLastError(); fprintf(stderr, "fortis: no memory for %zu bytes of conv partial sums\n", need); return nullptr; }
+        if (fortis_dev_malloc((void**)&p, need, "conv partial sums") != 0) return nullptr;
         scratch = p;
         cap = need;
     }
@@ -756,8 +766,8 @@ __global__ void conv_pack_kernel(const float* __restrict__ W, float* __restrict_
 
 const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, hipStream_t st, int kg)
 {
-    static float* buf = nullptr;
-    static size_t cap = 0;
+    float*& buf = g_pack;
+    size_t& cap = g_pack_cap;
     const long FT = kg > 1 ? 32 : conv_ft(F), CC = cm_cc(T) * kg;
     const long nch = cdiv(C, CC), n = cdiv(F, FT) * nch * (CC / 2) * T * 2 * FT;
     if (g_ws) {
@@ -770,7 +780,7 @@ const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, h
     }
     if ((size_t)n * sizeof(float) > cap) {
         float* p = nullptr;
-        if (hipMalloc((void**)&p, (size_t)n * sizeof(float)) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+        if (fortis_dev_malloc((void**)&p, (size_t)n * sizeof(float), "packed conv weights") != 0) return nullptr;
         buf = p;                                   // an outgrown buffer stays: a captured graph may name it
         cap = (size_t)n * sizeof(float);
     }

@@ -57,7 +57,8 @@ void mgpuStreamSynchronize(void*) {}
 #define FORTIS_POOL 256
 typedef int (*fortis_raw_alloc_fn)(void** p, size_t n);
 typedef void (*fortis_raw_free_fn)(void* p);
-static int dev_alloc(void** p, size_t n) { return hipMalloc(p, n) == hipSuccess ? 0 : -1; }
+static long g_raw_allocs = 0;   // raw allocations asked of the device allocator since the library was loaded
+static int dev_alloc(void** p, size_t n) { g_raw_allocs++; return hipMalloc(p, n) == hipSuccess ? 0 : -1; }
 static void dev_free(void* p) { HIP_OK(hipFree(p)); }
 static fortis_raw_alloc_fn g_alloc = dev_alloc;
 static fortis_raw_free_fn g_free = dev_free;
@@ -82,7 +83,11 @@ void fortis_pool_set_allocator(fortis_raw_alloc_fn a, fortis_raw_free_fn f)
     g_alloc = a ? a : dev_alloc;
     g_free = f ? f : dev_free;
     memset(g_pool, 0, sizeof g_pool);
+    fortis_conv_forget_buffers();
 }
+// Test hook: how many times the library has asked the device for memory (every hipMalloc of the library goes
+// through one function): a call that must allocate nothing leaves the count unchanged.
+long fortis_dev_alloc_calls(void) { return g_raw_allocs; }
 // Test hook: number of slots holding a buffer, and how many of them are in use.
 void fortis_pool_stats(int* held, int* used)
 {

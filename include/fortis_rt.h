@@ -42,6 +42,10 @@ void  fortis_free(void* p);
  * policy be exercised on a machine without a GPU. */
 void  fortis_pool_set_allocator(int (*raw_alloc)(void** p, unsigned long nbytes), void (*raw_free)(void* p));
 void  fortis_pool_stats(int* held, int* used);
+/* Grows the library's buffer for the partial sums of channel-split convolutions ahead of time (it otherwise grows on
+ * the first call that needs it): 0, or -1 with a message when the device has no memory.  No reference counterpart. */
+int   fortis_conv_scratch_reserve(long bytes);
+long  fortis_dev_alloc_calls(void);   /* test hook: raw device allocations the library has made since it was loaded */
 
 /* ---- GEMM -------------------------------------------------------------------------------- */
 /* C[B][N] = A[B][K] . W[N][K]^T, fp32, beta = 0.                     runtime/fortis_rt.c:45-75

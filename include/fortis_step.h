@@ -26,6 +26,9 @@ extern "C" {
 #endif
 
 /* ================================ model plan ============================================ */
+/* ReLU is v > 0 ? v : 0 and LeakyReLU v > 0 ? v : alpha * v on finite values and infinities.  A NaN pre-activation is
+ * outside the parity contract: ReLU turns it into 0 in most kernels, while the straight-line kernels of narrow
+ * networks (all widths <= 64) take the maximum on the bit pattern and keep a NaN whose sign bit is clear. */
 enum { FORTIS_ACT_NONE = 0, FORTIS_ACT_RELU = 1, FORTIS_ACT_LEAKY = 2 };
 
 typedef struct fortis_plan fortis_plan;
@@ -224,6 +227,9 @@ void fortis_scatter(int a0, float* H0, float* H1, float* H2, float* H3, float* H
 /* Device-resident forms (arrays already in HBM; nothing is copied).  dA: device pointers in
  * descriptor order.  Asynchronous on the persistent stream. */
 /* (With fp64 arrays in the table the matching entries of dA point to doubles.) */
+/* Host cost per call: the table is looked up in a small cache by its contents; a cell list at the address and with the
+ * count of the entry's last match is compared by 1024 sampled entries (microseconds), at a new address in full
+ * (4 bytes per cell).  A list rewritten in place must change its address, its count or a sampled entry to be seen. */
 void fortis_stencil_gather_dev(const fortis_stencil_t* g, const float* const* dA, float* dX);
 void fortis_stencil_scatter_dev(const fortis_stencil_t* s, float* const* dA, const float* dY, int kk);
 /* The whole lifted step in ONE kernel: gather (g) -> MLP chain (plan p, every op a linear or a

@@ -315,6 +315,24 @@ def test_memref_conv_entries_wide_shapes(L, gpu):
         d.free()
 
 
+@pytest.mark.parametrize("stride,pad,F,K", [((2, 1, 2), (1, 1, 1), 20, 3), ((2, 2, 2), (0, 1, 0), 5, 3), ((1, 3, 2), (1, 0, 1), 4, (3, 1, 2))])
+def test_fortis_conv3d_strided_batches(L, gpu, stride, pad, F, K):
+    """fortis_conv3d takes what the reference's library path takes (runtime/fortis_rt.c:137-155: the Nd descriptor
+    carries any stride and batch): N = 2 with strides other than 1, wide and thin outputs, against the oracle."""
+    rng = np.random.default_rng(31)
+    K = (K, K, K) if isinstance(K, int) else K
+    x = rng.standard_normal((2, 6, 9, 11, 12)).astype(np.float32)
+    w = (rng.standard_normal((F, 6) + K) / np.sqrt(6 * K[0] * K[1] * K[2])).astype(np.float32)
+    ref = O.conv3d(x, w, stride=stride, pad=pad)
+    assert ref.shape[0] == 2 and min(ref.shape) > 0
+    dx, dw, dy = DevBuf(L, x), DevBuf(L, w), DevBuf(L, np.full(ref.shape, 9, np.float32))
+    L.fortis_conv3d(*_memref(dx, x.shape), *_memref(dw, w.shape), *_memref(dy, ref.shape),
+                    2, 6, 9, 11, 12, F, *K, *ref.shape[2:], *stride, *pad)
+    assert maxrel(dy.get(ref.shape), ref) < TOL
+    for d in (dx, dw, dy):
+        d.free()
+
+
 @pytest.mark.parametrize("H,chans", [(32, (8, 16, 24, 32)), (256, (32, 64, 128, 256))])
 def test_config4_unet(L, gpu, H, chans):
     case = configs.unet(H=H, chans=chans)

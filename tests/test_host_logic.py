@@ -344,3 +344,15 @@ def test_buffer_walk_that_runs_out_of_memory_fails_cleanly(pool, capfd):
     frees0 = dev.frees
     L.fortis_plan_destroy(p)
     assert stats(L)[1] == 0 and dev.frees == frees0  # handed back to the pool (still held there), none freed twice
+
+
+def test_conv_partial_sum_buffer_fails_cleanly_without_memory(pool, capfd):
+    """The convolution path's own buffers come from the same switchable allocator: a request the device cannot
+    meet prints what was asked and returns -1 (the launchers then launch nothing), a smaller one succeeds and is
+    kept, and a later request that fits the kept buffer allocates nothing."""
+    L, dev = pool                                              # 1000 bytes
+    assert L.fortis_conv_scratch_reserve(5000) == -1
+    assert "device allocation of 5000 bytes failed (conv partial sums)" in capfd.readouterr().err
+    assert L.fortis_conv_scratch_reserve(600) == 0 and dev.allocs == 1
+    assert L.fortis_conv_scratch_reserve(400) == 0 and dev.allocs == 1
+    assert L.fortis_conv_scratch_reserve(-1) == -1

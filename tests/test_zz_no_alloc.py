@@ -51,6 +51,39 @@ def test_noalloc_entry_equals_the_allocating_entry_on_two_calls_in_a_row(L, gpu)
         _both(L, x, w, check_oracle=True)
 
 
+def test_noalloc_entry_asks_the_device_for_no_memory(L, gpu):
+    """The entry's defining property: on shapes this process has not run before (larger than any above, so the
+    allocating twins would have to grow their buffers), called before the allocating entry, the count of raw device
+    allocations the library has made does not move.  The allocating entry on the same shape then does move it."""
+    rng = np.random.default_rng(23)
+    for (xs, F) in [((1, 64, 17, 19, 21), 64), ((1, 48, 10, 22, 26), 3), ((1, 12, 11, 15, 13), 24)]:
+        x = rng.standard_normal(xs).astype(np.float32)
+        w = (rng.standard_normal((F, xs[1], 3, 3, 3)) / np.sqrt(27 * xs[1])).astype(np.float32)
+        N, Cc, D, H, W = xs
+        ys = (N, F, D, H, W)
+        dx, dw, dy = DevBuf(L, x), DevBuf(L, w), DevBuf(L, np.zeros(ys, np.float32))
+        tail = [N, Cc, D, H, W, F, 3, 3, 3, D, H, W, 1, 1, 1, 1, 1, 1]
+        L.fortis_sync()
+        before = L.fortis_dev_alloc_calls()
+        rc = L.fortis_conv3d_noalloc(*_memref(dx, xs), *_memref(dw, w.shape), *_memref(dy, ys), *tail)
+        L.fortis_sync()
+        assert rc == 0 and L.fortis_dev_alloc_calls() == before, (xs, F)
+        assert maxrel(dy.get(ys), O.conv3d(x, w, pad=(1, 1, 1))) < TOL
+        for d in (dx, dw, dy):
+            d.free()
+    # the counter is live: the allocating entry on the largest of these shapes grows its buffers
+    xs, F = (1, 64, 17, 19, 21), 64
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal((F, 64, 3, 3, 3)) / np.sqrt(27 * 64)).astype(np.float32)
+    dx, dw, dy = DevBuf(L, x), DevBuf(L, w), DevBuf(L, np.zeros((1, F) + xs[2:], np.float32))
+    before = L.fortis_dev_alloc_calls()
+    L.fortis_conv3d(*_memref(dx, xs), *_memref(dw, w.shape), *_memref(dy, (1, F) + xs[2:]), 1, 64, 17, 19, 21, F, 3, 3, 3, 17, 19, 21, 1, 1, 1, 1, 1, 1)
+    L.fortis_sync()
+    assert L.fortis_dev_alloc_calls() > before
+    for d in (dx, dw, dy):
+        d.free()
+
+
 def test_noalloc_entry_refuses_what_does_not_fit_its_scratch(L, gpu, capfd):
     """64 -> 64 channels on 27 x 40 x 40 is streamed over the chip in runs of 22 chunks: up to three partial sums for
     each of its 351 tiles of 128 positions x 64 channels are 34.5 MB behind 0.44 MB of packed weights, more than the
