@@ -20,6 +20,7 @@
 // caller that gets -1 must not launch anything on the pointer.
 int  fortis_dev_malloc(void** p, size_t nbytes, const char* what);
 void fortis_dev_free(void* p);
+long fortis_pool_best_fit(long nbytes);   // size of the released pool buffer fortis_alloc(nbytes) would hand out, or -1
 bool fortis_pool_on_device();   // false while a test has replaced the raw allocator (fortis_pool_set_allocator)
 
 extern "C" long fortis_step_generation(void);   // plan.hip: count of forward passes of the bound step

@@ -382,10 +382,14 @@ static int assign_buffers(fortis_plan* p)
         int best = -1;
         for (size_t b = 0; b < p->bufs.size(); b++)
             if (bfree[b] && bsize[b] >= n && (best < 0 || bsize[b] < bsize[best])) best = (int)b;
+        // a buffer the pool holds unused (left by a plan destroyed earlier) that fits more tightly is taken instead,
+        // as the pool's own best fit over all released buffers would
+        const long pool_fit = fortis_pool_best_fit(n);
+        if (best >= 0 && pool_fit >= 0 && pool_fit < bsize[best]) best = -1;
         if (best < 0) {
             void* d = fortis_alloc(n);
             if (!d) { rc = -1; return; }
-            p->bufs.push_back(d); bsize.push_back(n); bfree.push_back(0);
+            p->bufs.push_back(d); bsize.push_back(pool_fit >= 0 ? pool_fit : n); bfree.push_back(0);   // a released pool buffer keeps its own size
             best = (int)p->bufs.size() - 1;
         }
         bfree[best] = 0;

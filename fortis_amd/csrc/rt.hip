@@ -75,6 +75,13 @@ int fortis_dev_malloc(void** p, size_t nbytes, const char* what)
 }
 void fortis_dev_free(void* p) { if (p) g_free(p); }
 bool fortis_pool_on_device() { return g_alloc == dev_alloc; }
+long fortis_pool_best_fit(long n)
+{
+    long best = -1;
+    for (int i = 0; i < FORTIS_POOL; i++)
+        if (g_pool[i].p && !g_pool[i].used && g_pool[i].n >= n && (best < 0 || g_pool[i].n < best)) best = g_pool[i].n;
+    return best;
+}
 
 extern "C" {
 // Test hook: replaces the raw allocator (null restores hipMalloc/hipFree) and empties the pool table.
