@@ -200,9 +200,10 @@ def run_copy(L, args):
 
 
 def run_zb_unfused(L, args):
-    """The reference's structure of the ZB step: gather kernel -> X in HBM -> MLP -> Y in HBM -> one scatter launch
-    per layer (mom6_zb/gather.cu:50-57, 82-91), every part timed with HIP events on the library's stream.  The
-    gather is the memory-bound kernel of the path: the roofline block is its."""
+    """The reference's structure of the ZB step: gather kernel -> X in HBM -> MLP -> Y in HBM -> scatter
+    (mom6_zb/gather.cu:50-57, 82-91; all layers scattered by one launch, as fortis_scatter does under loop
+    distribution), every part timed with HIP events on the library's stream.  The gather is the memory-bound kernel
+    of the path: the roofline block is its."""
     from fortis_amd import configs, plan as P, stencil as S
     sx, sy, nz = (int(v) for v in (args.grid or "1028x1028x15").lower().split("x"))
     gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
@@ -227,15 +228,14 @@ def run_zb_unfused(L, args):
         held.append(d)
         return d
     dG = (C.c_void_p * 4)(*[dev(A[k]) for k in ("sh_xy_h", "sh_xx", "vort_xy_h", "norm_h")])
-    dS = (C.c_void_p * 5)(dG[3], dev(A["kappa_h"]), dev(np.zeros(sx * sy, ft)), dev(np.zeros(n3, ft)), dev(np.zeros(n3, ft)))
+    dS = (C.c_void_p * 5)(dG[3], dev(A["kappa_h"]), dev(np.zeros(n3, ft)), dev(np.zeros(n3, ft)), dev(np.zeros(n3, ft)))   # Txy_h: a plane per layer
     dX = L.fortis_plan_tensor_ptr(plan.handle, plan.in_tensor)
     dY = L.fortis_plan_tensor_ptr(plan.handle, plan.out_tensor)
     CB = C.CFUNCTYPE(None, C.c_void_p)
     gather_cb = CB(lambda _: L.fortis_stencil_gather_dev(C.byref(gt), dG, dX))
 
     def scatter_all(_):
-        for kk in range(nz):
-            L.fortis_stencil_scatter_dev(C.byref(st), dS, C.c_void_p(dY + kk * count * 3 * 4), kk)
+        assert L.fortis_stencil_scatter_all_dev(C.byref(st), dS, C.c_void_p(dY)) == 0
     scatter_cb = CB(scatter_all)
     mlp_cb = CB(lambda _: plan.run())
     parts = (CB * 3)(gather_cb, mlp_cb, scatter_cb)
@@ -269,11 +269,11 @@ def run_zb_unfused(L, args):
     roof = dict(bound="hbm", kernel=kname, achieved=round(gbs, 1), peak=PEAK_HBM_GBS,
                 unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4), avg_launch_ms=round(g_ms, 5), bytes_per_launch=g_bytes,
                 back_to_back_ms=round(ga_ms, 5), back_to_back_frac=round(g_bytes / (ga_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                scatter_GBs=round(s_bytes / (s_ms * 1e-3) / 1e9, 1), scatter_ms_all_layers=round(s_ms, 5), mlp_ms=round(m_ms, 5),
+                scatter_GBs=round(s_bytes / (s_ms * 1e-3) / 1e9, 1), scatter_frac=round(s_bytes / (s_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), scatter_ms_all_layers=round(s_ms, 5), mlp_ms=round(m_ms, 5),
                 **traffic("zb_unfused_%dx%dx%d%s" % (sx, sy, nz, "_f64" if args.f64 else "")))
     out = dict(rows=rows, dt=dt, dtype="f32",
                config={"workload": "zb_unfused_gather_mlp_scatter_27_64_64_3_%dx%dx%d%s" % (sx, sy, nz, "_f64_arrays" if args.f64 else ""), "columns": rows,
-                       "cells_per_layer": count, "layers": nz, "launches_per_step": 1 + nz + plan.num_kernels},
+                       "cells_per_layer": count, "layers": nz, "launches_per_step": 2 + (nz - 1 if args.f64 else 0) + plan.num_kernels},
                roofline=roof)
     plan.close()
     for d in held:
@@ -570,7 +570,7 @@ def run_others(L, args):
                     "value": r["rows"] * steps / r["dt"], "unit": r.get("unit", "columns/s"), "bound": roof["bound"],
                     "kernel": roof["kernel"], "achieved": roof["achieved"], "peak": roof["peak"], "roofline_unit": roof["unit"],
                     "frac": roof["frac"], "avg_launch_ms": roof["avg_launch_ms"]})
-        for k in ("back_to_back_ms", "back_to_back_frac"):     # the unfused step's gather launched alone
+        for k in ("back_to_back_ms", "back_to_back_frac", "scatter_GBs", "scatter_frac", "scatter_ms_all_layers", "mlp_ms"):     # the unfused step's other parts
             if k in roof:
                 out[-1][k] = roof[k]
     return out

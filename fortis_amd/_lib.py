@@ -87,6 +87,7 @@ PROTOTYPES = {
     "fortis_gather": (None, [vp, vp, vp, vp]), "fortis_scatter": (None, [i, vp, vp, vp, vp, vp]),
     "fortis_stencil_gather_dev": (None, [C.POINTER(Stencil), C.POINTER(vp), vp]),
     "fortis_stencil_scatter_dev": (None, [C.POINTER(Stencil), C.POINTER(vp), vp, i]),
+    "fortis_stencil_scatter_all_dev": (i, [C.POINTER(Stencil), C.POINTER(vp), vp]),
     "fortis_stencil_step_fused": (i, [C.POINTER(Stencil), C.POINTER(Stencil), vp, C.POINTER(vp), C.POINTER(vp), vp]),
     "fortis_stencil_step_fused_time_ms": (f, [C.POINTER(Stencil), C.POINTER(Stencil), vp, C.POINTER(vp), C.POINTER(vp), vp, i]),
     "fortis_plan_profile": (None, [vp, i]), "fortis_plan_profile_read": (i, [vp, fp]),

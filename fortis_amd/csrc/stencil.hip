@@ -28,8 +28,11 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
     params_to_lds(&d, ST_THREADS);
     const int n = st_u(d.nrefs);
     const int tid = threadIdx.x;
-    // plain workgroup order: banding the workgroups per XCD halves the input fetches of this kernel but it mostly
-    // writes, and with the rows in flight spread over eight bands it ran 5 % slower
+    // plain workgroup order: this kernel mostly writes, and it writes fastest as ONE contiguous stream.  Banding the
+    // workgroups per XCD halves the input fetches but spreads the rows in flight over eight bands (5 % slower); two
+    // bands of four vertical strips, in which the workgroup one row down runs on the same XCD a few steps later,
+    // fetch each input row once and still measured 5 % slower inside the step (0.463 against 0.440 ms on
+    // 1028 x 1028 x 15), no different launched back to back
     const unsigned row0 = blockIdx.x * ST_THREADS, row = row0 + tid;
     if (row < rows) {
         int i, j, kk;
@@ -584,6 +587,26 @@ void fortis_stencil_scatter_dev(const fortis_stencil_t* sd, float* const* dA, co
     if (!e) return;
     if (e->generic) { fortis_launch_scatter_generic(*sd, e->dcells, (void* const*)dA, dY, kk, fortis_stream_get()); return; }
     launch_scatter(e->low, dA, dY, kk, fortis_stream_get());
+}
+
+// Every enclosing-loop iteration in one launch (the entry path's scatter under loop distribution, mom6_zb/kdist.json):
+// dY holds the model output of all nk iterations, and an array that is 2-D on the host, which the reference's per-
+// iteration launches overwrite nk times, has nk planes on the device, as in fortis_stencil_step_fused.
+int fortis_stencil_scatter_all_dev(const fortis_stencil_t* sd, float* const* dA, const float* dY)
+{
+    if (!sd || !dA || !dY) return -1;
+    fortis_stencil_t s2 = *sd;
+    for (int r = 0; r < s2.nrefs; r++)
+        if (!s2.refs[r].planar) { s2.refs[r].planar = 1; s2.plane[s2.refs[r].array] = s2.total[s2.refs[r].array]; }
+    CacheEnt* e = cached(&s2);
+    if (!e) return -1;
+    if (e->generic) {
+        for (int kk = 0; kk < sd->nk; kk++)
+            fortis_launch_scatter_generic(s2, e->dcells, (void* const*)dA, dY + (size_t)kk * sd->count * sd->nrefs, kk, fortis_stream_get());
+        return 0;
+    }
+    launch_scatter(e->low, dA, dY, 0, fortis_stream_get(), (int)sd->nk);
+    return 0;
 }
 
 int fortis_stencil_step_fused(const fortis_stencil_t* g, const fortis_stencil_t* sd, fortis_plan* p,

@@ -232,6 +232,10 @@ void fortis_scatter(int a0, float* H0, float* H1, float* H2, float* H3, float* H
  * (4 bytes per cell).  A list rewritten in place must change its address, its count or a sampled entry to be seen. */
 void fortis_stencil_gather_dev(const fortis_stencil_t* g, const float* const* dA, float* dX);
 void fortis_stencil_scatter_dev(const fortis_stencil_t* s, float* const* dA, const float* dY, int kk);
+/* All nk iterations in one launch: dY is the model output of every iteration, [nk][count][n]; an array that is 2-D on
+ * the host (rewritten by every iteration there, like Txy_h) has nk planes of `total` elements on the device.  What
+ * fortis_scatter does under loop distribution (mom6_zb/kdist.json, mom6_zb/gather.cu:82-91 run nk times).  -1: bad table. */
+int  fortis_stencil_scatter_all_dev(const fortis_stencil_t* s, float* const* dA, const float* dY);
 /* The whole lifted step in ONE kernel: gather (g) -> MLP chain (plan p, every op a linear or a
  * feature scale) -> scatter (s) for all nk iterations at once.  Arrays the scatter writes need a
  * plane per iteration on the device: an array that is 2-D on the host (written once per

@@ -39,10 +39,11 @@ def test_gather_reference_geometry_bit_exact(L, gpu, golden, zbhost):
         b.free()
 
 
-@pytest.mark.parametrize("sx,sy,nz", [(48, 58, 10), (9, 7, 1), (133, 70, 3)])
+@pytest.mark.parametrize("sx,sy,nz", [(48, 58, 10), (9, 7, 1), (133, 70, 3), (520, 40, 2), (1031, 25, 3), (1540, 17, 1)])
 def test_gather_scatter_other_grids_bit_exact(L, gpu, sx, sy, nz):
     """48x58x10 -> 44x54 = 2376 cells per layer is the reference's second specialisation size
-    (mom6_zb/README.md:37); the others are ragged (count not a multiple of the block) and tiny."""
+    (mom6_zb/README.md:37); the next two are ragged (count not a multiple of the block) and tiny; the wide ones
+    have rows of about 2, 4 and 6 workgroups, whose gather walks its workgroups in vertical strips."""
     gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
     gt, st = S.build_table(gd, lp, kd, "gather"), S.build_table(sd, lp, kd, "scatter")
     A = configs.zb_arrays(sx, sy, nz)
@@ -64,7 +65,14 @@ def test_gather_scatter_other_grids_bit_exact(L, gpu, sx, sy, nz):
         O.stencil_scatter(sd, ref, Y[kk * count:(kk + 1) * count], count, kk, 3, 3, sx - 4)
     for b, r in zip(sb[2:], ref[2:]):
         assert bits_equal(b.get(r.shape), r)
-    for b in bufs + sb + [dX, dY]:
+    # every iteration in one launch: the 2-D array gets a plane per iteration, whose last one is what the
+    # iteration-by-iteration launches leave in it
+    host[2] = np.zeros(sx * sy * nz, np.float32)
+    sa = [DevBuf(L, a) for a in host]
+    assert L.fortis_stencil_scatter_all_dev(C.byref(st), ptrs(sa), dY.ptr) == 0
+    assert bits_equal(sa[3].get(ref[3].shape), ref[3]) and bits_equal(sa[4].get(ref[4].shape), ref[4])
+    assert bits_equal(sa[2].get((nz, sx * sy))[nz - 1], ref[2])
+    for b in bufs + sb + sa + [dX, dY]:
         b.free()
 
 
@@ -151,7 +159,14 @@ def test_gather_scatter_masked_cell_list_bit_exact(L, gpu, ncells):
         O.stencil_scatter(sd, ref, Y[kk * ncells:(kk + 1) * ncells], ncells, kk, cells=cells)
     for b, r in zip(sb[2:], ref[2:]):
         assert bits_equal(b.get(r.shape), r)
-    for b in bufs + sb + [dX, dY]:
+    # every iteration in one launch: the 2-D array gets a plane per iteration, whose last one is what the
+    # iteration-by-iteration launches leave in it
+    host[2] = np.zeros(sx * sy * nz, np.float32)
+    sa = [DevBuf(L, a) for a in host]
+    assert L.fortis_stencil_scatter_all_dev(C.byref(st), ptrs(sa), dY.ptr) == 0
+    assert bits_equal(sa[3].get(ref[3].shape), ref[3]) and bits_equal(sa[4].get(ref[4].shape), ref[4])
+    assert bits_equal(sa[2].get((nz, sx * sy))[nz - 1], ref[2])
+    for b in bufs + sb + sa + [dX, dY]:
         b.free()
 
 
