@@ -87,9 +87,19 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     constexpr int PADK = KS / 2;
     constexpr int TH = MT / 32, R2 = (TH + 2) * CM_TP;           // TILE2D: rows per tile, staged elements per channel
     static_assert(!TILE2D || (KD == 1 && KS == 3), "the 2-D tiling is for 3 x 3 convs");
+    // XDUMP: a chunk's stores into LDS are unconditional -- an input element that is padding sends its (unused) value to
+    // a spare slot behind the buffer's staged elements instead of being masked off, and the weights' buffer is padded
+    // to whole rounds of the workgroup's 16-byte stores (WCHP; the padding receives copies of the chunk's first
+    // weights and is never read).  One select per element and tile, where a mask costs a save, a branch and a restore
+    // of the lane mask per element and chunk; and a steady-state step without branches is one block of code whose
+    // loads and stores the scheduler can place between the matrix instructions (step_full).  Not in the form that runs
+    // four workgroups per CU (its registers have none to spare for the addresses, its LDS none for the padding), nor
+    // in the streamed one with 16 staging rounds.
+    constexpr bool XDUMP = SK ? NX <= 8 : !(KD == 3 && MT == 128 && FT == 64 && NX <= 8);
+    constexpr int WCHP = XDUMP ? NW * CM_THREADS * 4 : WCH;      // floats of LDS per weight buffer
     extern __shared__ float4 smem4[];
-    float* sW = (float*)smem4;                                    // [2][WCH]
-    float* sX = sW + 2 * WCH;                                     // [2][CC * KD * R rounded up to a wave's 64 lanes]
+    float* sW = (float*)smem4;                                    // [2][WCHP]
+    float* sX = sW + 2 * WCHP;                                    // [2][CC * KD * R rounded up to a wave's 64 lanes]
     const int RR = TILE2D ? R2 : KS == 1 ? MT : s.R;              // staged elements per channel and kd (s.R, a constant where it can be)
     const int XCH = CC * KD * RR;
     const int XCHP = (XCH + 64) / 64 * 64;                        // at least one spare slot behind the staged elements (see XDUMP)
@@ -144,18 +154,26 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     };
     // the first chunk's weights need nothing of the staging map below: they are on their way while it is worked out
     load_weights(rg[0], ch0);
+    // So are the epilogue's per-channel scale and shift for this workgroup's FT channels, which wait in LDS from the
+    // first barrier on: fetched in the epilogue they cost every launch a round trip to memory after its last matrix
+    // instruction.  (Not in the form that fills the CU's LDS with four workgroups, nor in the streamed one, whose
+    // epilogue is the reduce kernel's.)
+    constexpr bool EPILDS = !SK && !(KD == 3 && MT == 128 && FT == 64 && NX <= 8);
+    __shared__ float sEpi[EPILDS ? 2 * FT : 1];
+    float epi_sc = 1.f, epi_sf = 0.f;
+    if constexpr (EPILDS) {
+        if (tid < FT && s.ksplit == 1) {
+            const int f = fg * FT + tid, fc = f < s.F ? f : 0, fo = s.mode ? fc >> 2 : fc;
+            if (e.scale) epi_sc = e.scale[fo];
+            if (e.shift) epi_sf = e.shift[fo];
+        }
+    }
 
     // per-thread staging map of the input run (same for every chunk): byte offset inside a chunk's channel
     // group, (c * schan + offset in the channel) * 4.  Padding elements load from offset 0 (goff) and carry
     // the mark 0xffffffff in gchk, which the store compares with the chunk's limit.
     unsigned goff[NX], gchk[NX];
     bool inb[NX];                // the element lies inside the tensor (not padding, not past the staged run)
-    // XDUMP: a chunk's store is unconditional -- an element that is padding sends its (unused) value to the spare slot
-    // behind the buffer's staged elements instead of being masked off.  One select per element and tile, where the
-    // mask cost a save, a branch and a restore of the lane mask per element and chunk.  Not in the form that runs
-    // four workgroups per CU, nor in the streamed one with 16 staging rounds: their registers have none to spare for
-    // the addresses.
-    constexpr bool XDUMP = SK ? NX <= 8 : !(KD == 3 && MT == 128 && FT == 64 && NX <= 8);
     unsigned xslot[XDUMP ? NX : 1];
 #pragma unroll
     for (int i = 0; i < NX; i++) {
@@ -217,11 +235,11 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     // where a select of the value against zero cost two).  Only a partial last chunk still selects: its channels past
     // the last one store zeros.
     auto store_chunk = [&](const Regs& r, int buf, int ch) {
-        cm_v4f* wdst = (cm_v4f*)(sW + buf * WCH);
+        cm_v4f* wdst = (cm_v4f*)(sW + buf * WCHP);
 #pragma unroll
         for (int i = 0; i < NW; i++) {
             const int f4 = tid + i * CM_THREADS;
-            if (f4 < WCH / 4) wdst[f4] = r.rw[i];
+            if (XDUMP || f4 < WCH / 4) wdst[f4] = r.rw[i];
         }
         float* xdst = sX + buf * XCHP + tid;
         if ((ch + 1) * CC <= s.C) {
@@ -262,7 +280,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
     auto multiply = [&](int buf) {
-        const float* w = sW + buf * WCH + wbase;
+        const float* w = sW + buf * WCHP + wbase;
         const float* xs = sX + buf * XCHP + xbase;
 #pragma unroll
         for (int cp = 0; cp < NCPW; cp++)
@@ -284,7 +302,54 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     // chunk ch + 1 from `near` into the other LDS buffer.  The steady-state form is unconditional: the
     // compiler's wait insertion counts loads behind a branch as possibly absent and would then wait for
     // the newest loads where only the oldest are needed.
+    // (only where a wave is alone or nearly alone on its SIMD: the forms whose four waves divide the input channels,
+    // at one or two workgroups per CU.  With three or four waves per SIMD the other waves fill those gaps anyway and
+    // the block order with the multiply phase at raised priority measured 2-3 % faster.)
+    constexpr bool INTERLEAVE = XDUMP && KG == 4;
     auto step_full = [&](int ch, int buf, Regs& far, const Regs& near) {
+        if constexpr (INTERLEAVE) {
+            // Neither chunk ch + 1 nor ch + 2 is a partial one here (the loop below sees to it), so the step has no
+            // branch: the loads of chunk ch + 2 and the stores of chunk ch + 1 (into the LDS buffer nobody reads during
+            // this step) are spread between the matrix instructions.  Issued in a block in front of and behind them,
+            // a workgroup's 25 KB of loads hold its four waves at the CU's one address unit for 400-500 cycles and the
+            // stores for 300-400, beside 1152 cycles of matrix work per chunk: a wave alone on its SIMD multiplied
+            // half the time.
+            load_weights(far, ch + 2);
+            {
+                const char* xsrc = (const char*)(x + (long)(ch + 2) * CC * schan);
+#pragma unroll
+                for (int i = 0; i < NX; i++) far.rx[i] = *(const float*)(xsrc + goff[i]);
+            }
+            multiply(buf);
+            {
+                cm_v4f* wdst = (cm_v4f*)(sW + (buf ^ 1) * WCHP);
+#pragma unroll
+                for (int i = 0; i < NW; i++) wdst[tid + i * CM_THREADS] = near.rw[i];
+                float* xb = sX + (buf ^ 1) * XCHP;
+#pragma unroll
+                for (int i = 0; i < NX; i++) xb[xslot[i]] = near.rx[i];
+            }
+            constexpr int NMF = NCPW * T * NMT, NMOVE = NW + NX;          // matrix instructions; loads = stores
+            // loads behind the first matrix instructions, stores behind the later ones, evenly
+#pragma unroll
+            for (int m = 0; m < NMF; m++) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);        // LDS reads (operands a little ahead)
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        // one matrix instruction
+                constexpr int H = NMF / 2;
+                if (m < H) {
+                    const int a = m * NMOVE / H, b = (m + 1) * NMOVE / H;
+                    if (b - a >= 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    if (b - a >= 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    if (b - a >= 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                } else {
+                    const int a = (m - H) * NMOVE / (NMF - H), b = (m - H + 1) * NMOVE / (NMF - H);
+                    if (b - a >= 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                    if (b - a >= 2) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                    if (b - a >= 3) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                }
+            }
+            cm_lds_barrier();
+        } else {
         load_chunk(far, ch + 2);
         __builtin_amdgcn_sched_barrier(0);     // nothing of the store below (it waits for `near`) moves above the multiplies
         // the multiply phase outranks the other resident waves' staging at the issue port (UNet 0.266 -> 0.262 ms)
@@ -294,6 +359,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         __builtin_amdgcn_sched_barrier(0);
         store_chunk(near, buf ^ 1, ch + 1);
         cm_lds_barrier();
+        }
     };
     auto step_tail = [&](int ch, int buf, Regs& far, const Regs& near) {
         if (ch + 2 < ch1) load_chunk(far, ch + 2);
@@ -307,11 +373,17 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     };
     load_input(rg[0], ch0);
     zero_padding();
+    if constexpr (EPILDS) {
+        if (tid < FT) { sEpi[tid] = epi_sc; sEpi[FT + tid] = epi_sf; }
+    }
     store_chunk(rg[0], 0, ch0);
     cm_lds_barrier();
     load_chunk(rg[1], ch0 + 1 < ch1 ? ch0 + 1 : ch0);     // unconditional for the same reason (a lone chunk is fetched twice)
     int ch = ch0;
-    for (; ch + 3 < ch1; ch += 2) {
+    // the unconditional steps stop short of a partial last chunk (fewer than CC channels left), which only
+    // the tail steps load and store
+    const int chfull = INTERLEAVE && s.nchunks * CC > s.C && ch1 == s.nchunks ? ch1 - 1 : ch1;
+    for (; ch + 3 < chfull; ch += 2) {
         step_full(ch, 0, rg[0], rg[1]);
         step_full(ch + 1, 1, rg[1], rg[0]);
     }
@@ -367,13 +439,19 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         float t[N];
         if (e.scale) {
 #pragma unroll
-            for (int q = 0; q < N; q++) t[q] = e.scale[fo[q]];
+            for (int q = 0; q < N; q++) {
+                const int r = r0 + q;
+                t[q] = EPILDS ? sEpi[ft * 32 + 4 * (lane >> 5) + 8 * (r >> 2) + (r & 3)] : e.scale[fo[q]];
+            }
 #pragma unroll
             for (int q = 0; q < N; q++) v[q] = v[q] * t[q];
         }
         if (e.shift) {
 #pragma unroll
-            for (int q = 0; q < N; q++) t[q] = e.shift[fo[q]];
+            for (int q = 0; q < N; q++) {
+                const int r = r0 + q;
+                t[q] = EPILDS ? sEpi[FT + ft * 32 + 4 * (lane >> 5) + 8 * (r >> 2) + (r & 3)] : e.shift[fo[q]];
+            }
 #pragma unroll
             for (int q = 0; q < N; q++) v[q] = v[q] + t[q];
         }
@@ -803,15 +881,20 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     }
     s.mP = st_magic((unsigned)s.P); s.mR = st_magic((unsigned)s.R); s.mKR = st_magic((unsigned)(KD * s.R));
     s.mT = st_magic((unsigned)s.tiles); s.mTX = st_magic((unsigned)(TILE2D ? s.tiles_x : 1)); s.mNC = st_magic((unsigned)s.nchunks); s.mPer = st_magic(1u);
-    size_t shmem = (size_t)2 * (CC * T * FT + ((long)CC * KD * s.R + 64) / 64 * 64) * sizeof(float);
+    // the kernel's weight buffers are padded to whole rounds of 16-byte stores in its forms with unconditional stores
+    constexpr int WCH = CC * T * FT, WCHPAD = (WCH / 4 + CM_THREADS - 1) / CM_THREADS * CM_THREADS * 4;
+    constexpr bool four_per_cu = KD == 3 && MT == 128 && FT == 64 && NX <= 8;
+    const size_t xchp = (size_t)(((long)CC * KD * s.R + 64) / 64 * 64);
+    size_t shmem = (size_t)2 * ((four_per_cu ? WCH : WCHPAD) + xchp) * sizeof(float);
+    const size_t shmem_sk = (size_t)2 * ((NX <= 8 ? WCHPAD : WCH) + xchp) * sizeof(float);      // the streamed form's
     if (KG > 1 && shmem < 4 * 16 * 64 * sizeof(float)) shmem = 4 * 16 * 64 * sizeof(float);  // (4 / KG tiles) x KG groups x 16 registers x 64 lanes   // the groups' sums meet in LDS
     if (POOL && shmem < (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float)) shmem = (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float);   // the finished tile, for its 2 x 2 max pool
-    if (shmem > 160 * 1024) return -1;
+    if (shmem > 160 * 1024 || shmem_sk > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
         HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
         if constexpr (KD == 3 && KG == 1 && !POOL && !TILE2D)
-            HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+            HIP_OK(hipFuncSetAttribute((const void*)conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem_sk));
         attr = shmem;
     }
     // A launch that leaves most CUs idle (deep, small images) is split over the input channels: each
@@ -860,7 +943,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
                     hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL>), dim3((unsigned)tile0, (unsigned)nfg, 1), dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
                     HIP_OK(hipGetLastError());
                 }
-                hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL, true>), dim3((unsigned)cdiv(items, per), (unsigned)nfg, 1), dim3(CM_THREADS), shmem, st, x, wp, y, s, e);
+                hipLaunchKernelGGL((conv_mfma_kernel<KD, KS, MT, FT, NX, TILE2D, KG, POOL, true>), dim3((unsigned)cdiv(items, per), (unsigned)nfg, 1), dim3(CM_THREADS), shmem_sk, st, x, wp, y, s, e);
                 HIP_OK(hipGetLastError());
                 hipLaunchKernelGGL((conv_sk_reduce_kernel<MT, FT>), dim3((unsigned)(ntiles - tile0), (unsigned)nfg, (MT / 32 / (4 / (FT / 32))) * 4 / CM_RQB), dim3(CM_THREADS), 0, st, y, s, e);
                 HIP_OK(hipGetLastError());
