@@ -672,8 +672,12 @@ void chain_wave_kernel(ChainParams params)
 // loop: the lane's eight slot pointers stay in registers for the life of the (persistent) wave, scalar and store
 // pointers and all strides are wave-uniform scalar registers, a cell is decoded once and its element offsets are
 // 32-bit, and the expression interpreter looks at two scalars and two per-cell results instead of four and six.
-template <bool WLDS, int SIG = 0>
-__global__ __launch_bounds__(CH_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)))
+// PF: the next tile's loads are issued before the current tile is processed (two sets of tile inputs in registers:
+// four waves per SIMD).  Without it the kernel fits five waves per SIMD, which is what a launch of a little more than
+// four tiles per SIMD wants: each tile then has a wave of its own and no wave runs a second tile after the others
+// have finished.
+template <bool WLDS, int SIG = 0, bool PF = true>
+__global__ __launch_bounds__(CH_THREADS) __attribute__((amdgpu_waves_per_eu(PF ? 4 : 5, PF ? 4 : 5)))
 void chain_stencil_fast_kernel(ChainParams params)
 {
     constexpr int NS = 2, NC = 2;
@@ -693,9 +697,9 @@ void chain_stencil_fast_kernel(ChainParams params)
     const gfloat* in_div = st_g(d.in_div);
     const gfloat* out_mul = st_g(d.out_mul);
     // ---- hoisted table values -------------------------------------------------------------------------------
-    const gfloat* gp[8];                                   // this lane's slots q = 16 (t / 4) + 4 lq + t % 4
+    const gfloat* gp[PF ? 8 : 1];                          // this lane's slots q = 16 (t / 4) + 4 lq + t % 4
 #pragma unroll
-    for (int t = 0; t < 8; t++) gp[t] = st_g(g.refs[16 * (t >> 2) + 4 * lq + (t & 3)].p);
+    for (int t = 0; t < (PF ? 8 : 1); t++) gp[t] = st_g(g.refs[16 * (t >> 2) + 4 * lq + (t & 3)].p);   // (without prefetch: read per tile)
     const unsigned g_si = (unsigned)st_u(g.refs[0].si), g_sj = (unsigned)st_u(g.refs[0].sj), g_pl = (unsigned)st_u((int)g.refs[0].plane);
     const unsigned o_si = (unsigned)st_u(sc.refs[0].si), o_sj = (unsigned)st_u(sc.refs[0].sj), o_pl = (unsigned)st_u((int)sc.refs[0].plane);
     const bool o_as_g = g_si == o_si && g_sj == o_sj && g_pl == o_pl;
@@ -723,7 +727,7 @@ void chain_stencil_fast_kernel(ChainParams params)
         const unsigned goff = (unsigned)i * g_si + (unsigned)j * g_sj + (unsigned)kk * g_pl;
         in.soff = o_as_g ? goff : (unsigned)i * o_si + (unsigned)j * o_sj + (unsigned)kk * o_pl;
 #pragma unroll
-        for (int t = 0; t < 8; t++) in.x[t] = gp[t][goff];
+        for (int t = 0; t < 8; t++) in.x[t] = (PF ? gp[PF ? t : 0] : st_g(g.refs[16 * (t >> 2) + 4 * lq + (t & 3)].p))[goff];
 #pragma unroll
         for (int q = 0; q < NS; q++) in.gS[q] = gsp[q][goff];
 #pragma unroll
@@ -734,12 +738,13 @@ void chain_stencil_fast_kernel(ChainParams params)
     };
     // the input divisors of the lane's eight slots: the same for every tile, loaded once (slots past the network's
     // inputs take slot 0's; their quotients are replaced by zero)
-    float dv[8];
+    // (the form without prefetch has no registers for them and reads them per tile)
+    float dv[PF ? 8 : 1];
 #pragma unroll
-    for (int t = 0; t < 8; t++) dv[t] = 1.f;
-    if (in_div) {
+    for (int t = 0; t < (PF ? 8 : 1); t++) dv[t] = 1.f;
+    if (PF && in_div) {
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
+        for (int t = 0; t < (PF ? 8 : 1); t++) {
             const int q = 16 * (t >> 2) + 4 * lq + (t & 3);
             dv[t] = in_div[q < K0 ? q : 0];
         }
@@ -766,7 +771,8 @@ void chain_stencil_fast_kernel(ChainParams params)
 #pragma unroll
                 for (int t = 0; t < 8; t++) {
                     const int q = 16 * (t >> 2) + 4 * lq + (t & 3);
-                    a[t >> 2][t & 3] = (valid && q < K0) ? __fdiv_rn(tv[t], dv[t]) : 0.f;
+                    const float dq = PF ? dv[PF ? t : 0] : (float)in_div[q < K0 ? q : 0];
+                    a[t >> 2][t & 3] = (valid && q < K0) ? __fdiv_rn(tv[t], dq) : 0.f;
                 }
             }
             a[2] = a[3] = (v4f)(0.f);
@@ -816,7 +822,7 @@ void chain_stencil_fast_kernel(ChainParams params)
     } else {
         t = (unsigned long long)blockIdx.x * 4 + wave; tend = ntile; stride = (unsigned long long)gridDim.x * 4;
     }
-    TileIn cur, nxt;
+    TileIn cur;
     if (t < tend) issue(cur, (unsigned)(t * 16));       // in flight while the weights are staged
     if (WLDS) {
         const int n4 = wfloats / 4;
@@ -829,12 +835,21 @@ void chain_stencil_fast_kernel(ChainParams params)
         }
         __syncthreads();
     }
-    for (; t < tend; t += stride) {
-        asm volatile("" ::: "memory");
-        const bool more = t + stride < tend;
-        if (more) issue(nxt, (unsigned)((t + stride) * 16));
-        process(cur);
-        if (more) cur = nxt;
+    if constexpr (PF) {
+        TileIn nxt;
+        for (; t < tend; t += stride) {
+            asm volatile("" ::: "memory");
+            const bool more = t + stride < tend;
+            if (more) issue(nxt, (unsigned)((t + stride) * 16));
+            process(cur);
+            if (more) cur = nxt;
+        }
+    } else {
+        for (; t < tend; t += stride) {
+            asm volatile("" ::: "memory");
+            process(cur);
+            if (t + stride < tend) issue(cur, (unsigned)((t + stride) * 16));
+        }
     }
 }
 
@@ -1267,20 +1282,38 @@ static bool stencil_fast_ok(const ChainParams& P, const StencilDev& g, const Ste
     return fits(g) && fits(sc);
 }
 
+template <bool WLDS, int SIG = 0, bool PF = true>
+static long stencil_fast_slots(size_t shmem)
+{
+    static size_t attr = 0;
+    static long slots = 0;
+    if (shmem > attr || !slots) {
+        HIP_OK(hipFuncSetAttribute((const void*)chain_stencil_fast_kernel<WLDS, SIG, PF>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
+        attr = shmem;
+        int occ = 0;
+        HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void*)chain_stencil_fast_kernel<WLDS, SIG, PF>, CH_THREADS, shmem));
+        slots = (long)(occ < 1 ? 1 : occ) * num_cus();
+    }
+    return slots;
+}
 template <bool WLDS, int SIG = 0>
 static void launch_stencil_fast(ChainParams& P, hipStream_t s)
 {
     const size_t shmem = (size_t)(WLDS ? P.d.wfloats : 0) * sizeof(float);
-    static size_t attr = 0;
-    static long slots = 0;
-    if (shmem > attr || !slots) {
-        HIP_OK(hipFuncSetAttribute((const void*)chain_stencil_fast_kernel<WLDS, SIG>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem));
-        attr = shmem;
-        int occ = 0;
-        HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, (const void*)chain_stencil_fast_kernel<WLDS, SIG>, CH_THREADS, shmem));
-        slots = (long)(occ < 1 ? 1 : occ) * num_cus();
-    }
+    const long slots = stencil_fast_slots<WLDS, SIG, true>(shmem);
     long grid = cdiv(P.rows, 64);
+    static const int pf_only = getenv("FORTIS_STENCIL_PF") != nullptr;
+    if (WLDS && grid > slots && !pf_only) {
+        // more tiles than the prefetching form has waves: if the form with five waves per SIMD holds them all at
+        // once, every tile gets a wave of its own (the grid rounded up to whole rounds of the eight XCDs)
+        const long slots5 = stencil_fast_slots<WLDS, SIG, false>(shmem);
+        if (grid <= slots5) {
+            grid = (grid + 7) / 8 * 8;
+            hipLaunchKernelGGL((chain_stencil_fast_kernel<WLDS, SIG, false>), dim3((unsigned)(grid < slots5 ? grid : slots5)), dim3(CH_THREADS), shmem, s, P);
+            HIP_OK(hipGetLastError());
+            return;
+        }
+    }
     if (grid > slots) grid = slots;
     hipLaunchKernelGGL((chain_stencil_fast_kernel<WLDS, SIG>), dim3((unsigned)grid), dim3(CH_THREADS), shmem, s, P);
     HIP_OK(hipGetLastError());
