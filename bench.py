@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused inference step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload climsim|zb|zb_ref|zb_unfused|toy|unet|tsrgan|copy] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload climsim|zb|zb_ref|zb_unfused|toy|unet|tsrgan|copy|climsim_host|zb_host] [--no-cpu]
 
 One "step" is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  Prints ONE JSON line: columns/s for the whole job, the roofline figure of the dominant
@@ -364,6 +364,75 @@ def cpu_baseline_conv(case, which):
                        f"took {t_layer:.2f} s -> {case['voxels'] * share / t_layer:.3g} voxels/s extrapolated")
 
 
+def run_climsim_host(L, args):
+    """PCIe-inclusive: the boundary verdict's whole-array call, mlp_forward(host column-major A, host column-major B)
+    (driver/fortis_shim.py:126-133), on pageable host arrays as a Fortran host owns them.  Never the headline value."""
+    from fortis_amd import configs, step as ST
+    case = configs.climsim()
+    plan = configs.climsim_plan(case, boundary=True)
+    A = np.ascontiguousarray(case["A"].reshape(-1, order="F"))
+    rows = case["rows"]
+    nout = rows * case["widths"][-1]
+    ST.bind(plan, A.size, nout, verdict="boundary")
+    out = np.empty(nout, np.float32)
+    for _ in range(max(2, args.warmup)):
+        ST.mlp_forward(A, out)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ST.mlp_forward(A, out)
+    dt = time.perf_counter() - t0
+    nk = plan.num_kernels
+    ST.reset()
+    plan.close()
+    nbytes = A.nbytes + out.nbytes
+    ms = dt / args.steps * 1e3
+    return dict(rows=rows, dt=dt, dtype="f32",
+                config={"workload": "climsim_host_arrays_mlp_forward_24576x556_to_24576x368", "columns": rows, "launches_per_step": nk,
+                        "host_bytes_per_call": nbytes, "note": "host arrays pageable; in row bands through page-locked staging, copies under the computation"},
+                roofline=dict(bound="pcie", kernel="whole-array entry (host -> device -> host)", achieved=round(nbytes / (ms * 1e-3) / 1e9, 2), peak=None,
+                              unit="GB/s over the bus, both directions summed", frac=None, avg_launch_ms=round(ms, 4), traffic=None))
+
+
+def run_zb_host_step(L, args):
+    """PCIe-inclusive: the fissioned ZB host's step through the entries, fortis_gather(4 host arrays) ->
+    mlp_forward_batched() -> 15 x fortis_scatter(k, 5 host arrays) (mom6_zb/host_fissioned.fir:732-740), reference
+    geometry and network, pageable host arrays."""
+    from fortis_amd import configs, plan as P, stencil as S, step as ST
+    g = os.path.join(ROOT, "tests", "golden")
+    gt, st, gd, sd, lp, kd = S.load_tables(f"{g}/zb_gather.json", f"{g}/zb_scatter.json", f"{g}/zb_loop.json", f"{g}/zb_kdist.json")
+    W = np.load(f"{g}/zb_nn.npz")
+    A = configs.zb_arrays(68, 78, 15)
+    rows = 71040
+    plan = P.mlp_plan([W["A0"], W["A1"]], [W["b0"], W["b1"]], ["relu", None], rows, in_norms=W["in_norms"], out_norms=W["out_norms"])
+    ST.bind(plan, rows * 27, rows * 3, verdict="batched", expanded=True, count=rows, gather=True, scatter=True)
+    ST.gather_config(gt)
+    ST.scatter_config(st)
+    n3 = 68 * 78 * 15
+    Txy_h, Txx, Tyy = np.zeros(68 * 78, np.float32), np.zeros(n3, np.float32), np.zeros(n3, np.float32)
+    ga = [a.ctypes.data for a in (A["sh_xy_h"], A["sh_xx"], A["vort_xy_h"], A["norm_h"])]
+    sa = [a.ctypes.data for a in (A["norm_h"], A["kappa_h"], Txy_h, Txx, Tyy)]
+
+    def step():
+        L.fortis_gather(*ga)
+        ST.mlp_forward_batched()
+        for k in range(1, 16):
+            L.fortis_scatter(k, *sa)
+    for _ in range(max(3, args.warmup)):
+        step()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    dt = time.perf_counter() - t0
+    ST.reset()
+    plan.close()
+    ms = dt / args.steps * 1e3
+    return dict(rows=rows, dt=dt, dtype="f32",
+                config={"workload": "zb_host_step_gather_batched_15_scatters_68x78x15", "columns": rows, "launches_per_step": 3,
+                        "note": "host arrays pageable; includes the Python call overhead of 17 entry calls per step"},
+                roofline=dict(bound="pcie", kernel="fortis_gather + mlp_forward_batched + 15 fortis_scatter", achieved=None, peak=None,
+                              unit="", frac=None, avg_launch_ms=round(ms, 5), traffic=None))
+
+
 def run_toy(L, args):
     from fortis_amd import configs
     case = configs.toy_mlp()
@@ -501,7 +570,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20, help="untimed steps first; the clocks need about ten steps of this size to settle")
-    ap.add_argument("--workload", default=None, help="default: climsim, followed by short runs of the other configurations (others)", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan"])
+    ap.add_argument("--workload", default=None, help="default: climsim, followed by short runs of the other configurations (others)", choices=["climsim", "zb", "zb_ref", "zb_unfused", "toy", "copy", "unet", "tsrgan", "climsim_host", "zb_host"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the short runs of the other configurations that follow the default workload")
     ap.add_argument("--f64", action="store_true", help="zb_unfused only: double-precision host arrays (the general stencil kernels)")
@@ -544,6 +613,10 @@ def run_workload(L, args, workload):
         return run_conv(L, args, workload)
     if workload == "zb_unfused":
         return run_zb_unfused(L, args)
+    if workload == "climsim_host":
+        return run_climsim_host(L, args)
+    if workload == "zb_host":
+        return run_zb_host_step(L, args)
     return run_zb(L, args, reference_net=(workload == "zb_ref"))
 
 
@@ -556,7 +629,9 @@ OTHERS = [("toy 1024x(64-256-256-32)", "toy", None, 200, 50),
           ("zb 1028x1028x15 fused, reference net 27-20-3", "zb_ref", "1028x1028x15", 40, 20),
           ("zb 1028x1028x15 unfused (gather kernel is the roofline)", "zb_unfused", "1028x1028x15", 20, 10),
           ("unet 1x4x256x256", "unet", None, 100, 30),
-          ("tsrgan 33^3 -> 66^3", "tsrgan", None, 40, 15)]
+          ("tsrgan 33^3 -> 66^3", "tsrgan", None, 40, 15),
+          ("climsim whole-array call on host arrays (PCIe-inclusive)", "climsim_host", None, 20, 3),
+          ("zb host step through the entries (PCIe-inclusive)", "zb_host", None, 100, 10)]
 
 
 def run_others(L, args):

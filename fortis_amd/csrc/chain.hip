@@ -1243,16 +1243,19 @@ static void launch_wave(ChainParams& P, hipStream_t s)
     }
 }
 
-void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows, hipStream_t s)
+// form_rows: the row count that picks the kernel form (0: rows).  A caller that runs a batch in row bands passes the
+// whole batch's, so that every band is computed by the kernel -- and in the summation order -- of the whole batch.
+void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows, hipStream_t s, long form_rows)
 {
     if (!chain_ok(d, rows)) return;
     ChainParams P;
     fill_params(&P, d, X, Y, rows, nullptr);
+    if (form_rows <= 0) form_rows = rows;
     // many rows of a narrow input: the wave-independent kernel
-    if (rows >= 64L * num_cus()) { launch_wave<false>(P, s); return; }
+    if (form_rows >= 64L * num_cus()) { launch_wave<false>(P, s); return; }
     const bool wlds = chain_wlds(d);
     // few rows: 16-row tiles spread the work over more CUs (the four waves then split the n-tiles)
-    if (rows < 64L * num_cus()) {
+    if (form_rows < 64L * num_cus()) {
         if (wlds) launch_variant<16, true>(P, s);
         else launch_variant<16, false>(P, s);
     } else {

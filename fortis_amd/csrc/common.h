@@ -59,7 +59,7 @@ struct ChainDesc {
 // descriptor's shape fields; act/alpha/in_div/out_mul/mask_tail are left to the caller.
 int fortis_chain_build(ChainDesc* d, int nlayers, const float* const* W, const float* const* b, const int* K,
                        const int* N, float** blob_out);
-void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows, hipStream_t s);
+void fortis_launch_chain(const ChainDesc& d, const float* X, float* Y, long rows, hipStream_t s, long form_rows = 0);
 // rcp[c] = the refined reciprocal of div[c] exactly as the IEEE division sequence forms it (v_rcp_f32 and one Newton
 // step), computed on the device so that a kernel dividing many numerators by div[c] can take it from memory.
 void fortis_chain_fill_rcp(const float* div, float* rcp, int n, hipStream_t s);

@@ -3,6 +3,9 @@
 // buffer ownership, upload/download choreography, pack/unpack staging, graph capture on the
 // second call and replay afterwards, with an eager fallback.
 #include <atomic>
+#include <condition_variable>
+#include <mutex>
+#include <functional>
 #include <thread>
 #include <vector>
 #include "common.h"
@@ -57,6 +60,7 @@ struct fortis_plan {
     bool upload_failed = false; // a weight / vector upload found no device memory
     int in_t = -1, out_t = -1;
     long rows0 = 0;             // rows at finalize (row-wise plans), for run-time extents
+    long band_rows = 0;         // rows when every kernel works row by row, boundary transposes included (row bands can then run on their own)
     int exec_skip = 0;          // ops folded into a neighbour at finalize
     bool prof = false;          // per-kernel event timing (fortis_plan_profile)
     std::vector<hipEvent_t> ev; // events of the recorded passes: (nexec + 1) per pass
@@ -540,6 +544,16 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
         if (rows < 0) rows = e.rows; else if (rows != e.rows) rowwise = false;
     }
     p->rows0 = rowwise ? rows : 0;
+    {
+        bool bandable = true;
+        long br = -1;
+        for (const Exec& e : p->exec) {
+            if (e.kind > EX_POST) { bandable = false; break; }
+            if (br < 0) br = e.rows; else if (br != e.rows) bandable = false;
+        }
+        for (int v : p->view_of) if (v >= 0) bandable = false;
+        p->band_rows = bandable ? br : 0;
+    }
     if (p->upload_failed) return bad("finalize: out of device memory for the weights");
     if (assign_buffers(p) != 0) return bad("finalize: out of device memory for the activations");
     p->finalized = true;
@@ -608,6 +622,33 @@ void fortis_plan_run(fortis_plan* p)
         }
         if (rc != 0) fprintf(stderr, "fortis_plan_run: an op was rejected by its kernel launcher\n");
         mark();
+    }
+}
+
+// Rows [i0, i0 + n) of a plan whose kernels all work row by row (band_rows > 0), on the plan's own tensors: every
+// tensor is addressed i0 rows in.  A boundary transpose reads or writes its host-side tensor as a compact
+// column-major block of the band's n rows placed i0 rows (of the tensor's width) into it, so a band's input and
+// output are contiguous ranges of the input and output tensors.
+static void plan_run_rows(fortis_plan* p, long i0, long n, hipStream_t s)
+{
+    for (const Exec& e : p->exec) {
+        char* src = (char*)p->tptr[e.src];
+        char* dst = (char*)p->tptr[e.dst];
+        int rc = 0;
+        switch (e.kind) {
+            case EX_CHAIN: {
+                const long K0 = e.chain.L[0].K, NO = e.chain.L[e.chain.nlayers - 1].N;
+                fortis_launch_chain(e.chain, (const float*)src + i0 * K0, (float*)dst + i0 * NO, n, s, e.rows);
+                break;
+            }
+            case EX_GEMM: rc = fortis_launch_gemm((const float*)src + i0 * e.K, e.W, e.bias, (float*)dst + i0 * e.N, n, e.N, e.K, e.act, e.alpha, e.out_scale, e.mask_tail, s); break;
+            case EX_SCALE: fortis_launch_scale((const float*)src + i0 * e.N, (float*)dst + i0 * e.N, e.vec, n, e.N, e.flag, s); break;
+            case EX_MASK: fortis_launch_mask_relu((const float*)src + i0 * e.N, (float*)dst + i0 * e.N, n, e.N, e.mask_tail, s); break;
+            case EX_PRE: fortis_launch_boundary_pre(src + i0 * e.N * e.flag, (float*)dst + i0 * e.N, n, e.N, e.p0, e.p1, e.p2, e.flag, s); break;
+            case EX_POST: fortis_launch_boundary_post((const float*)src + i0 * e.N, dst + i0 * e.N * e.flag, n, e.N, e.p0, e.flag, s); break;
+            default: rc = -1; break;
+        }
+        if (rc != 0) fprintf(stderr, "fortis_plan_run: an op was rejected by its kernel launcher\n");
     }
 }
 
@@ -954,6 +995,129 @@ void mlp_forward_batched(void* in, void* out)
         memcpy((char*)out + (size_t)(h.minc - 1 + r * st) * NOUT, (const char*)g_step.Y + (size_t)r * NOUT, NOUT);
 }
 
+// ---- whole-array call on large host arrays, in row bands -------------------------------------------------------
+// Rows are independent, so the call is cut into a few bands: while band b computes, band b + 1 crosses the bus and
+// band b - 1 comes back (two copy streams beside the persistent one, events between them; all default priority).
+// Host arrays are pageable and cannot be page-locked in place here, so every band goes through the page-locked
+// staging buffers; a column-major boundary array is packed band by band into compact column-major blocks (one run
+// per feature), which is the layout plan_run_rows gives a boundary transpose.  FORTIS_BANDS=n sets the count
+// (1: the whole array at once, as without this path).
+static hipStream_t g_up = nullptr, g_down = nullptr;
+// Host copies are what bounds such a call (the bus and the GPU are faster than four threads copy), so the runs of a
+// band are dealt to a pool of threads that lives as long as the process (FORTIS_COPY_THREADS, default 12; starting
+// threads for every band cost about 0.1 ms each time).
+struct CopyPool {
+    std::mutex m;
+    std::condition_variable go, done;
+    const std::function<void(long)>* fn = nullptr;
+    long nruns = 0, gen = 0;
+    std::atomic<long> next{0};
+    int busy = 0, nthreads = 0;
+    void worker()
+    {
+        long seen = 0;
+        for (;;) {
+            const std::function<void(long)>* f;
+            long n;
+            {
+                std::unique_lock<std::mutex> l(m);
+                go.wait(l, [&] { return gen != seen; });
+                seen = gen; f = fn; n = nruns;
+            }
+            for (long k = next.fetch_add(1); k < n; k = next.fetch_add(1)) (*f)(k);
+            {
+                std::lock_guard<std::mutex> l(m);
+                if (--busy == 0) done.notify_one();
+            }
+        }
+    }
+    void run(long n, const std::function<void(long)>& f)
+    {
+        if (!nthreads) {
+            const char* e = getenv("FORTIS_COPY_THREADS");
+            nthreads = e ? atoi(e) : 12;
+            if (nthreads < 1) nthreads = 1;
+            if (nthreads > 32) nthreads = 32;
+            for (int t = 1; t < nthreads; t++) std::thread([this] { worker(); }).detach();
+        }
+        {
+            std::lock_guard<std::mutex> l(m);
+            fn = &f; nruns = n; next = 0; busy = nthreads - 1; gen++;
+        }
+        go.notify_all();
+        for (long k = next.fetch_add(1); k < n; k = next.fetch_add(1)) f(k);
+        std::unique_lock<std::mutex> l(m);
+        done.wait(l, [&] { return busy == 0; });
+    }
+};
+static void parallel_runs(long nruns, const std::function<void(long)>& run)
+{
+    static CopyPool* pool = new CopyPool();      // never destroyed: its threads wait for work until the process ends
+    pool->run(nruns, run);
+}
+static int forward_banded(void* in, void* out)
+{
+    fortis_plan* p = g_step.plan;
+    const fortis_host_t& h = g_step.h;
+    const long rows = p->band_rows;
+    const char* env = getenv("FORTIS_BANDS");
+    const int want = env ? atoi(env) : 0;
+    long nb = want > 0 ? want : rows / 6144;            // whole bands of about 8192 rows, half bands at both ends
+    if (nb > 8) nb = 8;
+    if (nb < 2 || rows <= 0 || h.n_in % rows || h.n_out % rows || p->in_t == p->out_t) return -1;
+    const long win = h.n_in / rows, wout = h.n_out / rows;           // elements per row
+    const size_t ein = (size_t)h.in_esz, eout = (size_t)h.out_esz;
+    const bool in_cm = p->exec.front().kind == EX_PRE, out_cm = p->exec.back().kind == EX_POST;
+    hipStream_t s = fortis_stream_get();
+    if (!g_up) { HIP_OK(hipStreamCreateWithFlags(&g_up, hipStreamNonBlocking)); HIP_OK(hipStreamCreateWithFlags(&g_down, hipStreamNonBlocking)); }
+    static std::vector<hipEvent_t> ev;
+    while (ev.size() < (size_t)3 * 8) { hipEvent_t e; HIP_OK(hipEventCreateWithFlags(&e, hipEventDisableTiming)); ev.push_back(e); }
+    if (!g_step.X) setup_xy();
+    HIP_OK(hipStreamSynchronize(s));                    // the staging buffers and the tensors are free again
+    HIP_OK(hipStreamSynchronize(g_up));
+    HIP_OK(hipStreamSynchronize(g_down));
+    // band edges: the first and the last band are half bands (the first computation starts, and the last copy back
+    // ends, half a band sooner), every edge a multiple of 128 rows
+    long edge[10];
+    {
+        const long q = (rows / (2 * (nb - 1)) + 127) / 128 * 128;
+        edge[0] = 0;
+        for (long b = 1; b <= nb; b++) { const long e = q * (2 * b - 1); edge[b] = b == nb || e > rows ? rows : e; }
+    }
+    g_forward_gen++;
+    for (long b = 0; b < nb; b++) {
+        const long i0 = edge[b], n = edge[b + 1] - edge[b];
+        if (n <= 0) continue;
+        char* stage = (char*)g_step.X + (size_t)i0 * win * ein;
+        if (in_cm) parallel_runs(win, [&](long k) { memcpy(stage + (size_t)k * n * ein, (const char*)in + ((size_t)k * rows + i0) * ein, (size_t)n * ein); });
+        else {
+            const size_t bytes = (size_t)n * win * ein, piece = (bytes / 32 + 4095) & ~(size_t)4095;
+            parallel_runs(32, [&](long k) { const size_t o = (size_t)k * piece; if (o < bytes) memcpy(stage + o, (const char*)in + (size_t)i0 * win * ein + o, o + piece < bytes ? piece : bytes - o); });
+        }
+        HIP_OK(hipMemcpyAsync((char*)g_step.din + (size_t)i0 * win * ein, stage, (size_t)n * win * ein, hipMemcpyHostToDevice, g_up));
+        HIP_OK(hipEventRecord(ev[3 * b], g_up));
+        HIP_OK(hipStreamWaitEvent(s, ev[3 * b], 0));
+        plan_run_rows(p, i0, n, s);
+        HIP_OK(hipEventRecord(ev[3 * b + 1], s));
+        HIP_OK(hipStreamWaitEvent(g_down, ev[3 * b + 1], 0));
+        HIP_OK(hipMemcpyAsync((char*)g_step.Y + (size_t)i0 * wout * eout, (char*)g_step.dout + (size_t)i0 * wout * eout, (size_t)n * wout * eout, hipMemcpyDeviceToHost, g_down));
+        HIP_OK(hipEventRecord(ev[3 * b + 2], g_down));
+    }
+    for (long b = 0; b < nb; b++) {
+        const long i0 = edge[b], n = edge[b + 1] - edge[b];
+        if (n <= 0) continue;
+        const char* stage = (const char*)g_step.Y + (size_t)i0 * wout * eout;
+        HIP_OK(hipEventSynchronize(ev[3 * b + 2]));
+        if (out_cm) parallel_runs(wout, [&](long k) { memcpy((char*)out + ((size_t)k * rows + i0) * eout, stage + (size_t)k * n * eout, (size_t)n * eout); });
+        else {
+            const size_t bytes = (size_t)n * wout * eout, piece = (bytes / 32 + 4095) & ~(size_t)4095;
+            parallel_runs(32, [&](long k) { const size_t o = (size_t)k * piece; if (o < bytes) memcpy((char*)out + (size_t)i0 * wout * eout + o, stage + o, o + piece < bytes ? piece : bytes - o); });
+        }
+    }
+    HIP_OK(hipStreamSynchronize(s));
+    return 0;
+}
+
 void mlp_forward(void* in, void* out)
 {
     if (!bound("mlp_forward")) return;
@@ -993,6 +1157,9 @@ void mlp_forward(void* in, void* out)
         memcpy(out, g_step.Y, nout);
         return;
     }
+    // large arrays of a step whose kernels all work row by row: in row bands, copies under the computation (after
+    // such a call the resident buffers hold a boundary array band by band, not as the host's array)
+    if (staged_copies(nin) && staged_copies(nout) && p->band_rows > 0 && forward_banded(in, out) == 0) return;
     mlp_upload(in);
     mlp_forward_dev();
     mlp_download(out);

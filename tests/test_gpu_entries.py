@@ -233,6 +233,45 @@ def test_boundary_verdict_f64_host_arrays(L, gpu):
     assert maxrel(B, ref) < TOL
 
 
+@pytest.mark.parametrize("dtype,hidden", [(np.float64, 320), (np.float32, 96)])
+def test_boundary_verdict_large_arrays_in_row_bands(L, gpu, monkeypatch, dtype, hidden):
+    """A whole-array call on large host arrays runs in row bands (copies of one band under the computation of
+    another); the host's column-major boundary arrays are packed band by band.  The result must be the one of the
+    whole array at once (FORTIS_BANDS=1), bit for bit, for a ragged last band, with the wide layers on the GEMM
+    kernel (hidden 320) and the narrow ones in the chain kernel, and a sample of rows must agree with the oracle."""
+    rng = np.random.default_rng(14)
+    NI, NIN, NOUT = 30011, 120, 72
+    Ws = [(rng.standard_normal((hidden, NIN)) / 11).astype(np.float32), (rng.standard_normal((NOUT, hidden)) / np.sqrt(hidden)).astype(np.float32)]
+    bs = [rng.standard_normal(hidden).astype(np.float32), rng.standard_normal(NOUT).astype(np.float32)]
+    A = np.asfortranarray(rng.standard_normal((NI, NIN)).astype(dtype))
+    mean, vmax, vmin, scale = (v.astype(dtype) for v in (rng.standard_normal(NIN), rng.uniform(2, 3, NIN), rng.uniform(0, 1, NIN), rng.uniform(0.5, 2, NOUT)))
+    esz = np.dtype(dtype).itemsize
+    outs = []
+    for bands in ("3", "1"):
+        monkeypatch.setenv("FORTIS_BANDS", bands)
+        ST.reset()
+        p = P.Plan()
+        t0, t1, t2, t3, t4 = p.tensor(NI * NIN, esz), p.tensor(NI * NIN), p.tensor(NI * hidden), p.tensor(NI * NOUT), p.tensor(NI * NOUT, esz)
+        p.boundary_pre(t0, t1, NI, NIN, mean, vmax, vmin, dtype)
+        p.linear(t1, t2, Ws[0], bs[0], NI, "leaky", 0.15)
+        p.linear(t2, t3, Ws[1], bs[1], NI, None)
+        p.boundary_post(t3, t4, NI, NOUT, scale, dtype)
+        p.finalize(t0, t4)
+        ST.bind(p, NI * NIN, NI * NOUT, verdict="boundary", in_dtype=dtype, out_dtype=dtype)
+        B = np.zeros((NI, NOUT), dtype, order="F")
+        ST.mlp_forward(A, B)
+        B2 = np.zeros((NI, NOUT), dtype, order="F")
+        ST.mlp_forward(A, B2)                                       # a second call reuses staging and events
+        assert bits_equal(B, B2)
+        outs.append(B)
+    assert bits_equal(outs[0], outs[1])
+    idx = np.sort(rng.choice(NI, 400, replace=False))
+    X = O.boundary_pre(np.asfortranarray(A[idx]), mean, vmax, vmin)
+    ref = O.boundary_post(O.mlp_f64(Ws, bs, ["leaky", "none"], X, alphas=[0.15, 0]), scale, dtype)
+    assert maxrel(outs[0][idx], ref) < TOL
+    ST.reset()
+
+
 def test_run_time_extents(L, gpu):
     """fortis_begin(count) (driver/fortis_stub.c:12-31): the step bound for 200 rows serves 120, then 333 (more
     than it was bound for: the reference's stub specialises for any count), then 200 again."""
