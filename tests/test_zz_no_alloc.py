@@ -72,9 +72,10 @@ def test_noalloc_entry_asks_the_device_for_no_memory(L, gpu):
         for d in (dx, dw, dy):
             d.free()
     # the counter is live: every raw allocation of the library (pool, weights, the convolution path's own buffers)
-    # goes through the one counted function; a pool request of a size never seen before must move it
+    # goes through the one counted function; a pool request larger than any buffer the pool can hold released (6 GiB)
+    # must move it
     before = L.fortis_dev_alloc_calls()
-    p = L.fortis_alloc(123456789)
+    p = L.fortis_alloc(6 << 30)
     assert p and L.fortis_dev_alloc_calls() == before + 1
     L.fortis_free(p)
 
