@@ -79,6 +79,8 @@ __global__ __launch_bounds__(ST_THREADS) void gather_kernel(GatherArgs args, flo
     }
 }
 
+// A workgroup takes SC_TILES consecutive tiles of 256 cells (the table's copy into LDS is paid once for all of them).
+#define SC_TILES 4
 __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, const float* __restrict__ Y, int kk)
 {
     __shared__ ScatterArgs d;
@@ -86,35 +88,39 @@ __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, c
     params_to_lds(&d, ST_THREADS);
     const int n = st_u(d.nrefs);
     const int tid = threadIdx.x;
-    const unsigned col0 = blockIdx.x * ST_THREADS, col = col0 + tid;
-    const unsigned lim = (d.count - col0 < ST_THREADS ? d.count - col0 : ST_THREADS) * n;
     kk += blockIdx.y;                                         // gridDim.y > 1: one enclosing-loop iteration per y
-    const float* in = Y + ((size_t)blockIdx.y * d.count + col0) * n;
-    if (((uintptr_t)in & 15) == 0) {
-        const unsigned lim4 = lim / 4;
-        for (unsigned idx = tid; idx < lim4; idx += ST_THREADS) ((st_v4f*)lds)[idx] = __builtin_nontemporal_load((const st_v4f*)in + idx);   // Y is read once
-        for (unsigned idx = lim4 * 4 + tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
-    } else {
-        for (unsigned idx = tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
-    }
-    __syncthreads();
-    if (col >= d.count) return;
-    int i, j;
-    st_cell(d, col, i, j);
-    StCell cell;
-    st_prepare(d, i, j, kk, cell);
-    // outputs are few (one per model output); handled eight at a time
-    for (int q0 = 0; q0 < n; q0 += 8) {
-        float tv[8];
+    for (int tile = 0; tile < SC_TILES; tile++) {
+        const unsigned col0 = (blockIdx.x * SC_TILES + tile) * ST_THREADS, col = col0 + tid;
+        if (col0 >= d.count) break;
+        const unsigned lim = (d.count - col0 < ST_THREADS ? d.count - col0 : ST_THREADS) * n;
+        const float* in = Y + ((size_t)blockIdx.y * d.count + col0) * n;
+        if (tile) __syncthreads();                            // the tile before has been read out of LDS
+        if (((uintptr_t)in & 15) == 0) {
+            const unsigned lim4 = lim / 4;
+            for (unsigned idx = tid; idx < lim4; idx += ST_THREADS) ((st_v4f*)lds)[idx] = __builtin_nontemporal_load((const st_v4f*)in + idx);   // Y is read once
+            for (unsigned idx = lim4 * 4 + tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
+        } else {
+            for (unsigned idx = tid; idx < lim; idx += ST_THREADS) lds[idx] = in[idx];
+        }
+        __syncthreads();
+        if (col >= d.count) continue;
+        int i, j;
+        st_cell(d, col, i, j);
+        StCell cell;
+        st_prepare(d, i, j, kk, cell);
+        // outputs are few (one per model output); handled eight at a time
+        for (int q0 = 0; q0 < n; q0 += 8) {
+            float tv[8];
 #pragma unroll
-        for (int t = 0; t < 8; t++) tv[t] = q0 + t < n ? lds[tid * n + q0 + t] : 0.f;
-        st_chain_apply(d, cell, tv);
+            for (int t = 0; t < 8; t++) tv[t] = q0 + t < n ? lds[tid * n + q0 + t] : 0.f;
+            st_chain_apply(d, cell, tv);
 #pragma unroll
-        for (int t = 0; t < 8; t++)
-            if (q0 + t < n) {
-                const StSlotT<float*> sl = d.refs[q0 + t];
-                st_g(sl.p)[st_off(sl, i, j, kk)] = tv[t];
-            }
+            for (int t = 0; t < 8; t++)
+                if (q0 + t < n) {
+                    const StSlotT<float*> sl = d.refs[q0 + t];
+                    __builtin_nontemporal_store(tv[t], st_g(sl.p) + st_off(sl, i, j, kk));     // written once, read by the host's next phase
+                }
+        }
     }
 }
 
@@ -380,7 +386,7 @@ static void launch_scatter(const StencilDev& low, float* const* dA, const float*
 {
     ScatterArgs a;
     st_make_args<float*>(low, low.cells, dA, &a);
-    hipLaunchKernelGGL(scatter_kernel, dim3((unsigned)cdiv(low.count, ST_THREADS), (unsigned)layers), dim3(ST_THREADS),
+    hipLaunchKernelGGL(scatter_kernel, dim3((unsigned)cdiv(low.count, ST_THREADS * SC_TILES), (unsigned)layers), dim3(ST_THREADS),
                        (size_t)ST_THREADS * low.nrefs * sizeof(float), s, a, dY, kk);
     HIP_OK(hipGetLastError());
 }
