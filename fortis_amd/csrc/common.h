@@ -122,7 +122,14 @@ struct ConvEpi {
     float alpha;
     const float* res;    // residual tensor added after the activation (same shape as output), or null
     float* pool;         // conv2d only: also receives the 2 x 2 stride-2 max pool of the output (H, W even), or null
+    // conv2d only: a following 1 x 1 convolution to head_n <= 4 channels (weights [head_n][F], bias or null) written to
+    // head_y INSTEAD of this conv's own output, which then is not stored (fortis_conv_mfma_head_ok says when)
+    const float* head_w;
+    const float* head_b;
+    float* head_y;
+    int head_n;
 };
+bool fortis_conv_mfma_head_ok(long C, long H, long Wd, long F, int KD, int KS, int nh);
 int fortis_launch_conv2d(const float* x, const float* w, float* y, long C, long H, long Wd, long F, long KH,
                          long KW, long Ho, long Wo, long sh, long sw, long ph, long pw, const ConvEpi& e,
                          long coff, long ctot, hipStream_t s);

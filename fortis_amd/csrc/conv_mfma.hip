@@ -70,7 +70,9 @@ __device__ __forceinline__ void cm_lds_barrier()
 // (part[slot][tile][register][thread], slot = the workgroup's rank among those that share the tile).
 // conv_sk_reduce_kernel adds a tile's slots in order and applies the epilogue.  Equal runs are what a split into
 // whole slices cannot give: 297 tiles in 3 slices are 891 workgroups, four on some CUs and three on others.
-template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1, bool POOL = false, bool SK = false>
+// POOL: 0, 1 (the kernel also writes the 2 x 2 max pool of its tiles) or 2 (instead of its own output the kernel writes a
+// following 1 x 1 convolution to at most four channels, computed from the finished tile in LDS: a thin head costs no launch).
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1, int POOL = 0, bool SK = false>
 __global__ __launch_bounds__(CM_THREADS) __attribute__((amdgpu_waves_per_eu(SK ? 2 : KD == 3 && MT == 128 && FT == 64 && NX <= 8 ? 4 : 1)))
 void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                                                                float* __restrict__ y, ConvMShape s, ConvEpi e)
@@ -471,8 +473,8 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 #pragma unroll
         for (int q = 0; q < N; q++) {
             if (!ok[q]) continue;
-            y[off[q]] = v[q];
-            if constexpr (POOL) {
+            if constexpr (POOL != 2) y[off[q]] = v[q];
+            if constexpr (POOL != 0) {
                 // the finished tile also goes to LDS as [channel][row][32 columns] for the 2 x 2 max pool below
                 // (behind the channel groups' sums, which other waves may still be reading)
                 const int r = r0 + q, f = fb + 8 * (r >> 2) + (r & 3);
@@ -483,7 +485,22 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     // 2 x 2 stride-2 max pool of the finished tile (H and W even, tiles start on even rows and columns: a 2 x 2
     // block lies inside the image or outside it as a whole); staging has ended, LDS is free
     auto pool_tile = [&]() __attribute__((always_inline)) {
-        if constexpr (POOL) {
+        if constexpr (POOL == 2) {
+            // head: out[o][pos] = head_b[o] + sum over this conv's channels of head_w[o][c] * tile[c][pos], channels in order
+            cm_lds_barrier();
+            const float* pt = (const float*)smem4 + (KG > 1 ? 4 * 16 * 64 : 0);
+            const int nh = e.head_n;
+            for (int idx = tid; idx < nh * MT; idx += CM_THREADS) {
+                const int pos = idx % MT, o = idx / MT, row = pos >> 5, col = pos & 31;
+                const int yy = y0 + row, xx = x0 + col;
+                if (yy >= s.H || xx >= s.W) continue;
+                float a = e.head_b ? e.head_b[o] : 0.f;
+                const float* hw = e.head_w + o * s.F;
+                for (int c = 0; c < s.F; c++) a = fmaf(hw[c], pt[(c * TH + row) * 32 + col], a);
+                e.head_y[((long)o * s.H + yy) * s.W + xx] = a;
+            }
+        }
+        if constexpr (POOL == 1) {
             cm_lds_barrier();
             const float* pt = (const float*)smem4 + (KG > 1 ? 4 * 16 * 64 : 0);
             const int Ho = s.H >> 1, Wo = s.W >> 1;
@@ -497,7 +514,8 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
             }
         }
     };
-    static_assert(!POOL || (TILE2D && (MT / 32) % 2 == 0), "the in-kernel pool needs the 32-column tiling and an even tile height");
+    static_assert(POOL != 1 || (TILE2D && (MT / 32) % 2 == 0), "the in-kernel pool needs the 32-column tiling and an even tile height");
+    static_assert(POOL != 2 || TILE2D, "the in-kernel head needs the 32-column tiling");
     if constexpr (SK) {
         // the accumulators as they are: slot = this workgroup's rank among those whose runs share the tile
         const int tl = bx - s.sk_tile0;
@@ -784,6 +802,13 @@ int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, i
     return 1;
 }
 
+// Whether the launcher writes a following thin 1 x 1 convolution (nh output channels) from this conv's finished tiles:
+// the 3 x 3 form with 64 x 32 tiles whose workgroup holds all of the conv's channels.
+bool fortis_conv_mfma_head_ok(long C, long H, long Wd, long F, int KD, int KS, int nh)
+{
+    return KD == 1 && KS == 3 && F <= 32 && nh >= 1 && nh <= 4 && fortis_conv_mfma_kgroups(C, 1, H, Wd, F, 1, 3) == 2;
+}
+
 // Packs conv weights W[F][C][T] (T taps, row-major) into the kernel's order
 //   [F/FT][ceil(C/CC)][channel pair CC/2][tap T][half 2][FT channels], zero padded; CC = cm_cc(T) * kg
 //   channels per chunk; FT = 32 when the GEMM has at most 32 output channels or kg > 1, else 64 (the launcher
@@ -867,7 +892,7 @@ const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, h
     return buf;
 }
 
-template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1, bool POOL = false>
+template <int KD, int KS, int MT, int FT, int NX, bool TILE2D, int KG = 1, int POOL = 0>
 static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, const ConvEpi& e, hipStream_t st)
 {
     constexpr int T = KD * KS * KS;
@@ -888,7 +913,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     size_t shmem = (size_t)2 * ((four_per_cu ? WCH : WCHPAD) + xchp) * sizeof(float);
     const size_t shmem_sk = (size_t)2 * ((NX <= 8 ? WCHPAD : WCH) + xchp) * sizeof(float);      // the streamed form's
     if (KG > 1 && shmem < 4 * 16 * 64 * sizeof(float)) shmem = 4 * 16 * 64 * sizeof(float);  // (4 / KG tiles) x KG groups x 16 registers x 64 lanes   // the groups' sums meet in LDS
-    if (POOL && shmem < (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float)) shmem = (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float);   // the finished tile, for its 2 x 2 max pool
+    if (POOL != 0 && shmem < (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float)) shmem = (size_t)((KG > 1 ? 4 * 16 * 64 : 0) + FT * MT) * sizeof(float);   // the finished tile, for its 2 x 2 max pool
     if (shmem > 160 * 1024 || shmem_sk > 160 * 1024) return -1;
     static size_t attr = 0;
     if (shmem > attr) {
@@ -969,7 +994,7 @@ static int launch_nx(const float* x, const float* wp, float* y, ConvMShape s, co
     } else if (s.ksplit > 1) {
         launch_split_reduce(s.part, y, s.osize, ospatial, s.ksplit, e, st);
         HIP_OK(hipGetLastError());
-    } else if (pooled && !POOL) {
+    } else if (pooled && POOL != 1) {
         fortis_launch_maxpool2d(y, e.pool, s.F, s.H, s.W, 2, st);
     }
     return 0;
@@ -1038,6 +1063,7 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
     s.ksplit = 1;
     s.ups = kind == 2 ? 1 : 0;
     if (kind == 2 && (KD != 3 || ((D | H | Wd) & 1))) return -1;     // the fused upsample is a form of the volume kernel
+    if (e.head_y && !fortis_conv_mfma_head_ok(C, H, Wd, F, KD, KS, e.head_n)) return -1;
     if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 2) {
         if (KS == 1) {
             s.P = s.W;
@@ -1050,7 +1076,8 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
         s.plane = s.H * s.P;
         s.nchunks = (int)cdiv(s.C, cm_cc(9) * 2);
         constexpr int NX2 = (cm_cc(9) * 2 * (64 / 32 + 2) * CM_TP + CM_THREADS - 1) / CM_THREADS;
-        if (e.pool && !s.mode && !(s.H & 1) && !(s.W & 1)) return launch_nx<1, 3, 64, 32, NX2, true, 2, true>(x, wp, y, s, e, st);
+        if (e.head_y) return e.pool || s.mode || s.F > 32 || e.head_n > 4 ? -1 : launch_nx<1, 3, 64, 32, NX2, true, 2, 2>(x, wp, y, s, e, st);
+        if (e.pool && !s.mode && !(s.H & 1) && !(s.W & 1)) return launch_nx<1, 3, 64, 32, NX2, true, 2, 1>(x, wp, y, s, e, st);
         return launch_nx<1, 3, 64, 32, NX2, true, 2>(x, wp, y, s, e, st);
     }
     if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 4) {

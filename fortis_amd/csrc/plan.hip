@@ -45,6 +45,9 @@ struct Exec {
     ConvEpi epi = { nullptr, nullptr, 0, 0.f, nullptr };
     const float* Wmfma = nullptr;   // weights packed for the MFMA implicit-GEMM kernel, when the shape qualifies
     int pool_dst = -1;              // conv2d: tensor that receives the 2 x 2 max pool folded into this conv
+    int head_dst = -1;              // conv2d: tensor that receives the thin 1 x 1 convolution folded into this conv (which then stores nothing itself)
+    const float *head_w = nullptr, *head_b = nullptr;
+    int head_n = 0;
 };
 
 struct fortis_plan {
@@ -365,7 +368,8 @@ static int assign_buffers(fortis_plan* p)
     for (int i = 0; i < ne; i++) {
         const Exec& e = p->exec[i];
         reads(e.src, i); reads(e.res, i);
-        writes(e.dst, i); writes(e.pool_dst, i);
+        if (e.head_dst < 0) writes(e.dst, i);
+        writes(e.pool_dst, i); writes(e.head_dst, i);
     }
     for (int t = 0; t < nt; t++) if (first[t] == -1) last[t] = ne;          // filled by the caller: never handed back
     first[base(p->in_t)] = -1; last[base(p->in_t)] = ne;
@@ -512,6 +516,25 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                     i += adv + 1;
                     continue;
                 }
+                // A 1 x 1 convolution to at most four channels (no BatchNorm, no activation) that is the only reader of
+                // this conv's output is computed by this conv's kernel from its finished tiles where the launcher has
+                // that form; the intermediate tensor is then never stored.
+                if (o.kind == OP_CONV2D && ex.Wmfma && i + 1 < ops.size() && o.coff == 0 && (o.ctot == 0 || o.ctot == o.F)) {
+                    const Op& h = ops[i + 1];
+                    if (h.kind == OP_CONV2D && h.src == o.dst && uses_of(p, o.dst) == 1 && h.KH == 1 && h.KW == 1 && h.stride == 1 && h.pad == 0 &&
+                        h.C == o.F && h.H == o.H && h.W == o.W && h.F <= 4 && !h.has_bn && h.act == FORTIS_ACT_NONE && h.coff == 0 &&
+                        (h.ctot == 0 || h.ctot == h.F) && h.dst != o.dst && o.dst != p->out_t && getenv("FORTIS_NO_HEAD_FOLD") == nullptr &&
+                        fortis_conv_mfma_head_ok(o.C, o.H, o.W, o.F, 1, (int)o.KH, (int)h.F)) {
+                        ex.head_dst = h.dst;
+                        ex.head_n = (int)h.F;
+                        ex.head_w = (const float*)upload(p, h.w.data(), h.w.size() * 4);
+                        ex.head_b = h.has_bias ? (const float*)upload(p, h.b.data(), h.b.size() * 4) : nullptr;
+                        p->exec.push_back(ex);
+                        p->exec_skip++;
+                        i += adv + 1;
+                        continue;
+                    }
+                }
                 break;
             }
             case OP_MAXPOOL: ex.kind = EX_MAXPOOL; break;
@@ -588,7 +611,9 @@ void fortis_plan_run(fortis_plan* p)
                 const long Ho = (o->H + 2 * o->pad - o->KH) / o->stride + 1, Wo = (o->W + 2 * o->pad - o->KW) / o->stride + 1;
                 ConvEpi epi = e.epi;
                 epi.pool = e.pool_dst >= 0 ? (float*)p->tptr[e.pool_dst] : nullptr;
+                if (e.head_dst >= 0) { epi.head_w = e.head_w; epi.head_b = e.head_b; epi.head_n = e.head_n; epi.head_y = (float*)p->tptr[e.head_dst]; }
                 rc = e.Wmfma ? fortis_launch_conv_mfma(src, e.Wmfma, dst + o->coff * Ho * Wo, o->C, 1, o->H, o->W, o->F, 1, (int)o->KH, 0, epi, s) : -1;
+                if (rc != 0 && e.head_dst >= 0) { fprintf(stderr, "fortis_plan_run: conv2d with a folded 1 x 1 head not taken by the kernel\n"); break; }
                 if (rc != 0) {
                     rc = fortis_launch_conv2d(src, e.W, dst, o->C, o->H, o->W, o->F, o->KH, o->KW, Ho, Wo, o->stride, o->stride,
                                               o->pad, o->pad, e.epi, o->coff, o->ctot, s);

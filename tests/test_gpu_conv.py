@@ -10,7 +10,7 @@ import torch
 from fortis_amd import configs, plan as P
 from oracle import oracle as O
 from refmodels import tsrgan_ref, unet_ref
-from util import TOL, DevBuf, maxrel
+from util import TOL, DevBuf, bits_equal, maxrel
 
 pytestmark = pytest.mark.gpu
 
@@ -365,3 +365,37 @@ def test_permute_channels_last_and_back_bit_exact(L, gpu, C_, S):
         got = p.forward(src, src.T.shape)
         p.close()
         assert np.array_equal(got.view(np.uint32), np.ascontiguousarray(src.T).view(np.uint32))
+
+
+@pytest.mark.parametrize("H,W,C_,F,NH", [(128, 128, 64, 32, 4), (128, 160, 48, 24, 3), (256, 256, 32, 32, 1)])
+def test_thin_1x1_head_folded_into_the_conv_before_it(L, gpu, monkeypatch, H, W, C_, F, NH):
+    """conv 3 x 3 + BN + ReLU followed by a 1 x 1 conv to a few channels (the UNet's last two layers): the plan lets the
+    3 x 3 kernel write the head from its finished tiles (one kernel, the wide tensor never stored); same result as the
+    two launches (FORTIS_NO_HEAD_FOLD) within the tolerance, and against the oracle."""
+    rng = np.random.default_rng(41)
+    x = rng.standard_normal((C_, H, W)).astype(np.float32)
+    w1 = (rng.standard_normal((F, C_, 3, 3)) / np.sqrt(9 * C_)).astype(np.float32)
+    b1 = rng.standard_normal(F).astype(np.float32)
+    bn = [rng.uniform(0.5, 1.5, F).astype(np.float32), rng.standard_normal(F).astype(np.float32) * np.float32(0.1),
+          rng.standard_normal(F).astype(np.float32) * np.float32(0.1), rng.uniform(0.5, 1.5, F).astype(np.float32)]
+    w2 = (rng.standard_normal((NH, F, 1, 1)) / np.sqrt(F)).astype(np.float32)
+    b2 = rng.standard_normal(NH).astype(np.float32)
+    outs = []
+    for fold in (True, False):
+        if not fold:
+            monkeypatch.setenv("FORTIS_NO_HEAD_FOLD", "1")
+        p = P.Plan()
+        t0, t1, t2 = p.tensor(C_ * H * W), p.tensor(F * H * W), p.tensor(NH * H * W)
+        p.conv2d(t0, t1, w1, b1, C_, H, W, 1, 1, "relu", 0.0, bn, 1e-5)
+        p.conv2d(t1, t2, w2, b2, F, H, W, 1, 0, None, 0.0)
+        p.finalize(t0, t2)
+        assert p.num_kernels == (1 if fold else 2)
+        outs.append(p.forward(x, (NH, H, W)))
+        outs.append(p.forward(x, (NH, H, W)))
+        assert bits_equal(outs[-1], outs[-2])
+        p.close()
+    mid = O.conv2d(x[None], w1, (1, 1), (1, 1))[0]
+    sc = (bn[0].astype(np.float64) / np.sqrt(bn[3].astype(np.float64) + 1e-5))
+    mid = np.maximum((mid.astype(np.float64) + b1[:, None, None] - bn[2][:, None, None]) * sc[:, None, None] + bn[1][:, None, None], 0).astype(np.float32)
+    ref = O.conv2d(mid[None], w2, (1, 1), (0, 0))[0] + b2[:, None, None]
+    assert maxrel(outs[0], ref) < TOL and maxrel(outs[2], ref) < TOL and maxrel(outs[0], outs[2]) < TOL
