@@ -142,7 +142,7 @@ int fortis_launch_conv3d(const float* x, const float* w, float* y, long C, long 
 // MFMA implicit-GEMM path (conv_mfma.hip).  kind 0: KD x KS x KS conv, pad KS/2, stride 1; kind 1: 2x2
 // stride-2 transposed conv.  wp: weights packed by fortis_conv_mfma_pack.  -1: shape not taken.
 // kg: fortis_conv_mfma_kgroups of the shape the weights will be used on (channel groups inside a workgroup).
-int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, int KS);
+int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, int KS, bool pooled = false);   // pooled: a 2 x 2 max pool of the output is asked for with the launch
 float* fortis_conv_mfma_pack(const float* W, long F, long C, int T, int transposed, long* nfloats, int kg = 1);
 const float* fortis_conv_mfma_pack_dev(const float* dW, long F, long C, int T, hipStream_t s, int kg = 1);   // device weights, packed into a library buffer; null: no memory
 int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, long D, long H, long Wd, long F, int KD,

@@ -790,14 +790,17 @@ int fortis_launch_conv_split_reduce(const float* part, float* y, long osize, lon
 // twice to four times the workgroups of the plain form, which at one or two workgroups per CU leaves the matrix
 // pipes idle while a workgroup stages); 1 otherwise.  Fg: output channels of the GEMM (4 F for the transposed conv).
 // Weights are packed for the answer, so packing and launching ask with the same arguments.
-int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, int KS)
+int fortis_conv_mfma_kgroups(long C, long D, long H, long Wd, long Fg, int KD, int KS, bool pooled)
 {
     static const int off = getenv("FORTIS_CONV_KGROUPS") != nullptr && atoi(getenv("FORTIS_CONV_KGROUPS")) == 0;
     if (off || KD != 1 || D != 1 || C < 32) return 1;
     if (KS == 3 && !(Wd >= 32 && cdiv(Wd, 32) * 32 * 4 <= 5L * Wd)) return 1;     // 3 x 3: the 32-column tiling only
     if (KS != 1 && KS != 3) return 1;
     const long pos = KS == 3 ? H * (Wd + 1) : H * Wd, tiles = cdiv(pos, 64) * cdiv(Fg, 64);
-    if (tiles < conv_cus()) return 4;
+    // (a 3 x 3 conv with a 2 x 2 max pool behind it takes the 64 x 32 form, which pools its own two-row tiles, rather
+    // than the 32 x 32 one and a pool launch)
+    static const int pool_kg2 = getenv("FORTIS_CONV_POOL_KG2") ? atoi(getenv("FORTIS_CONV_POOL_KG2")) : 1;
+    if (tiles < conv_cus()) return pooled && pool_kg2 && KS == 3 && !(H & 1) && !(Wd & 1) && tiles * 2 >= conv_cus() ? 2 : 4;
     if (tiles < 5L * conv_cus()) return 2;
     return 1;
 }
@@ -1064,7 +1067,8 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
     s.ups = kind == 2 ? 1 : 0;
     if (kind == 2 && (KD != 3 || ((D | H | Wd) & 1))) return -1;     // the fused upsample is a form of the volume kernel
     if (e.head_y && !fortis_conv_mfma_head_ok(C, H, Wd, F, KD, KS, e.head_n)) return -1;
-    if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 2) {
+    const int kgr = kind == 2 ? 1 : fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS, e.pool != nullptr && kind == 0);
+    if (kgr == 2) {
         if (KS == 1) {
             s.P = s.W;
             s.plane = s.H * s.P;
@@ -1080,7 +1084,7 @@ int fortis_launch_conv_mfma(const float* x, const float* wp, float* y, long C, l
         if (e.pool && !s.mode && !(s.H & 1) && !(s.W & 1)) return launch_nx<1, 3, 64, 32, NX2, true, 2, 1>(x, wp, y, s, e, st);
         return launch_nx<1, 3, 64, 32, NX2, true, 2>(x, wp, y, s, e, st);
     }
-    if (kind != 2 && fortis_conv_mfma_kgroups(C, D, H, Wd, s.F, KD, KS) == 4) {
+    if (kgr == 4) {
         // one 32 x 32 output tile per workgroup, the four waves share its input channels
         s.P = KS == 3 ? s.W + 1 : s.W;
         s.plane = s.H * s.P;

@@ -499,17 +499,19 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                 if (o.kind == OP_CONV2D) { ok = o.stride == 1 && o.KH == o.KW && (o.KH == 1 || o.KH == 3) && o.pad == o.KH / 2; T = (int)(o.KH * o.KW); }
                 else if (o.kind == OP_CONV3D) { ok = o.KD == 3 && o.pad == 1; T = 27; }
                 else { ok = o.KH == 2 && o.KW == 2 && o.stride == 2 && o.pad == 0 && o.opad == 0; T = 1; tr = 1; }
+                // (a 2 x 2 max pool that will be folded into this conv, see below, is part of the choice of the kernel form)
+                const bool will_pool = o.kind == OP_CONV2D && i + 1 < ops.size() && ops[i + 1].kind == OP_MAXPOOL && ops[i + 1].src == o.dst &&
+                    ops[i + 1].KH == 2 && ops[i + 1].C == o.F && ops[i + 1].H == o.H && ops[i + 1].W == o.W && o.coff == 0 &&
+                    (o.ctot == 0 || o.ctot == o.F) && !(o.H & 1) && !(o.W & 1) && ops[i + 1].dst != o.dst;
                 if (ok && wide && !direct_only) {
-                    const int kg = o.kind == OP_CONV3D ? 1 : fortis_conv_mfma_kgroups(o.C, 1, o.H, o.W, tr ? 4 * o.F : o.F, 1, tr ? 1 : (int)o.KH);
+                    const int kg = o.kind == OP_CONV3D ? 1 : fortis_conv_mfma_kgroups(o.C, 1, o.H, o.W, tr ? 4 * o.F : o.F, 1, tr ? 1 : (int)o.KH, will_pool);
                     float* wp = fortis_conv_mfma_pack(o.w.data(), o.F, o.C, T, tr, nullptr, kg);
                     if (!wp) p->upload_failed = true; else p->owned.push_back(wp);
                     ex.Wmfma = wp;
                 }
                 // A 2 x 2 max pool that directly follows and reads this conv's whole output is written by the conv's
                 // own last stage (the reduce of a channel-split launch, else a pool launch from the conv launcher).
-                if (o.kind == OP_CONV2D && ex.Wmfma && i + 1 < ops.size() && ops[i + 1].kind == OP_MAXPOOL && ops[i + 1].src == o.dst &&
-                    ops[i + 1].KH == 2 && ops[i + 1].C == o.F && ops[i + 1].H == o.H && ops[i + 1].W == o.W && o.coff == 0 &&
-                    (o.ctot == 0 || o.ctot == o.F) && !(o.H & 1) && !(o.W & 1) && ops[i + 1].dst != o.dst) {
+                if (ex.Wmfma && will_pool) {
                     ex.pool_dst = ops[i + 1].dst;
                     p->exec.push_back(ex);
                     p->exec_skip++;
