@@ -30,11 +30,9 @@ static inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 // ---- fused GEMM + bias + activation (gemm.hip) -------------------------------------------
 // C[B][N] = epi(A[B][K] . W[N][K]^T): + bias[n], activation, * out_scale[n], ReLU on the last
 // mask_tail columns.  bias/out_scale may be null.  Returns 0, or -1 on an unsupported shape.
-// cm_ld > 0: C is written column-major with leading dimension cm_ld, C[n * cm_ld + b], each value divided by
-// cm_div[n] when cm_div is given (the boundary's post transpose folded into the last layer).
 int fortis_launch_gemm(const float* A, const float* W, const float* bias, float* C, long B, long N,
                        long K, int act, float alpha, const float* out_scale, long mask_tail,
-                       hipStream_t s, const float* cm_div = nullptr, long cm_ld = 0);
+                       hipStream_t s);
 
 // ---- fused MLP chain (chain.hip) ----------------------------------------------------------
 #define FORTIS_CHAIN_MAX_LAYERS 8

@@ -26,10 +26,6 @@ struct GemmEpi {
     int act;
     float alpha;
     long mask_from;   // columns >= mask_from get ReLU (N when unused)
-    // cm_ld > 0: C is written column-major, C[n * cm_ld + m], each value divided by cm_div[n] (null: as it is): the
-    // boundary's post transpose (trt_backend/e3sm_boundary.cu:17-19, fp32 host arrays) done by the last layer's stores
-    const float* cm_div;
-    long cm_ld;
 };
 
 __device__ __forceinline__ float gemm_act(float v, int act, float alpha)
@@ -255,7 +251,7 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     // epilogue: lane holds column n = lr of 16 rows per MFMA tile.
     // Tiles with all their rows and a plain bias + activation epilogue (every hidden layer) take a path
     // with one add and the activation per element; everything else takes the guarded one.
-    const bool plain = !epi.out_scale && epi.mask_from >= N && m0 + BM <= B && !epi.cm_ld;
+    const bool plain = !epi.out_scale && epi.mask_from >= N && m0 + BM <= B;
     const int ncols = (int)(N - n0 < BN ? N - n0 : BN);                 // columns of this tile that exist
     if (plain) {
         float* cb = C + m0 * N + n0;                                    // uniform
@@ -273,31 +269,6 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
         const float bv = epi.bias ? epi.bias[n] : 0.f;
         const float sv = epi.out_scale ? epi.out_scale[n] : 1.f;
         const bool relu_tail = n >= epi.mask_from;
-        if (epi.cm_ld) {
-            // column-major: a lane's four consecutive rows of one column are 16 contiguous bytes
-            const float dv = epi.cm_div ? epi.cm_div[n] : 1.f;
-            float* col = C + n * epi.cm_ld;
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    const long m = m0 + wm + i * 32 + 8 * rq + 4 * lh;
-                    v4f o;
-#pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        float v = gemm_act(acc[i][j][4 * rq + t] + bv, epi.act, epi.alpha);
-                        if (epi.out_scale) v = v * sv;
-                        if (relu_tail) v = v > 0.f ? v : 0.f;
-                        o[t] = epi.cm_div ? __fdiv_rn(v, dv) : v;
-                    }
-                    if (m + 3 < B && (((uintptr_t)(col + m)) & 15) == 0) *(v4f*)(col + m) = o;
-                    else {
-#pragma unroll
-                        for (int t = 0; t < 4; t++) if (m + t < B) col[m + t] = o[t];
-                    }
-                }
-            continue;
-        }
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -402,13 +373,11 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(const float* __restrict
         const float bv = epi.bias ? epi.bias[n] : 0.f;
 #pragma unroll
         for (int r = 0; r < BR; r++) {
-            if (r < B) {
-                float v = gemm_act(acc[r] + bv, epi.act, epi.alpha);
-                if (epi.out_scale) v = v * epi.out_scale[n];
-                if (n >= epi.mask_from) v = v > 0.f ? v : 0.f;
-                if (epi.cm_ld) C[n * epi.cm_ld + r] = epi.cm_div ? __fdiv_rn(v, epi.cm_div[n]) : v;
-                else C[(long)r * N + n] = v;
-            }
+            if (r >= B) break;
+            float v = gemm_act(acc[r] + bv, epi.act, epi.alpha);
+            if (epi.out_scale) v = v * epi.out_scale[n];
+            if (n >= epi.mask_from) v = v > 0.f ? v : 0.f;
+            C[(long)r * N + n] = v;
         }
     }
 }
@@ -426,8 +395,7 @@ __global__ void gemm_naive_kernel(const float* __restrict__ A, const float* __re
     float v = gemm_act(acc + (epi.bias ? epi.bias[n] : 0.f), epi.act, epi.alpha);
     if (epi.out_scale) v = v * epi.out_scale[n];
     if (n >= epi.mask_from) v = v > 0.f ? v : 0.f;
-    if (epi.cm_ld) C[n * epi.cm_ld + m] = epi.cm_div ? __fdiv_rn(v, epi.cm_div[n]) : v;
-    else C[idx] = v;
+    C[idx] = v;
 }
 
 // Work list for C[B][N] on `slots` resident workgroups (a multiple of 8): whole rounds of 128 x 128 tiles,
@@ -485,10 +453,10 @@ static void launch_tiled(const float* A, const float* W, float* C, long B, long 
 }
 
 int fortis_launch_gemm(const float* A, const float* W, const float* bias, float* C, long B, long N, long K,
-                       int act, float alpha, const float* out_scale, long mask_tail, hipStream_t s, const float* cm_div, long cm_ld)
+                       int act, float alpha, const float* out_scale, long mask_tail, hipStream_t s)
 {
     if (B <= 0 || N <= 0 || K <= 0) return -1;
-    GemmEpi epi = { bias, out_scale, act, alpha, mask_tail > 0 ? N - mask_tail : N, cm_div, cm_ld };
+    GemmEpi epi = { bias, out_scale, act, alpha, mask_tail > 0 ? N - mask_tail : N };
     const bool vec_ok = (K % 4 == 0) && K < (1L << 22) && N < (1L << 24) && (((uintptr_t)A | (uintptr_t)W) % 16 == 0);
     if (!vec_ok) {
         hipLaunchKernelGGL(gemm_naive_kernel, dim3((unsigned)cdiv(B * N, 256)), dim3(256), 0, s, A, W, C, B, N, K, epi);

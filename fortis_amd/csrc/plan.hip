@@ -45,8 +45,6 @@ struct Exec {
     ConvEpi epi = { nullptr, nullptr, 0, 0.f, nullptr };
     const float* Wmfma = nullptr;   // weights packed for the MFMA implicit-GEMM kernel, when the shape qualifies
     int pool_dst = -1;              // conv2d: tensor that receives the 2 x 2 max pool folded into this conv
-    bool post_cm = false;           // gemm: writes the boundary's column-major fp32 host layout itself (the post transpose folded in)
-    const float* post_div = nullptr;
     int head_dst = -1;              // conv2d: tensor that receives the thin 1 x 1 convolution folded into this conv (which then stores nothing itself)
     const float *head_w = nullptr, *head_b = nullptr;
     int head_n = 0;
@@ -446,13 +444,6 @@ int fortis_plan_finalize(fortis_plan* p, int in_t, int out_t)
                         ex.dst = ops[i + 1].dst; adv = 2;
                     } else if (ops[i + 1].kind == OP_MASK_RELU) {
                         ex.mask_tail = ops[i + 1].tail; ex.dst = ops[i + 1].dst; adv = 2;
-                    } else if (ops[i + 1].kind == OP_POST && ops[i + 1].flag == 4 && o.B > 16 && getenv("FORTIS_POST_FOLD") != nullptr) {
-                        // the boundary's post transpose of fp32 host arrays: the GEMM stores column-major and divides.
-                        // Only on request (FORTIS_POST_FOLD=1): one launch and 72 MB of traffic less on the 24576 x 368
-                        // output, but a lane's stores are 16-byte pieces 96 KB apart and cost the last layer what
-                        // the transposing kernel costs (1.194 against 1.191 ms per step).
-                        ex.post_cm = true; ex.dst = ops[i + 1].dst; adv = 2;
-                        ex.post_div = ops[i + 1].has_v[0] ? (const float*)upload(p, ops[i + 1].v0.data(), ops[i + 1].v0.size() * 4) : nullptr;
                     }
                 }
                 break;
@@ -613,7 +604,7 @@ void fortis_plan_run(fortis_plan* p)
         int rc = 0;
         switch (e.kind) {
             case EX_CHAIN: fortis_launch_chain(e.chain, src, dst, e.rows, s); break;
-            case EX_GEMM: rc = fortis_launch_gemm(src, e.W, e.bias, dst, e.rows, e.N, e.K, e.act, e.alpha, e.out_scale, e.mask_tail, s, e.post_div, e.post_cm ? e.rows : 0); break;
+            case EX_GEMM: rc = fortis_launch_gemm(src, e.W, e.bias, dst, e.rows, e.N, e.K, e.act, e.alpha, e.out_scale, e.mask_tail, s); break;
             case EX_SCALE: fortis_launch_scale(src, dst, e.vec, e.rows, e.N, e.flag, s); break;
             case EX_MASK: fortis_launch_mask_relu(src, dst, e.rows, e.N, e.mask_tail, s); break;
             case EX_PRE: fortis_launch_boundary_pre(p->tptr[e.src], dst, e.rows, e.N, e.p0, e.p1, e.p2, e.flag, s); break;
@@ -677,7 +668,7 @@ static void plan_run_rows(fortis_plan* p, long i0, long n, hipStream_t s)
                 fortis_launch_chain(e.chain, (const float*)src + i0 * K0, (float*)dst + i0 * NO, n, s, e.rows);
                 break;
             }
-            case EX_GEMM: rc = fortis_launch_gemm((const float*)src + i0 * e.K, e.W, e.bias, (float*)dst + i0 * e.N, n, e.N, e.K, e.act, e.alpha, e.out_scale, e.mask_tail, s, e.post_div, e.post_cm ? n : 0); break;
+            case EX_GEMM: rc = fortis_launch_gemm((const float*)src + i0 * e.K, e.W, e.bias, (float*)dst + i0 * e.N, n, e.N, e.K, e.act, e.alpha, e.out_scale, e.mask_tail, s); break;
             case EX_SCALE: fortis_launch_scale((const float*)src + i0 * e.N, (float*)dst + i0 * e.N, e.vec, n, e.N, e.flag, s); break;
             case EX_MASK: fortis_launch_mask_relu((const float*)src + i0 * e.N, (float*)dst + i0 * e.N, n, e.N, e.mask_tail, s); break;
             case EX_PRE: fortis_launch_boundary_pre(src + i0 * e.N * e.flag, (float*)dst + i0 * e.N, n, e.N, e.p0, e.p1, e.p2, e.flag, s); break;
@@ -1103,8 +1094,7 @@ static int forward_banded(void* in, void* out)
     if (nb < 2 || rows <= 0 || h.n_in % rows || h.n_out % rows || p->in_t == p->out_t) return -1;
     const long win = h.n_in / rows, wout = h.n_out / rows;           // elements per row
     const size_t ein = (size_t)h.in_esz, eout = (size_t)h.out_esz;
-    const bool in_cm = p->exec.front().kind == EX_PRE;
-    const bool out_cm = p->exec.back().kind == EX_POST || (p->exec.back().kind == EX_GEMM && p->exec.back().post_cm);
+    const bool in_cm = p->exec.front().kind == EX_PRE, out_cm = p->exec.back().kind == EX_POST;
     hipStream_t s = fortis_stream_get();
     if (!g_up) { HIP_OK(hipStreamCreateWithFlags(&g_up, hipStreamNonBlocking)); HIP_OK(hipStreamCreateWithFlags(&g_down, hipStreamNonBlocking)); }
     static std::vector<hipEvent_t> ev;
