@@ -522,15 +522,17 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         unsigned w0q, rr;
         st_divmod((unsigned)(tl * s.nchunks), s.mPer, w0q, rr);
         const int slot = wgx - (int)w0q;
-        cm_v4f* pd = (cm_v4f*)s.part + (((long)slot * gridDim.y + fg) * (s.D * s.tiles - s.sk_tile0) + tl) * (NMT * 4 * CM_THREADS) + tid;
+        float* pd = s.part + (((long)slot * gridDim.y + fg) * (s.D * s.tiles - s.sk_tile0) + tl) * (NMT * 16 * CM_THREADS) + tid;
+        // (a register at a time, 256 consecutive bytes per wave, as device-scope stores: written through L2 as they are
+        // issued instead of lingering there dirty; TSRGAN step 1.897 -> 1.873 ms against 16-byte plain stores.  Letting
+        // the workgroup that brings a tile's last sum finish the tile, counted in through a device-scope atomic, instead
+        // of the second kernel measured 2.02 ms: the waits for the stores and the atomic, and the finishing at the
+        // kernel's tail, cost more than the 9 us launch they replace)
 #pragma unroll
         for (int j = 0; j < NMT; j++)
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                cm_v4f v;
-                v[0] = acc[j][4 * q]; v[1] = acc[j][4 * q + 1]; v[2] = acc[j][4 * q + 2]; v[3] = acc[j][4 * q + 3];
-                pd[(j * 4 + q) * CM_THREADS] = v;
-            }
+            for (int r = 0; r < 16; r++)
+                __hip_atomic_store(pd + (j * 16 + r) * CM_THREADS, acc[j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         it += ch1 - ch0;
         continue;
     } else if constexpr (KG == 1) {
@@ -569,68 +571,88 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
     }
 }
 
-// Second kernel of the streamed split: threads as in conv_mfma_kernel (the same registers of the same lanes), a
-// workgroup per tile and group of four accumulator registers (a tile alone would be too few workgroups for a
-// kernel that only moves memory).  A tile's partial sums are added in slot order, i.e. in the order of the input
-// channels.  part[slot][channel group][tile][register quad][thread][4].
-#define CM_RQB 2      // register quads per workgroup of the reduce kernel
+// The streamed split's finish: a tile's partial sums are added in slot order, i.e. in the order of the input
+// channels, then the epilogue.  Threads as in conv_mfma_kernel (the same registers of the same lanes); rq names a group
+// of four accumulator registers.  part[slot][channel group][tile][register][thread]; ntl tiles and nfg channel
+// groups are streamed, a tile's items meet nseg runs.
 template <int MT, int FT>
-__global__ __launch_bounds__(CM_THREADS) void conv_sk_reduce_kernel(float* __restrict__ y, ConvMShape s, ConvEpi e)
+__device__ __forceinline__ void conv_sk_finish_quad(float* __restrict__ y, const ConvMShape& s, const ConvEpi& e, const int tl, const int fg,
+                                                    const int ntl, const int nfg, const int nseg, const int rq, const int tid)
 {
     constexpr int FW = FT / 32, NMT = MT / 32 / (4 / FW), NQ = NMT * 4;
-    const int tl = blockIdx.x, fg = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = tid >> 6;
+    const long slot = (long)ntl * nfg * (NQ * 4 * CM_THREADS);
+    const float* p = s.part + (((long)fg * ntl + tl) * NQ + rq) * (4 * CM_THREADS) + tid;
+    // a thread's loads all leave before the first is needed: the first four slots (a tile always has two) and the
+    // residual values; the sums are then added in slot order
+    auto ld4 = [&](const long off) __attribute__((always_inline)) {
+        cm_v4f v;
+#pragma unroll
+        for (int q = 0; q < 4; q++) v[q] = p[off + q * CM_THREADS];
+        return v;
+    };
+    const cm_v4f a0 = ld4(0), a1 = ld4(nseg > 1 ? slot : 0);
+    const cm_v4f a2 = ld4(nseg > 2 ? 2 * slot : 0), a3 = ld4(nseg > 3 ? 3 * slot : 0);
+    unsigned zq, tileq;
+    st_divmod((unsigned)(tl + s.sk_tile0), s.mT, zq, tileq);
+    const int z = (int)zq, tile = (int)tileq;
+    const int ft = wave % FW, mt0 = (wave / FW) * NMT;
+    const long ospatial = (long)s.D * s.H * s.W;
+    const int m = tile * MT + (mt0 + rq / 4) * 32 + (lane & 31);
+    unsigned yy, xx;
+    st_divmod((unsigned)m, s.mP, yy, xx);
+    const bool inside = m < s.plane && (int)xx < s.W;
+    const long opos = inside ? ((long)z * s.H + yy) * s.W + xx : 0;
+    const int f0 = fg * FT + ft * 32 + 8 * (rq & 3) + 4 * (lane >> 5);             // registers 4 * (rq & 3) ... + 3 of the m-tile
+    float res[4], sc[4], sf[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int fc = f0 + q < s.F ? f0 + q : 0;
+        res[q] = e.res ? e.res[fc * ospatial + opos] : 0.f;
+        sc[q] = e.scale ? e.scale[fc] : 0.f;
+        sf[q] = e.shift ? e.shift[fc] : 0.f;
+    }
+    cm_v4f acc = a0;
+    if (nseg > 1) acc += a1;
+    if (nseg > 2) acc += a2;
+    if (nseg > 3) acc += a3;
+    for (int k = 4; k < nseg; k++) acc += ld4(k * slot);
+    if (!inside) return;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int f = f0 + q;
+        if (f >= s.F) continue;
+        float v = acc[q];
+        if (e.scale) v = v * sc[q];
+        if (e.shift) v = v + sf[q];
+        if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
+        else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
+        if (e.res) v = v + res[q];
+        y[f * ospatial + opos] = v;
+    }
+}
+// Runs of the streamed split that meet tile tl.
+__device__ __forceinline__ int conv_sk_nseg(const ConvMShape& s, const int tl)
+{
     const int first = tl * s.nchunks;
     unsigned w0q, w1q, rr;
     st_divmod((unsigned)first, s.mPer, w0q, rr);
     st_divmod((unsigned)(first + s.nchunks - 1), s.mPer, w1q, rr);
-    const int nseg = (int)(w1q - w0q) + 1;
-    const long slot = (long)gridDim.x * gridDim.y * (NQ * CM_THREADS);
+    return (int)(w1q - w0q) + 1;
+}
+
+// Second kernel of the streamed split, for launches with more tiles than there are counters: a workgroup per tile and
+// group of four accumulator registers (a tile alone would be too few workgroups for a kernel that only moves memory).
+#define CM_RQB 2      // register quads per workgroup of the reduce kernel
+template <int MT, int FT>
+__global__ __launch_bounds__(CM_THREADS) void conv_sk_reduce_kernel(float* __restrict__ y, ConvMShape s, ConvEpi e)
+{
+    const int tl = blockIdx.x, fg = blockIdx.y, tid = threadIdx.x;
+    const int nseg = conv_sk_nseg(s, tl);
     // a workgroup takes CM_RQB register quads of its tile, one after the other in the code and together in flight
-    auto quad = [&](const int rq) __attribute__((always_inline)) {
-        const cm_v4f* p = (const cm_v4f*)s.part + (((long)fg * gridDim.x + tl) * NQ + rq) * CM_THREADS + tid;
-        // a thread's loads all leave before the first is needed: the first four slots (a tile always has two) and the
-        // residual values; the sums are then added in slot order
-        const cm_v4f a0 = p[0], a1 = p[slot];
-        const cm_v4f a2 = p[nseg > 2 ? 2 * slot : 0], a3 = p[nseg > 3 ? 3 * slot : 0];
-        unsigned zq, tileq;
-        st_divmod((unsigned)(tl + s.sk_tile0), s.mT, zq, tileq);
-        const int z = (int)zq, tile = (int)tileq;
-        const int ft = wave % FW, mt0 = (wave / FW) * NMT;
-        const long ospatial = (long)s.D * s.H * s.W;
-        const int m = tile * MT + (mt0 + rq / 4) * 32 + (lane & 31);
-        unsigned yy, xx;
-        st_divmod((unsigned)m, s.mP, yy, xx);
-        const bool inside = m < s.plane && (int)xx < s.W;
-        const long opos = inside ? ((long)z * s.H + yy) * s.W + xx : 0;
-        const int f0 = fg * FT + ft * 32 + 8 * (rq & 3) + 4 * (lane >> 5);             // registers 4 * (rq & 3) ... + 3 of the m-tile
-        float res[4], sc[4], sf[4];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int fc = f0 + q < s.F ? f0 + q : 0;
-            res[q] = e.res ? e.res[fc * ospatial + opos] : 0.f;
-            sc[q] = e.scale ? e.scale[fc] : 0.f;
-            sf[q] = e.shift ? e.shift[fc] : 0.f;
-        }
-        cm_v4f acc = a0 + a1;
-        if (nseg > 2) acc += a2;
-        if (nseg > 3) acc += a3;
-        for (int k = 4; k < nseg; k++) acc += p[k * slot];
-        if (!inside) return;
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int f = f0 + q;
-            if (f >= s.F) continue;
-            float v = acc[q];
-            if (e.scale) v = v * sc[q];
-            if (e.shift) v = v + sf[q];
-            if (e.act == FORTIS_ACT_RELU) v = v > 0.f ? v : 0.f;
-            else if (e.act == FORTIS_ACT_LEAKY) v = v > 0.f ? v : e.alpha * v;
-            if (e.res) v = v + res[q];
-            y[f * ospatial + opos] = v;
-        }
-    };
-#pragma unroll
-    for (int u = 0; u < CM_RQB; u++) quad((int)blockIdx.z * CM_RQB + u);
+    for (int u = 0; u < CM_RQB; u++)
+        conv_sk_finish_quad<MT, FT>(y, s, e, tl, fg, (int)gridDim.x, (int)gridDim.y, nseg, (int)blockIdx.z * CM_RQB + u, tid);
 }
 
 // Sums the partial results of a channel-split launch in split order (deterministic) and applies the

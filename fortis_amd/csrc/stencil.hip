@@ -94,6 +94,11 @@ __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, c
         if (col0 >= d.count) break;
         const unsigned lim = (d.count - col0 < ST_THREADS ? d.count - col0 : ST_THREADS) * n;
         const float* in = Y + ((size_t)blockIdx.y * d.count + col0) * n;
+        // the cell's own reads are issued before Y is staged, so that both are in flight together (0.135 -> 0.129 ms
+        // for the 1028 x 1028 x 15 scatter; staging all four tiles before one barrier instead measured 0.162 ms)
+        int i = 0, j = 0;
+        StCell cell;
+        if (col < d.count) { st_cell(d, col, i, j); st_prepare(d, i, j, kk, cell); }
         if (tile) __syncthreads();                            // the tile before has been read out of LDS
         if (((uintptr_t)in & 15) == 0) {
             const unsigned lim4 = lim / 4;
@@ -104,10 +109,6 @@ __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, c
         }
         __syncthreads();
         if (col >= d.count) continue;
-        int i, j;
-        st_cell(d, col, i, j);
-        StCell cell;
-        st_prepare(d, i, j, kk, cell);
         // outputs are few (one per model output); handled eight at a time
         for (int q0 = 0; q0 < n; q0 += 8) {
             float tv[8];
