@@ -599,6 +599,8 @@ def main():
         line["cpu_baseline"] = r["cpu_baseline"]
     if with_others:
         line["others"] = run_others(L, args)
+    if L.fortis_error_count():
+        raise SystemExit("bench.py: %d HIP call(s) failed during the run (see stderr): no figure reported" % L.fortis_error_count())
     print(json.dumps(line))
 
 

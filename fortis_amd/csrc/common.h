@@ -7,11 +7,17 @@
 #include "../../include/fortis_rt.h"
 #include "../../include/fortis_step.h"
 
+// A failed runtime call is reported and counted and the library goes on, as the runtime it stands in for does
+// (runtime/fortis_rt.c:30-34, 124, 153 print and return); fortis_error_count() lets a caller that wants to stop on
+// the first failure see it.
+extern "C" void fortis_note_error(void);
 #define HIP_OK(call)                                                                              \
     do {                                                                                          \
         hipError_t e_ = (call);                                                                   \
-        if (e_ != hipSuccess)                                                                     \
+        if (e_ != hipSuccess) {                                                                   \
             fprintf(stderr, "fortis: %s failed: %s (%s:%d)\n", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+            fortis_note_error();                                                                  \
+        }                                                                                         \
     } while (0)
 
 // Raw device memory for what the library keeps itself (weights, tables, staging planes): hipMalloc / hipFree

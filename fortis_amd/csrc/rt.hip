@@ -95,6 +95,10 @@ void fortis_pool_set_allocator(fortis_raw_alloc_fn a, fortis_raw_free_fn f)
 // Test hook: how many times the library has asked the device for memory (every hipMalloc of the library goes
 // through one function): a call that must allocate nothing leaves the count unchanged.
 long fortis_dev_alloc_calls(void) { return g_raw_allocs; }
+// Runtime calls that have failed since the library was loaded (each was also printed).
+static long g_errors = 0;
+void fortis_note_error(void) { __atomic_add_fetch(&g_errors, 1, __ATOMIC_RELAXED); }
+long fortis_error_count(void) { return __atomic_load_n(&g_errors, __ATOMIC_RELAXED); }
 // Test hook: number of slots holding a buffer, and how many of them are in use.
 void fortis_pool_stats(int* held, int* used)
 {

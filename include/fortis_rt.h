@@ -46,6 +46,11 @@ void  fortis_pool_stats(int* held, int* used);
  * the first call that needs it): 0, or -1 with a message when the device has no memory.  No reference counterpart. */
 int   fortis_conv_scratch_reserve(long bytes);
 long  fortis_dev_alloc_calls(void);   /* test hook: raw device allocations the library has made since it was loaded */
+/* Runtime (HIP) calls that have failed since the library was loaded.  Like the reference runtime
+ * (runtime/fortis_rt.c:30-34, 124, 153: print and return) the library reports a failed call on stderr and goes on; a
+ * host that would rather stop reads this count after a step.  fortis_note_error adds one (the library's own use). */
+long  fortis_error_count(void);
+void  fortis_note_error(void);
 
 /* ---- GEMM -------------------------------------------------------------------------------- */
 /* C[B][N] = A[B][K] . W[N][K]^T, fp32, beta = 0.                     runtime/fortis_rt.c:45-75

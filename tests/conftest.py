@@ -37,4 +37,9 @@ def gpu(L):
 def _announce(request):
     # names the case before it runs, flushed, so a run that dies on the GPU still says where
     print(f"\n[case] {request.node.nodeid}", flush=True)
+    lib = request.getfixturevalue("L") if request.node.get_closest_marker("gpu") else None
+    before = lib.fortis_error_count() if lib is not None else 0
     yield
+    # the library prints a failed runtime call and goes on: a GPU case during which one failed is a failed case
+    if lib is not None:
+        assert lib.fortis_error_count() == before, "a HIP call failed during this case (see stderr)"
