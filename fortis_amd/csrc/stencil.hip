@@ -125,6 +125,44 @@ __global__ __launch_bounds__(ST_THREADS) void scatter_kernel(ScatterArgs args, c
     }
 }
 
+// All enclosing-loop iterations of a thin table (at most four outputs per cell) in one pass over the cells: a lane keeps
+// its cell and walks the layers, SC_LB of them at a time with all their reads (the cell's slice of Y straight from
+// global memory, its same-cell scalars) in flight before the first result is stored.  The cell list is read once
+// instead of once per layer and no barrier separates the lanes.
+#define SC_LB 5
+template <int N>
+__global__ __launch_bounds__(ST_THREADS) void scatter_layers_kernel(ScatterArgs args, const float* __restrict__ Y, int layers)
+{
+    __shared__ ScatterArgs d;
+    params_to_lds(&d, ST_THREADS);
+    const unsigned col = blockIdx.x * ST_THREADS + threadIdx.x;
+    if (col >= d.count) return;
+    int i, j;
+    st_cell(d, col, i, j);
+    for (int l0 = 0; l0 < layers; l0 += SC_LB) {
+        StCell cell[SC_LB];
+        float tv[SC_LB][8];
+#pragma unroll
+        for (int u = 0; u < SC_LB; u++) {
+            const int l = l0 + u < layers ? l0 + u : layers - 1;
+            const float* in = Y + ((size_t)l * d.count + col) * N;
+#pragma unroll
+            for (int q = 0; q < 8; q++) tv[u][q] = q < N ? __builtin_nontemporal_load(in + q) : 0.f;    // Y is read once
+            st_prepare(d, i, j, l, cell[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < SC_LB; u++) {
+            if (l0 + u >= layers) break;
+            st_chain_apply(d, cell[u], tv[u]);
+#pragma unroll
+            for (int q = 0; q < N; q++) {
+                const StSlotT<float*> sl = d.refs[q];
+                __builtin_nontemporal_store(tv[u][q], st_g(sl.p) + st_off(sl, i, j, l0 + u));
+            }
+        }
+    }
+}
+
 // ---- lowering: straight-line program -> per-cell code + tv chain -----------------------------
 static bool g_lower_quiet = false;     // set while a table is only being tried for the fused kernels
 #define LOWER_ERR(...) do { if (!g_lower_quiet) fprintf(stderr, __VA_ARGS__); } while (0)
@@ -387,6 +425,18 @@ static void launch_scatter(const StencilDev& low, float* const* dA, const float*
 {
     ScatterArgs a;
     st_make_args<float*>(low, low.cells, dA, &a);
+    static const bool by_layers = !(getenv("FORTIS_SCATTER_LAYERS") && atoi(getenv("FORTIS_SCATTER_LAYERS")) == 0);
+    if (by_layers && layers > 1 && kk == 0 && low.nrefs <= 4) {
+        const dim3 grid((unsigned)cdiv(low.count, ST_THREADS)), block(ST_THREADS);
+        switch (low.nrefs) {
+        case 1: hipLaunchKernelGGL(scatter_layers_kernel<1>, grid, block, 0, s, a, dY, layers); break;
+        case 2: hipLaunchKernelGGL(scatter_layers_kernel<2>, grid, block, 0, s, a, dY, layers); break;
+        case 3: hipLaunchKernelGGL(scatter_layers_kernel<3>, grid, block, 0, s, a, dY, layers); break;
+        default: hipLaunchKernelGGL(scatter_layers_kernel<4>, grid, block, 0, s, a, dY, layers); break;
+        }
+        HIP_OK(hipGetLastError());
+        return;
+    }
     hipLaunchKernelGGL(scatter_kernel, dim3((unsigned)cdiv(low.count, ST_THREADS * SC_TILES), (unsigned)layers), dim3(ST_THREADS),
                        (size_t)ST_THREADS * low.nrefs * sizeof(float), s, a, dY, kk);
     HIP_OK(hipGetLastError());

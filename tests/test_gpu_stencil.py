@@ -76,6 +76,49 @@ def test_gather_scatter_other_grids_bit_exact(L, gpu, sx, sy, nz):
         b.free()
 
 
+@pytest.mark.parametrize("n", [1, 2, 4])
+def test_scatter_all_iterations_other_output_counts(L, gpu, n):
+    """The scatter over all enclosing-loop iterations in one launch walks the iterations inside the kernel for tables
+    of at most four outputs per cell: the ZB scatter table cut down to one and two stores and grown to four, seven
+    iterations (one full group of five and a tail), against the oracle and against one launch per iteration."""
+    import copy
+    sx, sy, nz = 70, 37, 7
+    gd, sd, lp, kd = configs.zb_descriptors(sx, sy, nz)
+    sd, lp = copy.deepcopy(sd), copy.deepcopy(lp)
+    sd["n"], lp["out_shape"] = n, [n]
+    if n < 3:
+        sd["stores"] = [dict(s, slot=s["slot"] - (3 - n)) for s in sd["stores"] if s["slot"] >= 3 - n]
+    else:
+        sd["arrays"].append({"name": "tzz", "shape": [sx, sy, nz], "elt": "f32"})
+        sd["stores"].append({"slot": 3, "array": 5, "idx": [["i", 0], ["j", 0], ["v", 0]]})
+    st = S.build_table(sd, lp, kd, "scatter")
+    A = configs.zb_arrays(sx, sy, nz)
+    count = (sx - 4) * (sy - 4)
+    Y = np.random.default_rng(6).standard_normal((count * nz, n)).astype(np.float32)
+    host = [A["norm_h"], A["kappa_h"], np.zeros(sx * sy * nz, np.float32)] + [np.zeros(sx * sy * nz, np.float32) for _ in range(len(sd["arrays"]) - 3)]
+    # the oracle an iteration at a time; the 2-D array (slot 0 of the full table) gets a plane per iteration on the device
+    ref = [a.copy() for a in host]
+    flat2d = [A["norm_h"], A["kappa_h"], np.zeros(sx * sy, np.float32)] + [r for r in ref[3:]]
+    planes = np.zeros((nz, sx * sy), np.float32)
+    for kk in range(nz):
+        O.stencil_scatter(sd, flat2d, Y[kk * count:(kk + 1) * count], count, kk, 3, 3, sx - 4)
+        planes[kk] = flat2d[2]
+    written = sorted({s["array"] for s in sd["stores"]})
+    one, per = [DevBuf(L, a) for a in host], [DevBuf(L, a) for a in host]
+    dY = DevBuf(L, Y)
+    assert L.fortis_stencil_scatter_all_dev(C.byref(st), ptrs(one), dY.ptr) == 0
+    for a in written:
+        want = planes.reshape(-1) if a == 2 else flat2d[a]
+        assert bits_equal(one[a].get(want.shape), want), (n, a)
+    for kk in range(nz):
+        L.fortis_stencil_scatter_dev(C.byref(st), ptrs(per), C.c_void_p(dY.ptr + kk * count * n * 4), kk)
+    for a in written:
+        if a != 2:
+            assert bits_equal(per[a].get(flat2d[a].shape), flat2d[a]), (n, a)
+    for b in one + per + [dY]:
+        b.free()
+
+
 def test_gather_scatter_expressions_on_special_operands(L, gpu):
     """tv / (S0 + 1e-30f) in the gather and ((tv * S0) * S0) * S1 in the scatter with zeros of both signs, denormals, the
     smallest and largest normals, powers of two near the ends of the exponent range, all-ones mantissas, infinities and
