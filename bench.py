@@ -263,7 +263,7 @@ def run_zb_unfused(L, args):
     assert L.fortis_time_parts_ms(1, (CB * 1)(gather_cb), None, max(10, args.steps), alone) == 0
     ga_ms = alone[0] / max(10, args.steps)
     g_bytes = esz * 4 * n3 + 4 * 27 * rows                 # 4 planes read once, X written
-    s_bytes = 4 * 3 * rows + esz * (n3 + nz * sx * sy + 3 * rows)  # Y read, norm + kappa read per layer, 3 outputs written
+    s_bytes = 4 * 3 * rows + esz * (n3 + sx * sy + 3 * rows)       # Y read, norm's planes and the one kappa plane read once, 3 outputs written
     gbs = g_bytes / (g_ms * 1e-3) / 1e9
     kname = "gather_generic_kernel (typed stencil gather, fp64 host arrays)" if args.f64 else "gather_kernel (stencil gather with lifted expressions)"
     roof = dict(bound="hbm", kernel=kname, achieved=round(gbs, 1), peak=PEAK_HBM_GBS,

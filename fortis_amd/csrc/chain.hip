@@ -497,6 +497,8 @@ void chain_wave_kernel(ChainParams params)
             // X is read once and Y written once: both go through non-temporal accesses so that a row stream of
             // gigabytes does not push the neighbouring kernels' grids out of the 256 MB memory-side cache (the
             // stencil gather that follows a 1028 x 1028 x 15 step ran 0.43 ms behind plain accesses, 0.30 ms now).
+            // The price, for rows that are not whole 16-byte vectors: the 4-byte loads of a row come back to lines
+            // that have already left the cache, and the fetch counter reads 1.12 times X (1.00 with plain loads).
             const gfloat* xrow = st_g(P.X) + (size_t)(row < rows ? row : 0) * K0;
 #pragma unroll
             for (int kg = 0; kg < KG0; kg++) {
@@ -611,6 +613,27 @@ void chain_wave_kernel(ChainParams params)
                     }
                 }
             }
+        } else if (NO < 4) {
+            // Thin outputs (one to three per row): the tile's 16 rows are 16 NO consecutive floats of Y, held by the
+            // lanes of the first quarter of the wave (lane = row, NO values each).  They change lanes so that lane t
+            // holds float t of the run and the tile leaves in one store of whole, consecutive bytes; a lane storing its
+            // row's values one by one left 12-byte pieces that reached memory as separate partial writes (2.4 times
+            // the bytes of Y by the write counter).
+            v4f v = a[0];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (out_mul && r < NO) v[r] = __fmul_rn(v[r], out_mul[r]);
+                if (r >= NO - mask_tail) v[r] = v[r] > 0.f ? v[r] : 0.f;
+            }
+            const int src = NO == 3 ? (lane * 171) >> 9 : NO == 2 ? lane >> 1 : lane, rr = lane - src * NO;   // lane / NO
+            float out = 0.f;
+#pragma unroll
+            for (int r = 0; r < 3; r++) {
+                const float pr = __int_as_float(__builtin_amdgcn_ds_bpermute(src << 2, __float_as_int(v[r])));
+                out = rr == r ? pr : out;
+            }
+            if (lane < 16 * NO && in.row0 + (unsigned)src < rows)
+                __builtin_nontemporal_store(out, st_g(P.Y) + (size_t)in.row0 * NO + lane);
         } else {
             gfloat* yrow = st_g(P.Y) + (size_t)row * NO;
 #pragma unroll

@@ -88,6 +88,8 @@ def test_config3_climsim_full_size_row_sample(L, gpu):
     ref = O.mlp_f64(case["Ws"], case["bs"], case["acts"], X[idx], alphas=case["alphas"])
     assert maxrel(Y[idx], ref) < TOL
     assert np.isfinite(Y).all()
+    if widths[-1] < 4:     # every row once (a row stored twice or not at all would pass the sample above)
+        assert maxrel(Y, O.mlp_f64(Ws, bs, ["relu"] * (n - 1) + ["none"], X)) < TOL
     plan.close()
 
 
@@ -235,6 +237,9 @@ def test_gemm_schedule_phases(L, gpu, B, N, K, act):
     (20000, [200, 256, 17]),       # 13 k groups in, 16 n-tiles: the wide register-resident variant, ragged tail tile
     (16400, [61, 128, 128, 148]),  # SAM-shaped widths, input not a multiple of 4 (scalar loads), 148 outputs
     (16385, [64, 64, 8]),          # 16-byte input loads and output stores, one row past a tile
+    (16391, [27, 64, 3]),          # thin outputs leave a tile in one store after a change of lanes; ragged last tile
+    (16397, [20, 32, 2]),
+    (16387, [12, 48, 1]),
 ])
 def test_chain_wave_kernel_plain_shapes(L, gpu, rows, widths):
     """Many rows take the wave-per-16-rows chain kernel; widths up to 256, vector and scalar row access."""
