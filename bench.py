@@ -27,17 +27,17 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # same command (see profiles/), or None where no counter run has been made for the workload.
-MEASURED_TRAFFIC = {"climsim": (123448 + 68398) * 1024, "zb": int((1114.1 * 2 + 885.2) * 1024),
-                    "zb_ref": int((1005.6 * 2 + 885.2) * 1024), "zb_1028x1028x15": int((200333.1 * 2 + 192541.4) * 1024),
-                    "zb_ref_1028x1028x15": int((196300.7 * 2 + 195918.0) * 1024), "toy": None,
-                    "zb_unfused_1028x1028x15": int((242212.5 * 2 + 1658926.8) * 1024),
-                    "zb_unfused_1028x1028x15_f64": int((247386.7 * 2 + 1658898.9) * 1024),
-                    # conv workloads: every conv, split-reduce and thin-head dispatch of a step summed, divided by the
-                    # step's conv operations (18 and 19), like flop_per_launch
-                    "unet": int((1131516.0 * 2 + 544769.0) * 1024 / 7 / 18), "tsrgan": int((3423671.0 * 2 + 5019823.0) * 1024 / 7 / 19)}
+MEASURED_TRAFFIC = {"climsim": int((61617.6 * 2 + 68462.0) * 1024), "zb": int((1059.5 * 2 + 885.2) * 1024),
+                    "zb_ref": int((990.4 * 2 + 885.2) * 1024), "zb_1028x1028x15": int((200382.1 * 2 + 192014.2) * 1024),
+                    "zb_ref_1028x1028x15": int((196559.2 * 2 + 192937.5) * 1024), "toy": int((1638.8 * 2 + 128.0) * 1024),
+                    "zb_unfused_1028x1028x15": int((242206.1 * 2 + 1659097.0) * 1024),
+                    "zb_unfused_1028x1028x15_f64": int((247395.1 * 2 + 1659004.2) * 1024),
+                    # conv workloads: every dispatch of a step summed, divided by the step's conv operations (18 and 19),
+                    # like flop_per_launch
+                    "unet": int((1084761.3 * 2 + 491007.3) * 1024 / 7 / 18), "tsrgan": int((3433363.5 * 2 + 5010087.6) * 1024 / 7 / 19)}
 
 
-TRAFFIC_SOURCE = {"climsim": "profiles/gemm_bias_act_climsim.txt", "zb": "profiles/mlp_chain_stencil_zb.txt",
+TRAFFIC_SOURCE = {"climsim": "profiles/gemm_bias_act_climsim.txt", "zb": "profiles/mlp_chain_stencil_zb.txt", "toy": "profiles/mlp_chain_stencil_zb.txt",
                   "zb_ref": "profiles/mlp_chain_stencil_zb.txt", "zb_1028x1028x15": "profiles/mlp_chain_stencil_zb.txt",
                   "zb_ref_1028x1028x15": "profiles/mlp_chain_stencil_zb.txt",
                   "zb_unfused_1028x1028x15": "profiles/stencil_gather_scatter_zb_1028x1028x15.txt",
