@@ -53,7 +53,7 @@ PROTOTYPES = {
     "fortis_h2d": (None, [vp, vp, l]), "fortis_d2h": (None, [vp, vp, l]), "fortis_d2d": (None, [vp, vp, l]),
     "fortis_gemm_schedule": (i, [C.c_long, C.c_long, C.c_long, C.POINTER(C.c_long)]),
     "fortis_magic_divmod": (None, [C.c_uint, C.c_uint, C.POINTER(C.c_uint), C.POINTER(C.c_uint)]),
-    "fortis_sync": (None, []), "fortis_dev_alloc_calls": (l, []), "fortis_error_count": (l, []), "fortis_note_error": (None, []), "fortis_conv_scratch_reserve": (i, [l]), "fortis_pool_stats": (None, [C.POINTER(i), C.POINTER(i)]),
+    "fortis_sync": (None, []), "fortis_dev_alloc_calls": (l, []), "fortis_error_count": (l, []), "fortis_note_error": (None, []), "fortis_conv_scratch_reserve": (i, [l]), "fortis_pool_stats": (None, [C.POINTER(i), C.POINTER(i)]), "fortis_pool_trim": (i, []),
     "fortis_pool_set_allocator": (None, [vp, vp]), "fortis_device_info": (i, [C.c_char_p, i, C.POINTER(l)]),
     # fortis_step.h: plan
     "fortis_plan_create": (vp, []), "fortis_plan_destroy": (None, [vp]), "fortis_plan_tensor": (i, [vp, l]),

@@ -108,6 +108,16 @@ void fortis_pool_stats(int* held, int* used)
     if (used) *used = u;
 }
 
+// Gives the buffers the pool holds unused back to the device (a host between two phases of different sizes; the
+// benchmark between workloads, so that each starts on fresh memory).  Returns how many were freed.
+int fortis_pool_trim(void)
+{
+    int freed = 0;
+    for (int i = 0; i < FORTIS_POOL; i++)
+        if (g_pool[i].p && !g_pool[i].used) { g_free(g_pool[i].p); g_pool[i].p = nullptr; g_pool[i].n = 0; freed++; }
+    return freed;
+}
+
 void* fortis_alloc(long n)
 {
     int best = -1;

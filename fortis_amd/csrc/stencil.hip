@@ -245,6 +245,7 @@ struct BoundStencil {
     StencilDev low;              // lowered table
     int* dcells = nullptr;       // device copy of the cell list
     void* darr[FORTIS_MAX_ARRAYS] = {};       // planes of the host arrays: device memory (gather) or page-locked host memory (scatter)
+    void* dblock = nullptr;                   // gather: the one device allocation darr[] points into
     bool host_planes = false;
     // scatter under loop distribution: all iterations computed at the first call of a step (see fortis_scatter_v)
     StencilDev low_all;                       // the table with a plane per iteration for every written array
@@ -321,8 +322,10 @@ static int upload_table(const fortis_stencil_t* t, StencilDev* low, int** dcells
 static void release(BoundStencil& b)
 {
     cells_release(b.dcells);
-    for (int a = 0; a < FORTIS_MAX_ARRAYS; a++)
-        if (b.darr[a]) { if (b.host_planes) HIP_OK(hipHostFree(b.darr[a])); else fortis_dev_free(b.darr[a]); }
+    if (b.dblock) fortis_dev_free(b.dblock);                    // the gather's planes: one allocation
+    else
+        for (int a = 0; a < FORTIS_MAX_ARRAYS; a++)
+            if (b.darr[a]) { if (b.host_planes) HIP_OK(hipHostFree(b.darr[a])); else fortis_dev_free(b.darr[a]); }
     for (int a = 0; a < FORTIS_MAX_ARRAYS; a++) if (b.sall[a]) HIP_OK(hipHostFree(b.sall[a]));
     b = BoundStencil();
 }
@@ -480,8 +483,14 @@ void fortis_gather_v(const int* a, const void* const* H)
     const fortis_stencil_t& t = b.host;
     const bool kdist = t.nk > 1;
     if (!b.init) {
-        for (int ai = 0; ai < t.narrays; ai++)   // gather.cu:8-11
-            if (!b.darr[ai] && fortis_dev_malloc(&b.darr[ai], (size_t)t.plane[ai] * t.nk * esz_of(t, ai), "gather planes") != 0) return;
+        // gather.cu:8-11 allocates a buffer per array; here the arrays' planes sit one behind the other in ONE
+        // allocation: a set of planes that fits the memory-side cache stays in it from step to step only if its
+        // lines spread evenly over the cache's sets, which consecutive addresses do.
+        size_t off[FORTIS_MAX_ARRAYS + 1] = {0};
+        for (int ai = 0; ai < t.narrays; ai++)
+            off[ai + 1] = off[ai] + (((size_t)t.plane[ai] * t.nk * esz_of(t, ai) + 255) & ~(size_t)255);
+        if (fortis_dev_malloc(&b.dblock, off[t.narrays], "gather planes") != 0) return;
+        for (int ai = 0; ai < t.narrays; ai++) b.darr[ai] = (char*)b.dblock + off[ai];
         b.init = true;
     }
     const float* dptr[FORTIS_MAX_ARRAYS];

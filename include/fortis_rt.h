@@ -42,6 +42,9 @@ void  fortis_free(void* p);
  * policy be exercised on a machine without a GPU. */
 void  fortis_pool_set_allocator(int (*raw_alloc)(void** p, unsigned long nbytes), void (*raw_free)(void* p));
 void  fortis_pool_stats(int* held, int* used);
+/* Frees every buffer the pool holds unused (fortis_free only marks a buffer as reusable, runtime/fortis_rt.c:36-40) and
+ * returns their number.  No reference counterpart: there the pool only shrinks when an allocation fails. */
+int   fortis_pool_trim(void);
 /* Grows the library's buffer for the partial sums of channel-split convolutions ahead of time (it otherwise grows on
  * the first call that needs it): 0, or -1 with a message when the device has no memory.  No reference counterpart. */
 int   fortis_conv_scratch_reserve(long bytes);

@@ -75,6 +75,18 @@ def test_pool_release_all_and_retry_on_oom(pool):
     assert L.fortis_alloc(900) == c
 
 
+def test_pool_trim_frees_what_is_held_unused(pool):
+    L, dev = pool
+    a, b, c = L.fortis_alloc(100), L.fortis_alloc(300), L.fortis_alloc(200)
+    L.fortis_free(a)
+    L.fortis_free(c)
+    assert L.fortis_pool_trim() == 2 and dev.frees == 2 and stats(L) == (1, 1)      # b is in use and stays
+    assert sorted(dev.live.values()) == [300]
+    assert L.fortis_pool_trim() == 0
+    L.fortis_free(b)
+    assert L.fortis_alloc(250) == b                        # the pool goes on as before
+
+
 def test_pool_unknown_pointer_is_really_freed(pool):
     L, dev = pool
     p = C.c_void_p()
