@@ -194,14 +194,12 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, const flo
     };
     auto multiply = [&](int set) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < TM; i++)
+        for (int c = 0; c < 4; c++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[set][i].x, fw[set][j].x, acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[set][i].y, fw[set][j].y, acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[set][i].z, fw[set][j].z, acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[set][i].w, fw[set][j].w, acc[i][j], 0, 0, 0);
-            }
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[set][i][c], fw[set][j][c], acc[i][j], 0, 0, 0);
     };
 
     const int nslab = (int)((K + GM_BK - 1) / GM_BK);
