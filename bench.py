@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # same command (see profiles/), or None where no counter run has been made for the workload.
-MEASURED_TRAFFIC = {"climsim": int((61617.6 * 2 + 68462.0) * 1024), "zb": int((1059.5 * 2 + 885.2) * 1024),
+MEASURED_TRAFFIC = {"climsim": int((61642.6 * 2 + 68419.7) * 1024), "zb": int((1059.5 * 2 + 885.2) * 1024),
                     "zb_ref": int((990.4 * 2 + 885.2) * 1024), "zb_1028x1028x15": int((200382.1 * 2 + 192014.2) * 1024),
                     "zb_ref_1028x1028x15": int((196559.2 * 2 + 192937.5) * 1024), "toy": int((1638.8 * 2 + 128.0) * 1024),
                     "zb_unfused_1028x1028x15": int((242206.1 * 2 + 1659097.0) * 1024),
