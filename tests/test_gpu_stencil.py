@@ -360,6 +360,15 @@ def test_bench_grid_fused_equals_unfused_and_layer_vs_oracle(L, gpu):
         assert bits_equal(sb[q].get(host[q].shape), fused_out[q])
     # the 2-D Txy_h: the layer-by-layer scatters leave the last layer in it, the fused step keeps one plane per layer
     assert bits_equal(sb[2].get((n2,)), fused_out[2].reshape(nz, n2)[nz - 1])
+    # every layer scattered by ONE launch (the iterations walked inside the kernel): all three written fields as the
+    # fused step leaves them, the 2-D one with a plane per layer
+    sa = [DevBuf(L, a) for a in host]
+    assert L.fortis_stencil_scatter_all_dev(C.byref(st), ptrs(sa), C.c_void_p(dY)) == 0
+    L.fortis_sync()
+    for q in (2, 3, 4):
+        assert bits_equal(sa[q].get(host[q].shape), fused_out[q])
+    for b in sa:
+        b.free()
     # layer kk against the oracle: X rows of that layer, and the scatter of the GPU's own Y for it
     kk = 7
     Xk = np.empty((count, 27), np.float32)
