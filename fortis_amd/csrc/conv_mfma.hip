@@ -30,6 +30,9 @@ typedef float cm_v4f __attribute__((ext_vector_type(4)));   // native vector: co
 // chunk's global loads: with 9 or 27 taps 4 channels do, a single tap takes 16.  (8 channels at 9 taps
 // gain 10% on 32 x 32 images and lose 30% on 256 x 256 ones, whose halo then no longer fits the larger tile.)
 static constexpr int cm_cc(int T) { return T >= 27 ? 2 : T >= 9 ? 4 : 16; }
+#ifndef CM_STORE_NUM
+#define CM_STORE_NUM 6    // eighths of a chunk's products in front of the move of the next chunk into LDS (TSRGAN step, 8: 1.871 ms, 7: 1.873, 6: 1.858, 5: 1.876, 4: 1.872)
+#endif
 #define CM_NXMAX 16   // staging rounds of the input run, at most (the kernel is built for 8 and for 16)
 
 struct ConvMShape {
@@ -281,7 +284,8 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
-    auto multiply = [&](int buf) {
+    // products q0 <= q < q1 of the chunk's NCPW * T (channel pair, tap) products, in order
+    auto multiply_part = [&](int buf, const int q0, const int q1) __attribute__((always_inline)) {
         const float* w = sW + buf * WCHP + wbase;
         const float* xs = sX + buf * XCHP + xbase;
 #pragma unroll
@@ -293,6 +297,7 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
 #pragma unroll
                     for (int kw = 0; kw < KS; kw++) {
                         const int tap = (kd * KS + kh) * KS + kw;
+                        if (cp * T + tap < q0 || cp * T + tap >= q1) continue;
                         const float a = w[(cp * T + tap) * 2 * FT];
                         const int xoff = (2 * cp * KD + kd) * RR + kh * (TILE2D ? CM_TP : s.P) + kw;
 #pragma unroll
@@ -300,6 +305,10 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                             acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, xs[j * (TILE2D ? CM_TP : 32) + xoff], acc[j], 0, 0, 0);
                     }
     };
+    auto multiply = [&](int buf) __attribute__((always_inline)) { multiply_part(buf, 0, NCPW * T); };
+    // the product behind which a step moves the next chunk into LDS (the rest of the chunk's products then run
+    // beside those stores instead of in front of them)
+    constexpr int QS = NCPW * T * CM_STORE_NUM / 8;
     // One step of the pipeline on chunk ch (LDS buffer buf): fetch chunk ch + 2 into `far`, multiply, move
     // chunk ch + 1 from `near` into the other LDS buffer.  The steady-state form is unconditional: the
     // compiler's wait insertion counts loads behind a branch as possibly absent and would then wait for
@@ -356,10 +365,16 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         __builtin_amdgcn_sched_barrier(0);     // nothing of the store below (it waits for `near`) moves above the multiplies
         // the multiply phase outranks the other resident waves' staging at the issue port (UNet 0.266 -> 0.262 ms)
         __builtin_amdgcn_s_setprio(2);
-        multiply(buf);
+        multiply_part(buf, 0, QS);
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
         store_chunk(near, buf ^ 1, ch + 1);
+        if constexpr (QS < NCPW * T) {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(2);
+            multiply_part(buf, QS, NCPW * T);
+            __builtin_amdgcn_s_setprio(0);
+        }
         cm_lds_barrier();
         }
     };
