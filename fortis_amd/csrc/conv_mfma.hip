@@ -33,6 +33,9 @@ static constexpr int cm_cc(int T) { return T >= 27 ? 2 : T >= 9 ? 4 : 16; }
 #ifndef CM_STORE_NUM
 #define CM_STORE_NUM 6    // eighths of a chunk's products in front of the move of the next chunk into LDS (TSRGAN step, 8: 1.871 ms, 7: 1.873, 6: 1.858, 5: 1.876, 4: 1.872)
 #endif
+#ifndef CM_DEFER
+#define CM_DEFER 4         // products of a chunk kept behind the step's barrier (TSRGAN step, 0: 1.850 ms, 2: 1.845, 4: 1.839, 6: 1.849, 8: 1.888)
+#endif
 #define CM_NXMAX 16   // staging rounds of the input run, at most (the kernel is built for 8 and for 16)
 
 struct ConvMShape {
@@ -306,6 +309,31 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
                     }
     };
     auto multiply = [&](int buf) __attribute__((always_inline)) { multiply_part(buf, 0, NCPW * T); };
+    // The chunk's last ND products wait behind the step's barrier with their operands already in registers: they are what
+    // the matrix pipe has to do while the workgroup's waves meet and the next chunk's first operands come out of LDS.
+    // (Not in the form whose 128 registers have none to spare.)
+    constexpr int ND = (XDUMP || SK) && NCPW * T > 2 * CM_DEFER ? CM_DEFER : 0;
+    float dfa[ND > 0 ? ND : 1], dfx[ND > 0 ? ND : 1][NMT];
+    auto preread_last = [&](int buf) __attribute__((always_inline)) {
+        const float* w = sW + buf * WCHP + wbase;
+        const float* xs = sX + buf * XCHP + xbase;
+#pragma unroll
+        for (int d = 0; d < ND; d++) {
+            const int q = NCPW * T - ND + d, cp = q / T, tap = q % T;
+            const int kd = tap / (KS * KS), kh = (tap / KS) % KS, kw = tap % KS;
+            dfa[d] = w[(cp * T + tap) * 2 * FT];
+            const int xoff = (2 * cp * KD + kd) * RR + kh * (TILE2D ? CM_TP : s.P) + kw;
+#pragma unroll
+            for (int j = 0; j < NMT; j++) dfx[d][j] = xs[j * (TILE2D ? CM_TP : 32) + xoff];
+        }
+    };
+    auto multiply_last = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int d = 0; d < ND; d++)
+#pragma unroll
+            for (int j = 0; j < NMT; j++)
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(dfa[d], dfx[d][j], acc[j], 0, 0, 0);
+    };
     // the product behind which a step moves the next chunk into LDS (the rest of the chunk's products then run
     // beside those stores instead of in front of them)
     constexpr int QS = NCPW * T * CM_STORE_NUM / 8;
@@ -372,10 +400,15 @@ void conv_mfma_kernel(const float* __restrict__ x, const float* __restrict__ wp,
         if constexpr (QS < NCPW * T) {
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(2);
-            multiply_part(buf, QS, NCPW * T);
+            multiply_part(buf, QS, NCPW * T - ND);
             __builtin_amdgcn_s_setprio(0);
         }
+        if constexpr (ND > 0) preread_last(buf);
         cm_lds_barrier();
+        if constexpr (ND > 0) {
+            __builtin_amdgcn_sched_barrier(0);
+            multiply_last();
+        }
         }
     };
     auto step_tail = [&](int ch, int buf, Regs& far, const Regs& near) {
