@@ -34,7 +34,7 @@ MEASURED_TRAFFIC = {"climsim": int((61642.6 * 2 + 68419.7) * 1024), "zb": int((1
                     "zb_unfused_1028x1028x15_f64": int((247395.1 * 2 + 1659004.2) * 1024),
                     # conv workloads: every dispatch of a step summed, divided by the step's conv operations (18 and 19),
                     # like flop_per_launch
-                    "unet": int((1084761.3 * 2 + 491007.3) * 1024 / 7 / 18), "tsrgan": int((3433363.5 * 2 + 5010087.6) * 1024 / 7 / 19)}
+                    "unet": int((1084771.1 * 2 + 491007.3) * 1024 / 7 / 18), "tsrgan": int((3426949.4 * 2 + 4994724.7) * 1024 / 7 / 19)}
 
 
 TRAFFIC_SOURCE = {"climsim": "profiles/gemm_bias_act_climsim.txt", "zb": "profiles/mlp_chain_stencil_zb.txt", "toy": "profiles/mlp_chain_stencil_zb.txt",
