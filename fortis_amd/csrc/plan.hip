@@ -886,6 +886,7 @@ static void setup_xy()
 // chunks through the page-locked staging buffers (g_step.X / g_step.Y): worker threads copy chunks between
 // the host array and staging while the DMA engine moves the chunks already copied.
 // FORTIS_NO_STAGED_COPY=1 keeps the plain copies.
+static void copy_streaming(void* dst, const void* src, size_t n);
 #define STAGE_CHUNK ((size_t)4 << 20)
 #define STAGE_THREADS 4
 static bool staged_copies(size_t n)
@@ -899,7 +900,7 @@ static void staged_h2d(void* dev, const void* host, void* stage, size_t n, hipSt
     auto work = [&]() {
         for (size_t c = next.fetch_add(1); c < nchunks; c = next.fetch_add(1)) {
             const size_t o = c * STAGE_CHUNK, len = o + STAGE_CHUNK < n ? STAGE_CHUNK : n - o;
-            memcpy((char*)stage + o, (const char*)host + o, len);
+            copy_streaming((char*)stage + o, (const char*)host + o, len);
             HIP_OK(hipMemcpyAsync((char*)dev + o, (char*)stage + o, len, hipMemcpyHostToDevice, s));
         }
     };
@@ -927,7 +928,7 @@ static void staged_d2h(void* host, const void* dev, void* stage, size_t n, hipSt
         for (size_t c = next.fetch_add(1); c < nchunks; c = next.fetch_add(1)) {
             const size_t o = c * STAGE_CHUNK, len = o + STAGE_CHUNK < n ? STAGE_CHUNK : n - o;
             HIP_OK(hipEventSynchronize(ev[c]));
-            memcpy((char*)host + o, (const char*)stage + o, len);
+            copy_streaming((char*)host + o, (const char*)stage + o, len);
         }
     };
     std::thread th[STAGE_THREADS - 1];
@@ -1030,6 +1031,32 @@ void mlp_forward_batched(void* in, void* out)
 // per feature), which is the layout plan_run_rows gives a boundary transpose.  FORTIS_BANDS=n sets the count
 // (1: the whole array at once, as without this path).
 static hipStream_t g_up = nullptr, g_down = nullptr;
+// memcpy whose stores do not go through the CPU's caches: the bands' copies write megabytes that the CPU does not read
+// again (staging that the DMA engine reads, a host array the caller reads much later), and an ordinary store first
+// reads the line it is about to overwrite, which is a third of the memory traffic of a copy that is bound by it.
+// FORTIS_PLAIN_MEMCPY=1 keeps memcpy.
+typedef float hv4f __attribute__((ext_vector_type(4)));
+static void copy_streaming(void* dst, const void* src, size_t n)
+{
+    static const bool plain = getenv("FORTIS_PLAIN_MEMCPY") != nullptr;
+    char* d = (char*)dst;
+    const char* s = (const char*)src;
+    if (plain || n < 4096) { memcpy(d, s, n); return; }
+    const size_t head = (16 - ((uintptr_t)d & 15)) & 15;
+    memcpy(d, s, head);
+    d += head; s += head; n -= head;
+    const size_t nv = n / 64;
+    for (size_t i = 0; i < nv; i++) {
+        hv4f a, b, c, e;
+        memcpy(&a, s + 64 * i, 16); memcpy(&b, s + 64 * i + 16, 16); memcpy(&c, s + 64 * i + 32, 16); memcpy(&e, s + 64 * i + 48, 16);
+        __builtin_nontemporal_store(a, (hv4f*)(d + 64 * i));
+        __builtin_nontemporal_store(b, (hv4f*)(d + 64 * i + 16));
+        __builtin_nontemporal_store(c, (hv4f*)(d + 64 * i + 32));
+        __builtin_nontemporal_store(e, (hv4f*)(d + 64 * i + 48));
+    }
+    memcpy(d + 64 * nv, s + 64 * nv, n - 64 * nv);
+    __atomic_thread_fence(__ATOMIC_SEQ_CST);      // the streamed stores are visible before the copy is reported done
+}
 // Host copies are what bounds such a call (the bus and the GPU are faster than four threads copy), so the runs of a
 // band are dealt to a pool of threads that lives as long as the process (FORTIS_COPY_THREADS, default 12; starting
 // threads for every band cost about 0.1 ms each time).
@@ -1116,10 +1143,10 @@ static int forward_banded(void* in, void* out)
         const long i0 = edge[b], n = edge[b + 1] - edge[b];
         if (n <= 0) continue;
         char* stage = (char*)g_step.X + (size_t)i0 * win * ein;
-        if (in_cm) parallel_runs(win, [&](long k) { memcpy(stage + (size_t)k * n * ein, (const char*)in + ((size_t)k * rows + i0) * ein, (size_t)n * ein); });
+        if (in_cm) parallel_runs(win, [&](long k) { copy_streaming(stage + (size_t)k * n * ein, (const char*)in + ((size_t)k * rows + i0) * ein, (size_t)n * ein); });
         else {
             const size_t bytes = (size_t)n * win * ein, piece = (bytes / 32 + 4095) & ~(size_t)4095;
-            parallel_runs(32, [&](long k) { const size_t o = (size_t)k * piece; if (o < bytes) memcpy(stage + o, (const char*)in + (size_t)i0 * win * ein + o, o + piece < bytes ? piece : bytes - o); });
+            parallel_runs(32, [&](long k) { const size_t o = (size_t)k * piece; if (o < bytes) copy_streaming(stage + o, (const char*)in + (size_t)i0 * win * ein + o, o + piece < bytes ? piece : bytes - o); });
         }
         HIP_OK(hipMemcpyAsync((char*)g_step.din + (size_t)i0 * win * ein, stage, (size_t)n * win * ein, hipMemcpyHostToDevice, g_up));
         HIP_OK(hipEventRecord(ev[3 * b], g_up));
@@ -1135,10 +1162,10 @@ static int forward_banded(void* in, void* out)
         if (n <= 0) continue;
         const char* stage = (const char*)g_step.Y + (size_t)i0 * wout * eout;
         HIP_OK(hipEventSynchronize(ev[3 * b + 2]));
-        if (out_cm) parallel_runs(wout, [&](long k) { memcpy((char*)out + ((size_t)k * rows + i0) * eout, stage + (size_t)k * n * eout, (size_t)n * eout); });
+        if (out_cm) parallel_runs(wout, [&](long k) { copy_streaming((char*)out + ((size_t)k * rows + i0) * eout, stage + (size_t)k * n * eout, (size_t)n * eout); });
         else {
             const size_t bytes = (size_t)n * wout * eout, piece = (bytes / 32 + 4095) & ~(size_t)4095;
-            parallel_runs(32, [&](long k) { const size_t o = (size_t)k * piece; if (o < bytes) memcpy((char*)out + (size_t)i0 * wout * eout + o, stage + o, o + piece < bytes ? piece : bytes - o); });
+            parallel_runs(32, [&](long k) { const size_t o = (size_t)k * piece; if (o < bytes) copy_streaming((char*)out + (size_t)i0 * wout * eout + o, stage + o, o + piece < bytes ? piece : bytes - o); });
         }
     }
     HIP_OK(hipStreamSynchronize(s));
