@@ -218,7 +218,6 @@ def run_zb_unfused(L, args):
     A = {k: np.ascontiguousarray(v, dtype=ft) for k, v in configs.zb_arrays(sx, sy, nz).items()}
     rows, count, n3 = gt.count * gt.nk, int(gt.count), sx * sy * nz
     net = configs.zb_mlp()
-    plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows)
 
     held = []
 
@@ -230,6 +229,8 @@ def run_zb_unfused(L, args):
     # The gather's four planes live in ONE device allocation, one behind the other: together they just fit the chip's 256 MB
     # memory-side cache and stay in it from step to step only if their lines spread evenly over its sets, which
     # consecutive addresses do and four buffers placed wherever the pool has room do not (0.31 against 0.37 ms per gather).
+    # They are allocated before the plan's gigabytes of X and Y for the same reason (behind them, in a process that had run
+    # other large workloads, the gather read 0.325 ms).
     garr = [A[k] for k in ("sh_xy_h", "sh_xx", "vort_xy_h", "norm_h")]
     goff = np.cumsum([0] + [(a.nbytes + 255) // 256 * 256 for a in garr])
     gblock = L.fortis_alloc(int(goff[-1]))
@@ -238,6 +239,7 @@ def run_zb_unfused(L, args):
         L.fortis_h2d(gblock + int(o), a.ctypes.data, a.nbytes)
     dG = (C.c_void_p * 4)(*[gblock + int(o) for o in goff[:4]])
     dS = (C.c_void_p * 5)(dG[3], dev(A["kappa_h"]), dev(np.zeros(n3, ft)), dev(np.zeros(n3, ft)), dev(np.zeros(n3, ft)))   # Txy_h: a plane per layer
+    plan = P.mlp_plan(net["Ws"], net["bs"], net["acts"], rows)
     dX = L.fortis_plan_tensor_ptr(plan.handle, plan.in_tensor)
     dY = L.fortis_plan_tensor_ptr(plan.handle, plan.out_tensor)
     CB = C.CFUNCTYPE(None, C.c_void_p)
